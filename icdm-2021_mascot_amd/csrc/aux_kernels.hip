@@ -1,0 +1,436 @@
+// Kernels around the update loop: binary16 <-> binary32 conversion, grouped-storage scatter and
+// gather, the g-switching error estimate, test RMSE (dense and grouped), model init, histogram,
+// re-indexing.  All are streaming, HBM-bound, grid-stride kernels.
+#include "mf_host.h"
+#include "mf_device.h"
+
+namespace mf {
+
+constexpr int kStreamBlock = 256;
+static inline uint32_t stream_grid(uint64_t n, int per_thread = 1)
+{
+    uint64_t blocks = (n + (uint64_t)kStreamBlock * per_thread - 1) / ((uint64_t)kStreamBlock * per_thread);
+    const uint64_t cap = 256ull * 32;             // 32 workgroups per CU keeps every XCD busy
+    if (blocks > cap) blocks = cap;
+    if (blocks == 0) blocks = 1;
+    return (uint32_t)blocks;
+}
+
+// ---- conversions (model_init.cu:85-112, precision_switching.h:1-6) -----------------------------
+__global__ __launch_bounds__(kStreamBlock) void float2half_kernel(const float* __restrict__ in, uint16_t* __restrict__ out, uint64_t n)
+{
+    const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+    const uint64_t n2 = n / 2;
+    for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n2; i += stride) {
+        const float2 v = reinterpret_cast<const float2*>(in)[i];
+        half2_t h; h.x = (half_t)v.x; h.y = (half_t)v.y;
+        reinterpret_cast<uint32_t*>(out)[i] = bits(h);
+    }
+    if ((n & 1) && blockIdx.x == 0 && threadIdx.x == 0) out[n - 1] = (uint16_t)bits((half_t)in[n - 1]);
+}
+__global__ __launch_bounds__(kStreamBlock) void half2float_kernel(const uint16_t* __restrict__ in, float* __restrict__ out, uint64_t n)
+{
+    const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+    const uint64_t n2 = n / 2;
+    for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n2; i += stride) {
+        const half2_t h = from_bits<half2_t>(reinterpret_cast<const uint32_t*>(in)[i]);
+        reinterpret_cast<float2*>(out)[i] = make_float2((float)h.x, (float)h.y);
+    }
+    if ((n & 1) && blockIdx.x == 0 && threadIdx.x == 0) out[n - 1] = (float)from_bits<half_t>(in[n - 1]);
+}
+
+// min{g : idx <= end[g]}
+__device__ __forceinline__ uint32_t group_of(const uint32_t* end, uint32_t groups, uint32_t idx)
+{
+    uint32_t lo = 0, hi = groups - 1;
+    while (lo < hi) {
+        uint32_t mid = (lo + hi) >> 1;
+        if (idx <= end[mid]) hi = mid; else lo = mid + 1;
+    }
+    return lo;
+}
+
+// ---- scatter into grouped binary16 storage (model_init.cu:30-83) ---------------------------------
+template <int K>
+__global__ __launch_bounds__(kBlock) void scatter_to_groups_kernel(const float* __restrict__ params, void* const* __restrict__ group_ptr,
+                                                                  const uint32_t* __restrict__ group_end, const uint32_t* __restrict__ entity2group,
+                                                                  const uint32_t* __restrict__ entity2sorted, uint32_t n, uint32_t groups)
+{
+    const int lane = threadIdx.x & 63;
+    const uint32_t waves = gridDim.x * kWavesPerBlock;
+    for (uint32_t e = blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6); e < n; e += waves) {
+        const uint32_t g = entity2group[e];
+        if (g >= groups) continue;
+        const uint32_t first = g ? group_end[g - 1] + 1 : 0;
+        const uint32_t row = entity2sorted[e] - first;
+        uint16_t* dst = reinterpret_cast<uint16_t*>(group_ptr[g]) + (size_t)row * K;
+        const float* src = params + (size_t)e * K;
+        if constexpr (K == 128) {
+            const float2 v = reinterpret_cast<const float2*>(src)[lane];
+            half2_t h; h.x = (half_t)v.x; h.y = (half_t)v.y;
+            reinterpret_cast<uint32_t*>(dst)[lane] = bits(h);
+        } else {
+            dst[lane] = (uint16_t)bits((half_t)src[lane]);
+        }
+    }
+}
+
+// ---- gather grouped storage into a dense fp32 matrix in sorted row order (mf_methods.cu:249-313) --
+template <int K>
+__global__ __launch_bounds__(kBlock) void gather_from_groups_kernel(void* const* __restrict__ group_ptr, const uint32_t* __restrict__ group_end,
+                                                                   const uint8_t* __restrict__ prec, float* __restrict__ dense, uint32_t n, uint32_t groups)
+{
+    const int lane = threadIdx.x & 63;
+    const uint32_t waves = gridDim.x * kWavesPerBlock;
+    for (uint32_t row = blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6); row < n; row += waves) {
+        const uint32_t g = group_of(group_end, groups, row);
+        if (row > group_end[g]) continue;
+        const uint32_t local = g ? row - group_end[g - 1] - 1 : row;
+        float* dst = dense + (size_t)row * K;
+        if (prec[g]) {
+            const float* src = reinterpret_cast<const float*>(group_ptr[g]) + (size_t)local * K;
+            for (int e = lane; e < K; e += 64) dst[e] = src[e];
+        } else {
+            const uint16_t* src = reinterpret_cast<const uint16_t*>(group_ptr[g]) + (size_t)local * K;
+            for (int e = lane; e < K; e += 64) dst[e] = (float)from_bits<half_t>(src[e]);
+        }
+    }
+}
+
+// ---- per-group error (mf_methods.cu:327-379): one wavefront per group ---------------------------
+__global__ __launch_bounds__(kWave) void group_error_kernel(float* __restrict__ grad_sum, const float* __restrict__ norm_sum, uint32_t norm_blocks,
+                                                           const uint8_t* __restrict__ prec, const float* __restrict__ initial,
+                                                           float* __restrict__ error_out, int k, uint32_t groups)
+{
+    const uint32_t g = blockIdx.x;
+    if (g >= groups) return;
+    const int lane = threadIdx.x;
+    if (prec[g]) { if (lane == 0) error_out[g] = -1.f; return; }
+    float acc = 0.f, nacc = 0.f;
+    for (int e = lane; e < k; e += kWave) { const float v = grad_sum[(size_t)g * k + e]; acc += v * v; grad_sum[(size_t)g * k + e] = 0.f; }
+    for (uint32_t b = lane; b < norm_blocks; b += kWave) nacc += norm_sum[(size_t)g * norm_blocks + b];
+    acc = reduce_wave(acc, OpAdd());
+    nacc = reduce_wave(nacc, OpAdd());
+    if (lane == 0) error_out[g] = (acc / nacc) / initial[g];
+}
+
+// ---- test RMSE (rmse.h:26-189): wave reduction of each dot, per-wave double accumulation, LDS
+// reduction across the workgroup, one double atomic per workgroup ----------------------------------
+__device__ __forceinline__ void block_sum_to_global(double acc, double* out)
+{
+    __shared__ double part[kWavesPerBlock];
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    if (lane == 0) part[w] = acc;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        double s = 0;
+        for (int i = 0; i < kWavesPerBlock; ++i) s += part[i];
+        atomicAdd(out, s);
+    }
+}
+
+template <int K>
+__global__ __launch_bounds__(kBlock) void rmse_dense_kernel(const mf_node* __restrict__ test, uint32_t test_n, const float* __restrict__ P,
+                                                           const float* __restrict__ Q, double* sum_sq)
+{
+    constexpr int E = K / 64;
+    const int lane = threadIdx.x & 63;
+    const uint32_t waves = gridDim.x * kWavesPerBlock;
+    const uint32_t wid = blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+    double acc = 0;
+    for (uint64_t base = (uint64_t)wid * kWave; base < test_n; base += (uint64_t)waves * kWave) {
+        const uint64_t left = test_n - base;
+        const int n = left < (uint64_t)kWave ? (int)left : kWave;
+        Rating my = {0.f, 0u, 0u};
+        if (lane < n) my = load_rating(test, (uint32_t)(base + lane));
+        for (int j = 0; j < n; ++j) {
+            const float r = bcast(my.r, j);
+            const float* pp = P + (size_t)bcast(my.u, j) * K + lane;
+            const float* qq = Q + (size_t)bcast(my.v, j) * K + lane;
+            float d = pp[0] * qq[0];
+            if constexpr (E == 2) d = d + pp[64] * qq[64];
+            d = reduce_wave(d, OpAdd());
+            const double err = (double)(r - d);
+            acc += err * err;
+        }
+    }
+    block_sum_to_global(acc, sum_sq);
+}
+
+template <int K>
+__global__ __launch_bounds__(kBlock) void rmse_grouped_kernel(const mf_node* __restrict__ test, uint32_t test_n, void* const* __restrict__ p, void* const* __restrict__ q,
+                                                             const uint32_t* __restrict__ user_end, const uint32_t* __restrict__ item_end,
+                                                             const uint8_t* __restrict__ user_prec, const uint8_t* __restrict__ item_prec,
+                                                             uint32_t user_groups, uint32_t item_groups, double* sum_sq)
+{
+    constexpr int E = K / 64;
+    extern __shared__ __align__(16) uint8_t smem[];
+    uint64_t* pptr_s = reinterpret_cast<uint64_t*>(smem);
+    uint64_t* qptr_s = pptr_s + user_groups;
+    uint32_t* uend_s = reinterpret_cast<uint32_t*>(qptr_s + item_groups);
+    uint32_t* iend_s = uend_s + user_groups;
+    uint8_t* uprec_s = reinterpret_cast<uint8_t*>(iend_s + item_groups);
+    uint8_t* iprec_s = uprec_s + user_groups;
+    for (uint32_t g = threadIdx.x; g < user_groups; g += blockDim.x) { pptr_s[g] = reinterpret_cast<uint64_t>(p[g]); uend_s[g] = user_end[g]; uprec_s[g] = user_prec[g]; }
+    for (uint32_t g = threadIdx.x; g < item_groups; g += blockDim.x) { qptr_s[g] = reinterpret_cast<uint64_t>(q[g]); iend_s[g] = item_end[g]; iprec_s[g] = item_prec[g]; }
+    __syncthreads();
+    const int lane = threadIdx.x & 63;
+    const uint32_t waves = gridDim.x * kWavesPerBlock;
+    const uint32_t wid = blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+    double acc = 0;
+    for (uint64_t base = (uint64_t)wid * kWave; base < test_n; base += (uint64_t)waves * kWave) {
+        const uint64_t left = test_n - base;
+        const int n = left < (uint64_t)kWave ? (int)left : kWave;
+        Rating my = {0.f, 0u, 0u};
+        uint64_t pptr = 0, qptr = 0; uint32_t flags = 4u;
+        if (lane < n) {
+            my = load_rating(test, (uint32_t)(base + lane));
+            const uint32_t ug = group_of(uend_s, user_groups, my.u), ig = group_of(iend_s, item_groups, my.v);
+            const bool ok = my.u <= uend_s[ug] && my.v <= iend_s[ig];
+            const uint32_t urow = ug ? my.u - uend_s[ug - 1] - 1 : my.u;
+            const uint32_t irow = ig ? my.v - iend_s[ig - 1] - 1 : my.v;
+            const uint32_t up = uprec_s[ug] ? 1u : 0u, ip = iprec_s[ig] ? 1u : 0u;
+            pptr = pptr_s[ug] + (uint64_t)urow * (K * (up ? 4u : 2u));
+            qptr = qptr_s[ig] + (uint64_t)irow * (K * (ip ? 4u : 2u));
+            flags = up | (ip << 1) | (ok ? 0u : 4u);
+        }
+        for (int j = 0; j < n; ++j) {
+            const uint32_t f = bcast(flags, j);
+            if (f & 4u) continue;
+            const float r = bcast(my.r, j);
+            const uint64_t pa = bcast(pptr, j), qa = bcast(qptr, j);
+            float pv[E], qv[E];
+#pragma unroll
+            for (int e = 0; e < E; ++e) {
+                const int el = lane + 64 * e;
+                pv[e] = (f & 1u) ? reinterpret_cast<const float*>(pa)[el] : (float)from_bits<half_t>(reinterpret_cast<const uint16_t*>(pa)[el]);
+                qv[e] = (f & 2u) ? reinterpret_cast<const float*>(qa)[el] : (float)from_bits<half_t>(reinterpret_cast<const uint16_t*>(qa)[el]);
+            }
+            float d = pv[0] * qv[0];
+            if constexpr (E == 2) d = d + pv[1] * qv[1];
+            d = reduce_wave(d, OpAdd());
+            const double err = (double)(r - d);
+            acc += err * err;
+        }
+    }
+    block_sum_to_global(acc, sum_sq);
+}
+
+// ---- model init (model_init.cu:19-28): N(0,1)*0.01 from counter-derived bits ----------------------
+// ln x, x in (0,1], from +,-,*,/ only (identical bits on any IEEE machine).
+__device__ __forceinline__ double det_log(double x)
+{
+    const uint64_t b = __builtin_bit_cast(uint64_t, x);
+    int e = (int)((b >> 52) & 0x7ff) - 1022;
+    double m = __builtin_bit_cast(double, (b & 0x000fffffffffffffull) | 0x3fe0000000000000ull);
+    if (m < 0.70710678118654752440) { m = m * 2.0; e = e - 1; }
+    const double s = (m - 1.0) / (m + 1.0);
+    const double s2 = s * s;
+    double acc = 1.0 / 21.0;
+    acc = acc * s2 + 1.0 / 19.0;
+    acc = acc * s2 + 1.0 / 17.0;
+    acc = acc * s2 + 1.0 / 15.0;
+    acc = acc * s2 + 1.0 / 13.0;
+    acc = acc * s2 + 1.0 / 11.0;
+    acc = acc * s2 + 1.0 / 9.0;
+    acc = acc * s2 + 1.0 / 7.0;
+    acc = acc * s2 + 1.0 / 5.0;
+    acc = acc * s2 + 1.0 / 3.0;
+    acc = acc * s2 + 1.0;
+    const double lnm = (2.0 * s) * acc;
+    return (double)e * 0.69314718055994530942 + lnm;
+}
+__device__ __forceinline__ double det_cos2pi(double t)
+{
+    const double t4 = t * 4.0;
+    const int q = (int)t4;
+    const double f = t4 - (double)q;
+    const double a = f * 1.57079632679489661923;
+    const double a2 = a * a;
+    double c = 1.0 / 2432902008176640000.0;
+    c = -1.0 / 6402373705728000.0 + a2 * c;
+    c = 1.0 / 20922789888000.0 + a2 * c;
+    c = -1.0 / 87178291200.0 + a2 * c;
+    c = 1.0 / 479001600.0 + a2 * c;
+    c = -1.0 / 3628800.0 + a2 * c;
+    c = 1.0 / 40320.0 + a2 * c;
+    c = -1.0 / 720.0 + a2 * c;
+    c = 1.0 / 24.0 + a2 * c;
+    c = -1.0 / 2.0 + a2 * c;
+    c = 1.0 + a2 * c;
+    double s = 1.0 / 51090942171709440000.0;
+    s = -1.0 / 121645100408832000.0 + a2 * s;
+    s = 1.0 / 355687428096000.0 + a2 * s;
+    s = -1.0 / 1307674368000.0 + a2 * s;
+    s = 1.0 / 6227020800.0 + a2 * s;
+    s = -1.0 / 39916800.0 + a2 * s;
+    s = 1.0 / 362880.0 + a2 * s;
+    s = -1.0 / 5040.0 + a2 * s;
+    s = 1.0 / 120.0 + a2 * s;
+    s = -1.0 / 6.0 + a2 * s;
+    s = 1.0 + a2 * s;
+    s = a * s;
+    switch (q & 3) { case 0: return c; case 1: return -s; case 2: return -c; default: return s; }
+}
+__global__ __launch_bounds__(kStreamBlock) void init_normal_kernel(float* __restrict__ out, uint64_t n, uint64_t base)
+{
+    const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+    for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+        const uint64_t h = mix64(base ^ i);
+        const uint32_t a = (uint32_t)(h >> 32), b = (uint32_t)h;
+        const double u1 = ((double)a + 1.0) * 2.3283064365386962890625e-10;
+        const double u2 = (double)b * 2.3283064365386962890625e-10;
+        const double rad = __builtin_sqrt(-2.0 * det_log(u1));
+        const double z = rad * det_cos2pi(u2);
+        out[i] = (float)(z * 0.01);
+    }
+}
+
+// ---- preprocessing (preprocess_utils.h:6-36) ---------------------------------------------------
+__global__ __launch_bounds__(kStreamBlock) void iota_kernel(uint32_t* __restrict__ a, uint32_t n)
+{
+    const uint32_t stride = gridDim.x * blockDim.x;
+    for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) a[i] = i;
+}
+__global__ __launch_bounds__(kStreamBlock) void histogram_kernel(const mf_node* __restrict__ R, uint32_t n, uint32_t* user_bin, uint32_t* item_bin)
+{
+    const uint32_t stride = gridDim.x * blockDim.x;
+    for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+        atomicAdd(&user_bin[R[i].u], 1u);
+        atomicAdd(&item_bin[R[i].i], 1u);
+    }
+}
+__global__ __launch_bounds__(kStreamBlock) void reindex_kernel(mf_node* R, const uint32_t* __restrict__ user2sorted, const uint32_t* __restrict__ item2sorted, uint32_t n)
+{
+    const uint32_t stride = gridDim.x * blockDim.x;
+    for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+        const uint32_t u = R[i].u, v = R[i].i;
+        R[i].u = user2sorted[u];
+        R[i].i = item2sorted[v];
+    }
+}
+
+static size_t group_table_lds(uint32_t ug, uint32_t ig) { return (size_t)(ug + ig) * (8 + 4 + 1) + 16; }
+
+}  // namespace mf
+
+using namespace mf;
+
+extern "C" {
+
+int mf_transform_float2half(const float* in, uint16_t* out, uint64_t n, void* stream)
+{
+    if (n == 0) return MF_OK;
+    if (!in || !out) return invalid("mf_transform_float2half: null pointer");
+    if ((reinterpret_cast<uintptr_t>(in) & 7) || (reinterpret_cast<uintptr_t>(out) & 3)) return invalid("mf_transform_float2half: input must be 8-byte and output 4-byte aligned");
+    hipLaunchKernelGGL(float2half_kernel, dim3(stream_grid(n / 2 + 1, 4)), dim3(kStreamBlock), 0, as_stream(stream), in, out, n);
+    return launch_status("mf_transform_float2half");
+}
+int mf_transform_half2float(const uint16_t* in, float* out, uint64_t n, void* stream)
+{
+    if (n == 0) return MF_OK;
+    if (!in || !out) return invalid("mf_transform_half2float: null pointer");
+    if ((reinterpret_cast<uintptr_t>(in) & 3) || (reinterpret_cast<uintptr_t>(out) & 7)) return invalid("mf_transform_half2float: input must be 4-byte and output 8-byte aligned");
+    hipLaunchKernelGGL(half2float_kernel, dim3(stream_grid(n / 2 + 1, 4)), dim3(kStreamBlock), 0, as_stream(stream), in, out, n);
+    return launch_status("mf_transform_half2float");
+}
+
+int mf_cpyparams2grouped_params(const float* original_params, void* const* converted_params,
+                                const uint32_t* group_end_idx, const uint32_t* entity2group,
+                                const uint32_t* entity2sorted_idx, int k, uint32_t n, uint32_t group_num, void* stream)
+{
+    if (k != 64 && k != 128) return invalid("mf_cpyparams2grouped_params: k must be 64 or 128 (got %d)", k);
+    if (n == 0) return MF_OK;
+    if (!original_params || !converted_params || !group_end_idx || !entity2group || !entity2sorted_idx || group_num == 0)
+        return invalid("mf_cpyparams2grouped_params: null pointer or no groups");
+    const uint32_t grid = stream_grid((uint64_t)n * kWave);
+    if (k == 128) hipLaunchKernelGGL(scatter_to_groups_kernel<128>, dim3(grid), dim3(kBlock), 0, as_stream(stream), original_params, converted_params, group_end_idx, entity2group, entity2sorted_idx, n, group_num);
+    else hipLaunchKernelGGL(scatter_to_groups_kernel<64>, dim3(grid), dim3(kBlock), 0, as_stream(stream), original_params, converted_params, group_end_idx, entity2group, entity2sorted_idx, n, group_num);
+    return launch_status("mf_cpyparams2grouped_params");
+}
+
+int mf_grouped_params2dense(void* const* group_ptr, const uint32_t* group_end_idx, const uint8_t* group_prec_info,
+                            float* dense, int k, uint32_t n, uint32_t group_num, void* stream)
+{
+    if (k != 64 && k != 128) return invalid("mf_grouped_params2dense: k must be 64 or 128 (got %d)", k);
+    if (n == 0) return MF_OK;
+    if (!group_ptr || !group_end_idx || !group_prec_info || !dense || group_num == 0) return invalid("mf_grouped_params2dense: null pointer or no groups");
+    const uint32_t grid = stream_grid((uint64_t)n * kWave);
+    if (k == 128) hipLaunchKernelGGL(gather_from_groups_kernel<128>, dim3(grid), dim3(kBlock), 0, as_stream(stream), group_ptr, group_end_idx, group_prec_info, dense, n, group_num);
+    else hipLaunchKernelGGL(gather_from_groups_kernel<64>, dim3(grid), dim3(kBlock), 0, as_stream(stream), group_ptr, group_end_idx, group_prec_info, dense, n, group_num);
+    return launch_status("mf_grouped_params2dense");
+}
+
+int mf_group_error(float* grad_sum_norm, const float* norm_sum, uint32_t norm_blocks, const uint8_t* group_prec_info,
+                   const float* initial_error, float* error_out, int k, uint32_t group_num, void* stream)
+{
+    if (k != 64 && k != 128) return invalid("mf_group_error: k must be 64 or 128 (got %d)", k);
+    if (group_num == 0) return MF_OK;
+    if (!grad_sum_norm || !norm_sum || !group_prec_info || !initial_error || !error_out) return invalid("mf_group_error: null pointer");
+    hipLaunchKernelGGL(group_error_kernel, dim3(group_num), dim3(kWave), 0, as_stream(stream), grad_sum_norm, norm_sum, norm_blocks, group_prec_info, initial_error, error_out, k, group_num);
+    return launch_status("mf_group_error");
+}
+
+int mf_test_rmse(const mf_node* test, uint32_t test_n, const float* p, const float* q, int k, double* sum_sq, void* stream)
+{
+    if (k != 64 && k != 128) return invalid("mf_test_rmse: k must be 64 or 128 (got %d)", k);
+    if (test_n == 0) return MF_OK;
+    if (!test || !p || !q || !sum_sq) return invalid("mf_test_rmse: null pointer");
+    const uint32_t grid = stream_grid((uint64_t)test_n * 4);
+    if (k == 128) hipLaunchKernelGGL(rmse_dense_kernel<128>, dim3(grid), dim3(kBlock), 0, as_stream(stream), test, test_n, p, q, sum_sq);
+    else hipLaunchKernelGGL(rmse_dense_kernel<64>, dim3(grid), dim3(kBlock), 0, as_stream(stream), test, test_n, p, q, sum_sq);
+    return launch_status("mf_test_rmse");
+}
+
+int mf_test_rmse_grouped(const mf_node* test, uint32_t test_n, void* const* p, void* const* q, int k,
+                         const uint32_t* user_group_end_idx, const uint32_t* item_group_end_idx,
+                         const uint8_t* user_group_prec_info, const uint8_t* item_group_prec_info,
+                         uint32_t user_group_num, uint32_t item_group_num, double* sum_sq, void* stream)
+{
+    if (k != 64 && k != 128) return invalid("mf_test_rmse_grouped: k must be 64 or 128 (got %d)", k);
+    if (test_n == 0) return MF_OK;
+    if (!test || !p || !q || !sum_sq || !user_group_end_idx || !item_group_end_idx || !user_group_prec_info || !item_group_prec_info)
+        return invalid("mf_test_rmse_grouped: null pointer");
+    if (user_group_num == 0 || item_group_num == 0) return invalid("mf_test_rmse_grouped: at least one group per side is required");
+    const size_t lds = group_table_lds(user_group_num, item_group_num);
+    if (lds > 60 * 1024) return invalid("mf_test_rmse_grouped: group tables need %zu bytes of LDS", lds);
+    const uint32_t grid = stream_grid((uint64_t)test_n * 4);
+    if (k == 128) hipLaunchKernelGGL(rmse_grouped_kernel<128>, dim3(grid), dim3(kBlock), lds, as_stream(stream), test, test_n, p, q, user_group_end_idx, item_group_end_idx, user_group_prec_info, item_group_prec_info, user_group_num, item_group_num, sum_sq);
+    else hipLaunchKernelGGL(rmse_grouped_kernel<64>, dim3(grid), dim3(kBlock), lds, as_stream(stream), test, test_n, p, q, user_group_end_idx, item_group_end_idx, user_group_prec_info, item_group_prec_info, user_group_num, item_group_num, sum_sq);
+    return launch_status("mf_test_rmse_grouped");
+}
+
+int mf_init_rand_feature(float* array, uint64_t n, uint64_t seed, uint64_t stream_id, void* stream)
+{
+    if (n == 0) return MF_OK;
+    if (!array) return invalid("mf_init_rand_feature: null pointer");
+    const uint64_t base = mix64(mix64(seed ^ 0x494E49544E4F524Dull) + stream_id);
+    hipLaunchKernelGGL(init_normal_kernel, dim3(stream_grid(n)), dim3(kStreamBlock), 0, as_stream(stream), array, n, base);
+    return launch_status("mf_init_rand_feature");
+}
+
+int mf_init_idx_arr(uint32_t* arr, uint32_t n, void* stream)
+{
+    if (n == 0) return MF_OK;
+    if (!arr) return invalid("mf_init_idx_arr: null pointer");
+    hipLaunchKernelGGL(iota_kernel, dim3(stream_grid(n)), dim3(kStreamBlock), 0, as_stream(stream), arr, n);
+    return launch_status("mf_init_idx_arr");
+}
+
+int mf_user_item_histogram(const mf_node* R, uint32_t n, uint32_t* user_bin, uint32_t* item_bin, void* stream)
+{
+    if (n == 0) return MF_OK;
+    if (!R || !user_bin || !item_bin) return invalid("mf_user_item_histogram: null pointer");
+    hipLaunchKernelGGL(histogram_kernel, dim3(stream_grid(n)), dim3(kStreamBlock), 0, as_stream(stream), R, n, user_bin, item_bin);
+    return launch_status("mf_user_item_histogram");
+}
+
+int mf_matrix_reconst_triplet(mf_node* R, const uint32_t* user2sorted_idx, const uint32_t* item2sorted_idx, uint32_t n, void* stream)
+{
+    if (n == 0) return MF_OK;
+    if (!R || !user2sorted_idx || !item2sorted_idx) return invalid("mf_matrix_reconst_triplet: null pointer");
+    hipLaunchKernelGGL(reindex_kernel, dim3(stream_grid(n)), dim3(kStreamBlock), 0, as_stream(stream), R, user2sorted_idx, item2sorted_idx, n);
+    return launch_status("mf_matrix_reconst_triplet");
+}
+
+}  // extern "C"

@@ -1,0 +1,182 @@
+// extern "C" launchers of the five Hogwild update kernels.
+#include "mf_host.h"
+#include "rules_fp32.h"
+#include "rule_mascot.h"
+#include "rules_fixed_point.h"
+#include <cmath>
+#include <cstring>
+
+namespace mf {
+
+static thread_local char g_error[512] = "";
+void set_error(const char* fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_error, sizeof g_error, fmt, ap);
+    va_end(ap);
+}
+
+static int check_schedule(const char* who, const void* R, uint32_t nnz, int k, uint32_t num_workers,
+                          uint32_t update_count, uint32_t update_vector_size)
+{
+    if (k != 64 && k != 128) return invalid("%s: k must be 64 or 128 (got %d)", who, k);
+    if (!R || nnz == 0) return invalid("%s: empty rating array", who);
+    if (num_workers == 0) return invalid("%s: num_workers must be positive", who);
+    if ((uint64_t)update_count * update_vector_size > 0xffffffffull) return invalid("%s: update_count*update_vector_size overflows 32 bits", who);
+    if ((uint64_t)nnz + update_vector_size > 0xffffffffull) return invalid("%s: nnz + update_vector_size overflows 32 bits", who);
+    (void)update_count;
+    return MF_OK;
+}
+static Schedule make_schedule(const mf_node* R, uint32_t nnz, uint32_t num_workers, uint32_t update_count,
+                              uint32_t update_vector_size, uint64_t seed, uint32_t epoch, const uint32_t* window_start)
+{
+    Schedule s;
+    s.R = R; s.nnz = nnz; s.num_workers = num_workers; s.update_count = update_count;
+    s.update_vector_size = update_vector_size; s.epoch_key = window_epoch_key(seed, epoch); s.window_start = window_start;
+    return s;
+}
+static inline uint32_t grid_for(uint32_t num_workers) { return (num_workers + kWavesPerBlock - 1) / kWavesPerBlock; }
+
+template <class Rule>
+static int launch(const char* who, const Schedule& s, const typename Rule::Params& prm, size_t lds, void* stream)
+{
+    if (s.update_count == 0 || s.update_vector_size == 0) return MF_OK;
+    hipLaunchKernelGGL((hogwild_kernel<Rule>), dim3(grid_for(s.num_workers)), dim3(kBlock), lds, as_stream(stream), s, prm);
+    return launch_status(who);
+}
+
+}  // namespace mf
+
+using namespace mf;
+
+extern "C" {
+
+int mf_version(void) { return 1; }
+const char* mf_last_error(void) { return g_error; }
+uint32_t mf_mascot_norm_blocks(uint32_t num_workers) { return grid_for(num_workers); }
+
+uint32_t mf_update_count(uint32_t n, uint32_t num_workers, uint32_t update_vector_size)
+{
+    if (num_workers == 0 || update_vector_size == 0) return 0;
+    return (uint32_t)std::ceil((double)n / (double)((uint64_t)num_workers * update_vector_size));
+}
+uint32_t mf_first_sample_rating_idx(uint32_t e, uint32_t interval, uint32_t epochs, uint32_t update_count,
+                                    uint32_t update_vector_size, float sample_ratio)
+{
+    const uint32_t start_idx = 5;
+    const uint32_t total = update_count * update_vector_size;
+    if (interval == 0) return total;
+    const bool check = (e >= start_idx) && (e % interval == (start_idx % interval)) && (epochs - 1 != e);
+    if (!check) return total;
+    const uint32_t sample_ratings_num = (uint32_t)((float)total * sample_ratio);
+    return total - sample_ratings_num;
+}
+float mf_lr_schedule(float lr, float decay, uint32_t e)
+{
+    return (float)((double)lr / (1.0 + ((double)decay * std::pow((double)e, 1.5))));
+}
+uint32_t mf_window_start(uint64_t seed, uint32_t epoch, uint32_t worker, uint32_t ite, uint32_t nnz)
+{
+    if (nnz == 0) return 0;
+    return window_start_rng(window_epoch_key(seed, epoch), worker, ite, nnz);
+}
+
+int mf_single_sgd_hogwild(const mf_node* R, uint32_t nnz, float* p, float* q, int k,
+                          uint32_t num_workers, uint32_t update_count, uint32_t update_vector_size,
+                          float lrate, float lambda,
+                          uint64_t seed, uint32_t epoch, const uint32_t* window_start, void* stream)
+{
+    if (int rc = check_schedule("mf_single_sgd_hogwild", R, nnz, k, num_workers, update_count, update_vector_size)) return rc;
+    if (!p || !q) return invalid("mf_single_sgd_hogwild: null model pointer");
+    Schedule s = make_schedule(R, nnz, num_workers, update_count, update_vector_size, seed, epoch, window_start);
+    if (k == 128) { SgdRule<128>::Params a{p, q, lrate, lambda}; return launch<SgdRule<128>>("mf_single_sgd_hogwild", s, a, 0, stream); }
+    SgdRule<64>::Params a{p, q, lrate, lambda};
+    return launch<SgdRule<64>>("mf_single_sgd_hogwild", s, a, 0, stream);
+}
+
+int mf_mpt_sgd_hogwild(const mf_node* R, uint32_t nnz, float* p, float* q, int k,
+                       uint32_t num_workers, uint32_t update_count, uint32_t update_vector_size,
+                       float lrate, uint16_t scaled_lambda_half, float scaling_factor,
+                       uint64_t seed, uint32_t epoch, const uint32_t* window_start, void* stream)
+{
+    if (int rc = check_schedule("mf_mpt_sgd_hogwild", R, nnz, k, num_workers, update_count, update_vector_size)) return rc;
+    if (!p || !q) return invalid("mf_mpt_sgd_hogwild: null model pointer");
+    if (!(scaling_factor > 0)) return invalid("mf_mpt_sgd_hogwild: scaling_factor must be positive");
+    Schedule s = make_schedule(R, nnz, num_workers, update_count, update_vector_size, seed, epoch, window_start);
+    if (k == 128) { MptRule<128>::Params a{p, q, lrate, scaled_lambda_half, scaling_factor}; return launch<MptRule<128>>("mf_mpt_sgd_hogwild", s, a, 0, stream); }
+    MptRule<64>::Params a{p, q, lrate, scaled_lambda_half, scaling_factor};
+    return launch<MptRule<64>>("mf_mpt_sgd_hogwild", s, a, 0, stream);
+}
+
+static bool muppet_precision_ok(uint8_t b) { return b == 8 || b == 12 || b == 14 || b == 16 || b == 32; }
+
+int mf_muppet_sgd_hogwild(const mf_node* R, uint32_t nnz, float* p, float* q, int k,
+                          uint32_t num_workers, uint32_t update_count, uint32_t update_vector_size,
+                          float lrate, float lambda, uint32_t first_sample_rating_idx,
+                          float* sum_updated_val, float* sum_norms,
+                          uint8_t forward_prop_precision, uint8_t backward_prop_precision,
+                          uint64_t seed, uint32_t epoch, const uint32_t* window_start, void* stream)
+{
+    if (int rc = check_schedule("mf_muppet_sgd_hogwild", R, nnz, k, num_workers, update_count, update_vector_size)) return rc;
+    if (!p || !q || !sum_updated_val || !sum_norms) return invalid("mf_muppet_sgd_hogwild: null pointer");
+    if (!muppet_precision_ok(forward_prop_precision) || !muppet_precision_ok(backward_prop_precision))
+        return invalid("mf_muppet_sgd_hogwild: precisions must be one of 8, 12, 14, 16, 32");
+    if ((forward_prop_precision == 32) != (backward_prop_precision == 32))
+        return invalid("mf_muppet_sgd_hogwild: forward and backward precision must both be 32 or both below (the backward scale reuses forward statistics)");
+    Schedule s = make_schedule(R, nnz, num_workers, update_count, update_vector_size, seed, epoch, window_start);
+    if (k == 128) {
+        MuppetRule<128>::Params a{p, q, lrate, lambda, first_sample_rating_idx, sum_updated_val, sum_norms, num_workers, forward_prop_precision, backward_prop_precision};
+        return launch<MuppetRule<128>>("mf_muppet_sgd_hogwild", s, a, 0, stream);
+    }
+    MuppetRule<64>::Params a{p, q, lrate, lambda, first_sample_rating_idx, sum_updated_val, sum_norms, num_workers, forward_prop_precision, backward_prop_precision};
+    return launch<MuppetRule<64>>("mf_muppet_sgd_hogwild", s, a, 0, stream);
+}
+
+int mf_afp_sgd_hogwild(const mf_node* R, uint32_t nnz, float* p, float* q, int k,
+                       uint32_t num_workers, uint32_t update_count, uint32_t update_vector_size,
+                       float lrate, float lambda, int afp_epoch,
+                       uint64_t seed, uint32_t epoch, const uint32_t* window_start, void* stream)
+{
+    if (int rc = check_schedule("mf_afp_sgd_hogwild", R, nnz, k, num_workers, update_count, update_vector_size)) return rc;
+    if (!p || !q) return invalid("mf_afp_sgd_hogwild: null model pointer");
+    Schedule s = make_schedule(R, nnz, num_workers, update_count, update_vector_size, seed, epoch, window_start);
+    // afp_sgd_kernel.h:145: int initialization_threshold = (float)(update_count*update_vector_size)/10.0f
+    const int init_threshold = (int)((float)(update_count * update_vector_size) / 10.0f);
+    if (k == 128) { AfpRule<128>::Params a{p, q, lrate, lambda, afp_epoch, init_threshold}; return launch<AfpRule<128>>("mf_afp_sgd_hogwild", s, a, 0, stream); }
+    AfpRule<64>::Params a{p, q, lrate, lambda, afp_epoch, init_threshold};
+    return launch<AfpRule<64>>("mf_afp_sgd_hogwild", s, a, 0, stream);
+}
+
+int mf_mascot_sgd_hogwild(const mf_node* R, uint32_t nnz, void* const* p, void* const* q, int k,
+                          uint32_t num_workers, uint32_t update_count, uint32_t update_vector_size,
+                          float lrate, float lambda,
+                          const uint32_t* user_group_end_idx, const uint32_t* item_group_end_idx,
+                          const uint8_t* user_group_prec_info, const uint8_t* item_group_prec_info,
+                          float* grad_sum_norm_p, float* grad_sum_norm_q, float* norm_sum_p, float* norm_sum_q,
+                          uint32_t first_sample_rating_idx, uint32_t user_group_num, uint32_t item_group_num,
+                          uint64_t seed, uint32_t epoch, const uint32_t* window_start, void* stream)
+{
+    const char* who = "mf_mascot_sgd_hogwild";
+    if (int rc = check_schedule(who, R, nnz, k, num_workers, update_count, update_vector_size)) return rc;
+    if (!p || !q || !user_group_end_idx || !item_group_end_idx || !user_group_prec_info || !item_group_prec_info)
+        return invalid("%s: null group table", who);
+    if (!grad_sum_norm_p || !grad_sum_norm_q || !norm_sum_p || !norm_sum_q) return invalid("%s: null statistics buffer", who);
+    if (user_group_num == 0 || item_group_num == 0) return invalid("%s: at least one group per side is required", who);
+    if (user_group_num > 16383 || item_group_num > 16383) return invalid("%s: at most 16383 groups per side", who);
+    const size_t lds = MascotRule<128>::lds_bytes(user_group_num, item_group_num);
+    if (lds > 64 * 1024) return invalid("%s: group tables need %zu bytes of LDS (limit 65536)", who, lds);
+    Schedule s = make_schedule(R, nnz, num_workers, update_count, update_vector_size, seed, epoch, window_start);
+    if (k == 128) {
+        MascotRule<128>::Params a{p, q, user_group_end_idx, item_group_end_idx, user_group_prec_info, item_group_prec_info,
+                                  grad_sum_norm_p, grad_sum_norm_q, norm_sum_p, norm_sum_q,
+                                  first_sample_rating_idx, user_group_num, item_group_num, lrate, lambda};
+        return launch<MascotRule<128>>(who, s, a, lds, stream);
+    }
+    MascotRule<64>::Params a{p, q, user_group_end_idx, item_group_end_idx, user_group_prec_info, item_group_prec_info,
+                             grad_sum_norm_p, grad_sum_norm_q, norm_sum_p, norm_sum_q,
+                             first_sample_rating_idx, user_group_num, item_group_num, lrate, lambda};
+    return launch<MascotRule<64>>(who, s, a, lds, stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,141 @@
+// Device-side building blocks shared by the gfx950 kernels: wave64 cross-lane
+// reductions (DPP row rotates + v_permlane{16,32}_swap), binary16 vector types,
+// the counter-based window generator and the rating-chunk loader.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include "../../include/mascot_hip.h"
+
+namespace mf {
+
+typedef _Float16 half_t;
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+
+constexpr int kWave = 64;
+constexpr int kBlock = 256;              // 4 wavefronts per workgroup
+constexpr int kWavesPerBlock = kBlock / kWave;
+
+// ---- bit casts -----------------------------------------------------------------------
+__device__ __forceinline__ uint32_t bits(float x) { return __builtin_bit_cast(uint32_t, x); }
+__device__ __forceinline__ uint32_t bits(int x) { return (uint32_t)x; }
+__device__ __forceinline__ uint32_t bits(uint32_t x) { return x; }
+__device__ __forceinline__ uint32_t bits(half2_t x) { return __builtin_bit_cast(uint32_t, x); }
+__device__ __forceinline__ uint32_t bits(half_t x) { return (uint32_t)__builtin_bit_cast(uint16_t, x); }
+template <class T> __device__ __forceinline__ T from_bits(uint32_t b);
+template <> __device__ __forceinline__ float from_bits<float>(uint32_t b) { return __builtin_bit_cast(float, b); }
+template <> __device__ __forceinline__ int from_bits<int>(uint32_t b) { return (int)b; }
+template <> __device__ __forceinline__ uint32_t from_bits<uint32_t>(uint32_t b) { return b; }
+template <> __device__ __forceinline__ half2_t from_bits<half2_t>(uint32_t b) { return __builtin_bit_cast(half2_t, b); }
+template <> __device__ __forceinline__ half_t from_bits<half_t>(uint32_t b) { return __builtin_bit_cast(half_t, (uint16_t)b); }
+
+// ---- cross-lane moves ------------------------------------------------------------------
+// Value held by lane (L ^ 32).
+template <class T> __device__ __forceinline__ T lane_xor32(T x)
+{
+    auto r = __builtin_amdgcn_permlane32_swap(bits(x), bits(x), false, false);
+    // r[0] = lanes 0-31 of x replicated in both halves, r[1] = lanes 32-63 replicated.
+    return from_bits<T>((threadIdx.x & 32) ? r[0] : r[1]);
+}
+// Value held by lane ((L + N) mod 16) of the same row of 16 lanes.
+template <int N, class T> __device__ __forceinline__ T row_ror(T x)
+{
+    return from_bits<T>((uint32_t)__builtin_amdgcn_update_dpp(0, (int)bits(x), 0x120 + N, 0xf, 0xf, false));
+}
+
+// Reduction steps: every lane ends with op(own, partner); op must be commutative.
+struct OpAdd { template <class T> __device__ __forceinline__ T operator()(T a, T b) const { return a + b; } };
+struct OpMin { __device__ __forceinline__ float operator()(float a, float b) const { return fminf(a, b); } };
+struct OpMax { __device__ __forceinline__ float operator()(float a, float b) const { return fmaxf(a, b); } };
+
+template <class T, class Op> __device__ __forceinline__ T step_xor32(T x, Op op)
+{
+    auto r = __builtin_amdgcn_permlane32_swap(bits(x), bits(x), false, false);
+    return op(from_bits<T>(r[0]), from_bits<T>(r[1]));
+}
+template <class T, class Op> __device__ __forceinline__ T step_xor16(T x, Op op)
+{
+    auto r = __builtin_amdgcn_permlane16_swap(bits(x), bits(x), false, false);
+    return op(from_bits<T>(r[0]), from_bits<T>(r[1]));
+}
+template <int N, class T, class Op> __device__ __forceinline__ T step_ror(T x, Op op) { return op(x, row_ror<N>(x)); }
+
+// Tail shared by all layouts: the reference's shfl_down 8,4,2,1 steps inside a row of 16.
+template <class T, class Op> __device__ __forceinline__ T reduce_row16(T x, Op op)
+{
+    x = step_ror<8>(x, op);
+    x = step_ror<4>(x, op);
+    x = step_ror<2>(x, op);
+    x = step_ror<1>(x, op);
+    return x;
+}
+// All 64 lanes, order 32,16,8,4,2,1.  With one element per lane (element L) this is exactly the
+// reference's (m[l] + m[l+32]) followed by its 16,8,4,2,1 tree (sgd/sgd_kernel_k64.h:49-57).
+template <class T, class Op> __device__ __forceinline__ T reduce_wave(T x, Op op)
+{
+    x = step_xor32(x, op);
+    x = step_xor16(x, op);
+    return reduce_row16(x, op);
+}
+// The reference's tree over 32 lanes when lanes L and L^32 already hold the same value.
+template <class T, class Op> __device__ __forceinline__ T reduce_half_wave(T x, Op op)
+{
+    x = step_xor16(x, op);
+    return reduce_row16(x, op);
+}
+
+__device__ __forceinline__ uint32_t bcast(uint32_t v, int lane) { return (uint32_t)__builtin_amdgcn_readlane((int)v, lane); }
+__device__ __forceinline__ float bcast(float v, int lane) { return from_bits<float>(bcast(bits(v), lane)); }
+__device__ __forceinline__ uint64_t bcast(uint64_t v, int lane)
+{
+    return (uint64_t)bcast((uint32_t)v, lane) | ((uint64_t)bcast((uint32_t)(v >> 32), lane) << 32);
+}
+
+// ---- counter-based generator -----------------------------------------------------------
+__host__ __device__ __forceinline__ uint64_t mix64(uint64_t z)
+{
+    z += 0x9E3779B97F4A7C15ull;
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    return z ^ (z >> 31);
+}
+// start of window `ite` of worker `wid`: the mapping of sgd/sgd_kernel.h:22-26 applied to 32
+// counter-derived bits (u01 = x*2^-32 + 2^-33 in (0,1], origin = (unsigned)(u01*nnz), start = origin % nnz).
+__host__ __device__ __forceinline__ uint32_t window_start_rng(uint64_t epoch_key, uint32_t wid, uint32_t ite, uint32_t nnz)
+{
+    uint64_t h = mix64(epoch_key ^ (((uint64_t)wid << 32) | (uint64_t)ite));
+    uint32_t x = (uint32_t)(h >> 32);
+    float t = (float)x * 2.3283064365386963e-10f;
+    float u01 = t + 1.1641532182693481e-10f;
+    float scaled = u01 * (float)nnz;
+    uint32_t origin = (scaled >= 4294967296.0f) ? 0xffffffffu : (uint32_t)scaled;
+    return origin % nnz;
+}
+__host__ __device__ __forceinline__ uint64_t window_epoch_key(uint64_t seed, uint32_t epoch)
+{
+    return mix64(mix64(seed ^ 0x57494E444F575321ull) + (uint64_t)epoch);
+}
+
+// ---- the Hogwild schedule shared by every update kernel ---------------------------------
+struct Schedule {
+    const mf_node* R;
+    uint32_t nnz;
+    uint32_t num_workers;
+    uint32_t update_count;
+    uint32_t update_vector_size;
+    uint64_t epoch_key;
+    const uint32_t* window_start;   // optional [update_count][num_workers]
+};
+
+// One lane's rating of a 64-rating chunk; the stream is read once per epoch, so bypass-style loads.
+struct Rating { float r; uint32_t u; uint32_t v; };
+__device__ __forceinline__ Rating load_rating(const mf_node* R, uint32_t idx)
+{
+    const uint32_t* w = reinterpret_cast<const uint32_t*>(R + idx);
+    Rating x;
+    x.r = from_bits<float>(__builtin_nontemporal_load(w));
+    x.u = __builtin_nontemporal_load(w + 1);
+    x.v = __builtin_nontemporal_load(w + 2);
+    return x;
+}
+
+}  // namespace mf

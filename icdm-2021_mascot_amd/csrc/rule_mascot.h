@@ -1,0 +1,274 @@
+// MASCOT update rule: P/Q stored per popularity group as binary16 or binary32 rows
+// (mascot/mascot_sgd_kernel.h:1-457 and _k64.h of the reference), four precision cases per rating,
+// sampled gradient statistics for the g-switching estimator.
+//
+// Register layout: lane L holds elements 2L, 2L+1 of a row (k = 128; one packed dword for a binary16
+// row, one 8-byte load for a binary32 row) or element L (k = 64).  For k = 128 the reference's
+// order -- warp lane l sums elements l, l+32, l+64, l+96 as ((a+b)+(c+d)), then a 16,8,4,2,1 tree --
+// maps onto packed lanes as: step over lanes L^16 (elements +32), lanes L^32 (+64), then rotates by
+// 8,4,2,1 inside a row of 16 lanes (warp lanes +16,+8,+4,+2) and finally low half + high half
+// (warp lanes +1).  Every add is a packed v_pk_add_f16, each half rounded separately, so the
+// binary16 dot is bit-identical to the reference's sequence of roundings.
+//
+// The group search of the reference (two 32-wide register compares plus a shared-memory fallback per
+// rating, mascot_sgd_kernel.h:104-180) is replaced by one binary search per lane over the end-index
+// table in LDS, done once for the 64 ratings of a chunk; the result is the row address, which is
+// what the per-rating loop broadcasts.
+#pragma once
+#include "hogwild.h"
+
+namespace mf {
+
+template <int K> struct MascotRule {
+    static constexpr int E = K / 64;                        // elements per lane
+    using HV = typename std::conditional<E == 2, half2_t, half_t>::type;
+
+    struct Params {
+        void* const* p; void* const* q;
+        const uint32_t* user_end; const uint32_t* item_end;
+        const uint8_t* user_prec; const uint8_t* item_prec;
+        float* grad_sum_p; float* grad_sum_q; float* norm_sum_p; float* norm_sum_q;
+        uint32_t first_sample; uint32_t user_groups; uint32_t item_groups;
+        float lrate; float lambda;
+    };
+    // raw row registers: binary16 rows use r[0] only
+    struct Row { uint32_t p[E], q[E]; };
+    struct Prep { uint64_t pptr, qptr; uint32_t flags; };
+    struct Info { float r; uint64_t pptr, qptr; uint32_t flags; };
+    // flags: bit0 user row is fp32, bit1 item row is fp32, bit2 rating is skipped (index outside the
+    // group table), bits 3..16 user group, bits 17..30 item group
+    static constexpr uint32_t kSkip = 4u;
+
+    uint64_t* pptr_s; uint64_t* qptr_s;
+    float* unorm_s; float* inorm_s;
+    uint32_t* uend_s; uint32_t* iend_s;
+    uint8_t* uprec_s; uint8_t* iprec_s;
+    float* grad_sum_p; float* grad_sum_q;
+    uint32_t first_sample, user_groups, item_groups;
+    float lrate, lambda;
+    int lane;
+
+    static size_t lds_bytes(uint32_t ug, uint32_t ig) { return (size_t)(ug + ig) * (8 + 4 + 4 + 1) + 16; }
+
+    __device__ __forceinline__ void init(const Params& a, uint8_t* smem, int lane_, uint32_t)
+    {
+        lane = lane_;
+        user_groups = a.user_groups; item_groups = a.item_groups;
+        pptr_s = reinterpret_cast<uint64_t*>(smem);
+        qptr_s = pptr_s + user_groups;
+        unorm_s = reinterpret_cast<float*>(qptr_s + item_groups);
+        inorm_s = unorm_s + user_groups;
+        uend_s = reinterpret_cast<uint32_t*>(inorm_s + item_groups);
+        iend_s = uend_s + user_groups;
+        uprec_s = reinterpret_cast<uint8_t*>(iend_s + item_groups);
+        iprec_s = uprec_s + user_groups;
+        for (uint32_t g = threadIdx.x; g < user_groups; g += blockDim.x) {
+            pptr_s[g] = reinterpret_cast<uint64_t>(a.p[g]); uend_s[g] = a.user_end[g];
+            uprec_s[g] = a.user_prec[g]; unorm_s[g] = 0.f;
+        }
+        for (uint32_t g = threadIdx.x; g < item_groups; g += blockDim.x) {
+            qptr_s[g] = reinterpret_cast<uint64_t>(a.q[g]); iend_s[g] = a.item_end[g];
+            iprec_s[g] = a.item_prec[g]; inorm_s[g] = 0.f;
+        }
+        grad_sum_p = a.grad_sum_p; grad_sum_q = a.grad_sum_q;
+        first_sample = a.first_sample; lrate = a.lrate; lambda = a.lambda;
+        __syncthreads();
+    }
+
+    // min{g : idx <= end[g]}; rows of a group are idx - end[g-1] - 1 (mascot_sgd_kernel.h:104-143).
+    static __device__ __forceinline__ uint32_t search(const uint32_t* end, uint32_t groups, uint32_t idx)
+    {
+        uint32_t lo = 0, hi = groups - 1;
+        while (lo < hi) {
+            uint32_t mid = (lo + hi) >> 1;
+            if (idx <= end[mid]) hi = mid; else lo = mid + 1;
+        }
+        return lo;
+    }
+    __device__ __forceinline__ Prep prepare(const Rating& my, bool valid) const
+    {
+        Prep pr; pr.pptr = 0; pr.qptr = 0; pr.flags = kSkip;
+        if (valid) {
+            const uint32_t ug = search(uend_s, user_groups, my.u);
+            const uint32_t ig = search(iend_s, item_groups, my.v);
+            const bool ok = my.u <= uend_s[ug] && my.v <= iend_s[ig];
+            const uint32_t urow = ug ? my.u - uend_s[ug - 1] - 1 : my.u;
+            const uint32_t irow = ig ? my.v - iend_s[ig - 1] - 1 : my.v;
+            const uint32_t up = uprec_s[ug] ? 1u : 0u, ip = iprec_s[ig] ? 1u : 0u;
+            pr.pptr = pptr_s[ug] + (uint64_t)urow * (K * (up ? 4u : 2u));
+            pr.qptr = qptr_s[ig] + (uint64_t)irow * (K * (ip ? 4u : 2u));
+            pr.flags = up | (ip << 1) | (ok ? 0u : kSkip) | (ug << 3) | (ig << 17);
+        }
+        return pr;
+    }
+    __device__ __forceinline__ Info info(const Rating& my, const Prep& pr, int j) const
+    {
+        Info i;
+        i.r = bcast(my.r, j);
+        i.pptr = bcast(pr.pptr, j);
+        i.qptr = bcast(pr.qptr, j);
+        i.flags = bcast(pr.flags, j);
+        return i;
+    }
+
+    static __device__ __forceinline__ void load_side(uint32_t* r, uint64_t ptr, bool fp32, int lane)
+    {
+        if (fp32) {
+            if constexpr (E == 2) {
+                const uint2 v = *reinterpret_cast<const uint2*>(ptr + (uint64_t)lane * 8);
+                r[0] = v.x; r[1] = v.y;
+            } else {
+                r[0] = *reinterpret_cast<const uint32_t*>(ptr + (uint64_t)lane * 4);
+            }
+        } else {
+            if constexpr (E == 2) r[0] = *reinterpret_cast<const uint32_t*>(ptr + (uint64_t)lane * 4);
+            else r[0] = *reinterpret_cast<const uint16_t*>(ptr + (uint64_t)lane * 2);
+        }
+    }
+    static __device__ __forceinline__ void store_side(const uint32_t* r, uint64_t ptr, bool fp32, int lane)
+    {
+        if (fp32) {
+            if constexpr (E == 2) *reinterpret_cast<uint2*>(ptr + (uint64_t)lane * 8) = make_uint2(r[0], r[1]);
+            else *reinterpret_cast<uint32_t*>(ptr + (uint64_t)lane * 4) = r[0];
+        } else {
+            if constexpr (E == 2) *reinterpret_cast<uint32_t*>(ptr + (uint64_t)lane * 4) = r[0];
+            else *reinterpret_cast<uint16_t*>(ptr + (uint64_t)lane * 2) = (uint16_t)r[0];
+        }
+    }
+    __device__ __forceinline__ void load(Row& row, const Info& i) const
+    {
+#pragma unroll
+        for (int e = 0; e < E; ++e) { row.p[e] = 0; row.q[e] = 0; }
+        if (i.flags & kSkip) return;
+        load_side(row.p, i.pptr, i.flags & 1u, lane);
+        load_side(row.q, i.qptr, i.flags & 2u, lane);
+    }
+    __device__ __forceinline__ void forward(Row& nxt, const Info& in, const Row& cur, const Info& ic) const
+    {
+        if ((in.flags | ic.flags) & kSkip) return;
+        if (in.pptr == ic.pptr) {
+#pragma unroll
+            for (int e = 0; e < E; ++e) nxt.p[e] = cur.p[e];
+        }
+        if (in.qptr == ic.qptr) {
+#pragma unroll
+            for (int e = 0; e < E; ++e) nxt.q[e] = cur.q[e];
+        }
+    }
+
+    // ---- reductions in the reference order ------------------------------------------------
+    static __device__ __forceinline__ half_t dot_half(HV m)
+    {
+        if constexpr (E == 2) {
+            m = step_xor16(m, OpAdd());
+            m = step_xor32(m, OpAdd());
+            m = reduce_row16(m, OpAdd());
+            return m.x + m.y;
+        } else {
+            return reduce_wave(m, OpAdd());
+        }
+    }
+    static __device__ __forceinline__ float dot_float(const float* m)
+    {
+        if constexpr (E == 2) {
+            float a = m[0], b = m[1];
+            a = step_xor16(a, OpAdd()); b = step_xor16(b, OpAdd());
+            a = step_xor32(a, OpAdd()); b = step_xor32(b, OpAdd());
+            a = reduce_row16(a, OpAdd()); b = reduce_row16(b, OpAdd());
+            return a + b;
+        } else {
+            return reduce_wave(m[0], OpAdd());
+        }
+    }
+    static __device__ __forceinline__ float widen(HV h, int e)
+    {
+        if constexpr (E == 2) return (float)(e ? h.y : h.x); else return (float)h;
+    }
+    static __device__ __forceinline__ HV narrow(const float* f)
+    {
+        if constexpr (E == 2) { HV h; h.x = (half_t)f[0]; h.y = (half_t)f[1]; return h; } else return (half_t)f[0];
+    }
+    static __device__ __forceinline__ HV splat(half_t v)
+    {
+        if constexpr (E == 2) { HV h; h.x = v; h.y = v; return h; } else return v;
+    }
+    // sampled statistics of one binary16 side: ||g||^2 into the block's LDS slot, g into the global sums
+    __device__ __forceinline__ void sample(const float* g, uint32_t group, float* norm_s, float* grad_sum) const
+    {
+        float n = g[0] * g[0];
+        if constexpr (E == 2) n = n + g[1] * g[1];
+        n = reduce_wave(n, OpAdd());
+        if (lane == 0) atomicAdd(&norm_s[group], n);
+        float* dst = grad_sum + (size_t)group * K + (size_t)lane * E;
+#pragma unroll
+        for (int e = 0; e < E; ++e) atomicAdd(dst + e, g[e]);
+    }
+
+    __device__ __forceinline__ void update(Row& row, const Info& i, uint32_t processed) const
+    {
+        if (i.flags & kSkip) return;
+        const bool up = i.flags & 1u, ip = i.flags & 2u;
+        const bool sampled = processed >= first_sample;
+        const uint32_t ug = (i.flags >> 3) & 0x3fffu, ig = (i.flags >> 17) & 0x3fffu;
+        if (!up && !ip) {
+            // mascot_sgd_kernel.h:188-278: everything in binary16, one rounding per operation
+            const HV lr_h = splat((half_t)lrate), lam_h = splat((half_t)lambda);
+            const half_t r_h = (half_t)i.r;
+            const HV P = from_bits<HV>(row.p[0]), Q = from_bits<HV>(row.q[0]);
+            const half_t dot = dot_half(P * Q);
+            const HV ruv = splat(r_h - dot);
+            const HV gp = ruv * Q - lam_h * P;
+            const HV gq = ruv * P - lam_h * Q;
+            row.p[0] = bits(HV(__builtin_elementwise_fma(lr_h, gp, P)));
+            row.q[0] = bits(HV(__builtin_elementwise_fma(lr_h, gq, Q)));
+            store_side(row.p, i.pptr, false, lane);
+            store_side(row.q, i.qptr, false, lane);
+            if (sampled) {
+                float g[E];
+#pragma unroll
+                for (int e = 0; e < E; ++e) g[e] = widen(gp, e);
+                sample(g, ug, unorm_s, grad_sum_p);
+#pragma unroll
+                for (int e = 0; e < E; ++e) g[e] = widen(gq, e);
+                sample(g, ig, inorm_s, grad_sum_q);
+            }
+        } else {
+            float pf[E], qf[E], m[E];
+            if (up) { for (int e = 0; e < E; ++e) pf[e] = from_bits<float>(row.p[e]); }
+            else { const HV P = from_bits<HV>(row.p[0]); for (int e = 0; e < E; ++e) pf[e] = widen(P, e); }
+            if (ip) { for (int e = 0; e < E; ++e) qf[e] = from_bits<float>(row.q[e]); }
+            else { const HV Q = from_bits<HV>(row.q[0]); for (int e = 0; e < E; ++e) qf[e] = widen(Q, e); }
+#pragma unroll
+            for (int e = 0; e < E; ++e) m[e] = pf[e] * qf[e];
+            const float ruv = i.r - dot_float(m);
+            float gp[E], gq[E], np_[E], nq_[E];
+#pragma unroll
+            for (int e = 0; e < E; ++e) {
+                gp[e] = ruv * qf[e] - lambda * pf[e];
+                gq[e] = ruv * pf[e] - lambda * qf[e];
+                np_[e] = __builtin_fmaf(lrate, gp[e], pf[e]);
+                nq_[e] = __builtin_fmaf(lrate, gq[e], qf[e]);
+            }
+            if (up) { for (int e = 0; e < E; ++e) row.p[e] = bits(np_[e]); }
+            else row.p[0] = bits(narrow(np_));
+            if (ip) { for (int e = 0; e < E; ++e) row.q[e] = bits(nq_[e]); }
+            else row.q[0] = bits(narrow(nq_));
+            store_side(row.p, i.pptr, up, lane);
+            store_side(row.q, i.qptr, ip, lane);
+            if (sampled) {
+                if (!up) sample(gp, ug, unorm_s, grad_sum_p);
+                if (!ip) sample(gq, ig, inorm_s, grad_sum_q);
+            }
+        }
+    }
+
+    // mascot_sgd_kernel.h:448-456: per-block norm sums, layout [group][block]
+    __device__ __forceinline__ void finish(const Params& a, uint32_t) const
+    {
+        __syncthreads();
+        for (uint32_t g = threadIdx.x; g < user_groups; g += blockDim.x) a.norm_sum_p[(size_t)gridDim.x * g + blockIdx.x] = unorm_s[g];
+        for (uint32_t g = threadIdx.x; g < item_groups; g += blockDim.x) a.norm_sum_q[(size_t)gridDim.x * g + blockIdx.x] = inorm_s[g];
+    }
+};
+
+}  // namespace mf

@@ -1,0 +1,147 @@
+// Update rules over dense fp32 P/Q: plain SGD and MPT (fp32 master, binary16 arithmetic).
+//
+// Row layout in registers: lane L holds element L (k = 64) or elements L and L+64 (k = 128); every
+// row access is one or two fully coalesced 256-byte loads.  With that ownership the reference's
+// summation order -- warp lane l adds elements l, l+32, l+64, l+96 as ((a+b)+(c+d)) and a
+// 16,8,4,2,1 tree follows (sgd/sgd_kernel.h:55-63) -- is reproduced exactly by
+//   t0 = m[L] + m[L^32]; t1 = m[L+64] + m[(L^32)+64]; s = t0 + t1; tree over 16,8,4,2,1,
+// so results are bit-identical to a sequential evaluation in the reference's order.
+#pragma once
+#include "hogwild.h"
+
+namespace mf {
+
+template <int K> struct DenseRow {
+    static constexpr int E = K / 64;
+    float p[E], q[E];
+};
+struct DenseInfo { float r; uint32_t u, v; };
+struct NoPrep {};
+
+template <int K> struct DenseBase {
+    static constexpr int E = K / 64;
+    using Row = DenseRow<K>;
+    using Info = DenseInfo;
+    using Prep = NoPrep;
+    float* P;
+    float* Q;
+    int lane;
+
+    __device__ __forceinline__ Prep prepare(const Rating&, bool) const { return Prep(); }
+    __device__ __forceinline__ Info info(const Rating& my, const Prep&, int j) const
+    {
+        Info i;
+        i.r = bcast(my.r, j);
+        i.u = bcast(my.u, j);
+        i.v = bcast(my.v, j);
+        return i;
+    }
+    __device__ __forceinline__ void load(Row& row, const Info& i) const
+    {
+        const float* pp = P + (size_t)i.u * K + lane;
+        const float* qq = Q + (size_t)i.v * K + lane;
+#pragma unroll
+        for (int e = 0; e < E; ++e) { row.p[e] = pp[64 * e]; row.q[e] = qq[64 * e]; }
+    }
+    __device__ __forceinline__ void store(const Row& row, const Info& i) const
+    {
+        float* pp = P + (size_t)i.u * K + lane;
+        float* qq = Q + (size_t)i.v * K + lane;
+#pragma unroll
+        for (int e = 0; e < E; ++e) { pp[64 * e] = row.p[e]; qq[64 * e] = row.q[e]; }
+    }
+    __device__ __forceinline__ void forward(Row& nxt, const Info& in, const Row& cur, const Info& ic) const
+    {
+        if (in.u == ic.u) {
+#pragma unroll
+            for (int e = 0; e < E; ++e) nxt.p[e] = cur.p[e];
+        }
+        if (in.v == ic.v) {
+#pragma unroll
+            for (int e = 0; e < E; ++e) nxt.q[e] = cur.q[e];
+        }
+    }
+};
+
+// Sum over the k products in the reference order; T is float or half_t, m[e] the product of element L+64e.
+template <int E, class T> __device__ __forceinline__ T dot_reference_order(const T* m)
+{
+    if constexpr (E == 1) {
+        return reduce_wave(m[0], OpAdd());
+    } else {
+        T t0 = step_xor32(m[0], OpAdd());
+        T t1 = step_xor32(m[1], OpAdd());
+        T s = t0 + t1;
+        return reduce_half_wave(s, OpAdd());
+    }
+}
+
+// single_sgd_k128/k64_hogwild_kernel, sgd/sgd_kernel.h:55-76.
+template <int K> struct SgdRule : DenseBase<K> {
+    using Base = DenseBase<K>;
+    using typename Base::Row;
+    using typename Base::Info;
+    static constexpr int E = Base::E;
+    struct Params { float* p; float* q; float lrate; float lambda; };
+    float lrate, lambda;
+
+    __device__ __forceinline__ void init(const Params& a, uint8_t*, int lane_, uint32_t)
+    {
+        this->P = a.p; this->Q = a.q; this->lane = lane_; lrate = a.lrate; lambda = a.lambda;
+    }
+    __device__ __forceinline__ void update(Row& row, const Info& i, uint32_t) const
+    {
+        float m[E];
+#pragma unroll
+        for (int e = 0; e < E; ++e) m[e] = row.p[e] * row.q[e];
+        const float dot = dot_reference_order<E, float>(m);
+        const float ruv = i.r - dot;
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+            const float pe = row.p[e], qe = row.q[e];
+            row.p[e] = pe + lrate * (ruv * qe - lambda * pe);
+            row.q[e] = qe + lrate * (ruv * pe - lambda * qe);
+        }
+        this->store(row, i);
+    }
+    __device__ __forceinline__ void finish(const Params&, uint32_t) const {}
+};
+
+// mpt_sgd_k128/k64_hogwild_kernel, mpt/mpt_sgd_kernel.h:15-16,38-91.
+template <int K> struct MptRule : DenseBase<K> {
+    using Base = DenseBase<K>;
+    using typename Base::Row;
+    using typename Base::Info;
+    static constexpr int E = Base::E;
+    struct Params { float* p; float* q; float lrate; uint16_t scaled_lambda_half; float scaling_factor; };
+    float lrate, scaling_factor_rev;
+    half_t lambda_h, scaling_factor_h;
+
+    __device__ __forceinline__ void init(const Params& a, uint8_t*, int lane_, uint32_t)
+    {
+        this->P = a.p; this->Q = a.q; this->lane = lane_; lrate = a.lrate;
+        scaling_factor_rev = 1 / a.scaling_factor;
+        scaling_factor_h = (half_t)a.scaling_factor;
+        lambda_h = from_bits<half_t>(a.scaled_lambda_half);
+    }
+    __device__ __forceinline__ void update(Row& row, const Info& i, uint32_t) const
+    {
+        const half_t r_h = (half_t)i.r;
+        half_t ph[E], qh[E], m[E];
+#pragma unroll
+        for (int e = 0; e < E; ++e) { ph[e] = (half_t)row.p[e]; qh[e] = (half_t)row.q[e]; m[e] = ph[e] * qh[e]; }
+        const half_t dot = dot_reference_order<E, half_t>(m);
+        const half_t ruv = scaling_factor_h * (r_h - dot);
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+            const half_t gp = ruv * qh[e] - lambda_h * ph[e];
+            const half_t gq = ruv * ph[e] - lambda_h * qh[e];
+            row.p[e] = row.p[e] + (lrate * (scaling_factor_rev * (float)gp));
+            row.q[e] = row.q[e] + (lrate * (scaling_factor_rev * (float)gq));
+        }
+        this->store(row, i);
+    }
+    __device__ __forceinline__ void finish(const Params&, uint32_t) const {}
+};
+
+}  // namespace mf

@@ -1,0 +1,162 @@
+/*
+ * libmascot_hip -- C ABI of the MI355X (gfx950) matrix-factorization training path.
+ *
+ * Every entry point below stands in for one kernel launch (or one host driver) of
+ * Yujaeseo/ICDM-2021_MASCOT; the comment on each names the reference file:line it
+ * replaces (paths relative to the reference checkout).  Conventions:
+ *   - plain C types only; all pointers are DEVICE pointers unless a parameter is
+ *     documented as host memory; the caller owns every buffer;
+ *   - `stream` is a hipStream_t passed as void* (NULL = default stream); launches are
+ *     asynchronous, nothing here synchronises unless documented;
+ *   - return value: 0 on success, a positive hipError_t when the HIP runtime refused
+ *     something, MF_EINVAL (-1) for arguments the kernels cannot take (the call then
+ *     launches nothing); mf_last_error() gives the message of the last failure on the
+ *     calling thread;
+ *   - a "worker" is one 64-lane wavefront processing one rating at a time, the
+ *     counterpart of the reference's 32-lane warp (`-wg`); k is 64 or 128.
+ *
+ * Scheduling.  A launch runs `num_workers` workers; each runs `update_count` windows of
+ * `update_vector_size` consecutive ratings (offset = (start + i) % nnz), as
+ * sgd/sgd_kernel.h:14-37 does.  The reference draws `start` from cuRAND states seeded
+ * with clock() (model_init.cu:12-17); here it is
+ *     start = window_start[ite * num_workers + worker] % nnz     if window_start != NULL
+ *     start = counter_rng(seed, epoch, worker, ite) * nnz        otherwise
+ * so that a run is reproducible and a caller (or a test) can pin the schedule.
+ */
+#ifndef MASCOT_HIP_H
+#define MASCOT_HIP_H
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MF_OK 0
+#define MF_EINVAL (-1)
+
+/* COO rating triple, common_struct.h:8-12 (12 bytes, array of structures). */
+typedef struct { float r; uint32_t u; uint32_t i; } mf_node;
+
+int mf_version(void);
+const char* mf_last_error(void);
+/* Number of per-block columns mf_mascot_sgd_hogwild writes into norm_sum_p / norm_sum_q
+ * (the reference's `block_num`, mf_methods.cu:109). */
+uint32_t mf_mascot_norm_blocks(uint32_t num_workers);
+/* Host-side closed forms of the schedule (mf_methods.cu:94-111,170-175). */
+uint32_t mf_update_count(uint32_t n, uint32_t num_workers, uint32_t update_vector_size);
+uint32_t mf_first_sample_rating_idx(uint32_t e, uint32_t interval, uint32_t epochs, uint32_t update_count,
+                                    uint32_t update_vector_size, float sample_ratio);
+float mf_lr_schedule(float lr, float decay, uint32_t e);
+/* The counter-based window start the kernels use when window_start == NULL (host twin). */
+uint32_t mf_window_start(uint64_t seed, uint32_t epoch, uint32_t worker, uint32_t ite, uint32_t nnz);
+
+/* ---- Hogwild SGD update launches ---------------------------------------------------- */
+
+/* single_sgd_k128/k64_hogwild_kernel, sgd/sgd_kernel.h:1-79, sgd/sgd_kernel_k64.h:1-67;
+ * launch site mf_methods.cu:879-905.  p: [users][k] fp32, q: [items][k] fp32. */
+int mf_single_sgd_hogwild(const mf_node* R, uint32_t nnz, float* p, float* q, int k,
+                          uint32_t num_workers, uint32_t update_count, uint32_t update_vector_size,
+                          float lrate, float lambda,
+                          uint64_t seed, uint32_t epoch, const uint32_t* window_start, void* stream);
+
+/* mpt_sgd_k128/k64_hogwild_kernel, mpt/mpt_sgd_kernel.h:1-93, mpt/mpt_sgd_kernel_k64.h;
+ * launch site mf_methods.cu:772-799.  scaled_lambda_half = binary16 bits of lambda*scaling_factor
+ * (mf_methods.cu:764-765). */
+int mf_mpt_sgd_hogwild(const mf_node* R, uint32_t nnz, float* p, float* q, int k,
+                       uint32_t num_workers, uint32_t update_count, uint32_t update_vector_size,
+                       float lrate, uint16_t scaled_lambda_half, float scaling_factor,
+                       uint64_t seed, uint32_t epoch, const uint32_t* window_start, void* stream);
+
+/* muppet_sgd_k128/k64_hogwild_kernel, muppet/muppet_sgd_kernel.h:50-292, _k64.h; launch site
+ * mf_methods.cu:613-647.  sum_updated_val: [k] (+=, caller zeroes, mf_methods.cu:606-607);
+ * sum_norms: [num_workers] (overwritten).  Precisions are 8, 12, 14, 16 or 32. */
+int mf_muppet_sgd_hogwild(const mf_node* R, uint32_t nnz, float* p, float* q, int k,
+                          uint32_t num_workers, uint32_t update_count, uint32_t update_vector_size,
+                          float lrate, float lambda, uint32_t first_sample_rating_idx,
+                          float* sum_updated_val, float* sum_norms,
+                          uint8_t forward_prop_precision, uint8_t backward_prop_precision,
+                          uint64_t seed, uint32_t epoch, const uint32_t* window_start, void* stream);
+
+/* afp_sgd_k128/k64_hogwild_kernel, afp/afp_sgd_kernel.h:127-375, _k64.h; launch site
+ * mf_methods.cu:480-507.  `afp_epoch` is the kernel's `epoch` argument (first tenth of
+ * epoch 0 re-measures every update). */
+int mf_afp_sgd_hogwild(const mf_node* R, uint32_t nnz, float* p, float* q, int k,
+                       uint32_t num_workers, uint32_t update_count, uint32_t update_vector_size,
+                       float lrate, float lambda, int afp_epoch,
+                       uint64_t seed, uint32_t epoch, const uint32_t* window_start, void* stream);
+
+/* mascot_sgd_k128/k64_hogwild_kernel, mascot/mascot_sgd_kernel.h:1-457, _k64.h:1-397; launch
+ * site mf_methods.cu:189-237.
+ *   p, q              device arrays of user_group_num / item_group_num device pointers; group g is
+ *                     [group_size][k] binary16 (prec 0) or binary32 (prec 1), rows in sorted order
+ *   *_group_end_idx   inclusive last sorted row of each group (preprocess_utils.h:189-213)
+ *   *_group_prec_info one byte per group
+ *   grad_sum_norm_*   [groups][k] fp32, += of the sampled gradients (caller zeroes on check epochs)
+ *   norm_sum_*        [groups][mf_mascot_norm_blocks(num_workers)] fp32, overwritten
+ *   ratings with processed index >= first_sample_rating_idx are sampled. */
+int mf_mascot_sgd_hogwild(const mf_node* R, uint32_t nnz, void* const* p, void* const* q, int k,
+                          uint32_t num_workers, uint32_t update_count, uint32_t update_vector_size,
+                          float lrate, float lambda,
+                          const uint32_t* user_group_end_idx, const uint32_t* item_group_end_idx,
+                          const uint8_t* user_group_prec_info, const uint8_t* item_group_prec_info,
+                          float* grad_sum_norm_p, float* grad_sum_norm_q, float* norm_sum_p, float* norm_sum_q,
+                          uint32_t first_sample_rating_idx, uint32_t user_group_num, uint32_t item_group_num,
+                          uint64_t seed, uint32_t epoch, const uint32_t* window_start, void* stream);
+
+/* ---- m-quantization: conversion and grouped storage ---------------------------------- */
+
+/* transform_float2half, model_init.cu:96-105 (round to nearest even). */
+int mf_transform_float2half(const float* in, uint16_t* out, uint64_t n, void* stream);
+/* transform_half2float / mem_cpy_fp16tofp32 / mem_cpy_fp162fp32, model_init.cu:85-112,
+ * precision_switching.h:1-6 (exact widening; promotes one group on a precision switch). */
+int mf_transform_half2float(const uint16_t* in, float* out, uint64_t n, void* stream);
+/* cpyparams2grouped_params_for_comparison_indexing(+_k64), model_init.cu:30-83: row e of the dense
+ * fp32 matrix -> binary16 row (entity2sorted_idx[e] - first row of its group) of group entity2group[e]. */
+int mf_cpyparams2grouped_params(const float* original_params, void* const* converted_params,
+                                const uint32_t* group_end_idx, const uint32_t* entity2group,
+                                const uint32_t* entity2sorted_idx, int k, uint32_t n, uint32_t group_num, void* stream);
+/* The gather the reference does on the host every epoch (mf_methods.cu:249-313): grouped storage
+ * -> dense fp32 [n][k] in sorted row order, widening binary16 groups exactly. */
+int mf_grouped_params2dense(void* const* group_ptr, const uint32_t* group_end_idx, const uint8_t* group_prec_info,
+                            float* dense, int k, uint32_t n, uint32_t group_num, void* stream);
+
+/* ---- g-switching: error estimate and evaluation -------------------------------------- */
+
+/* Per-group error of mf_methods.cu:327-379 on the device:
+ *   error[g] = (sum_k grad_sum_norm[g][k]^2) / (sum_b norm_sum[g][b]) / initial_error[g],  -1 for fp32 groups.
+ * grad_sum_norm is zeroed afterwards like the host loop does (mf_methods.cu:333). */
+int mf_group_error(float* grad_sum_norm, const float* norm_sum, uint32_t norm_blocks, const uint8_t* group_prec_info,
+                   const float* initial_error, float* error_out, int k, uint32_t group_num, void* stream);
+/* get_test_rmse_coalesced_k128/k64 + host finish, rmse.h:26-189.  Adds sum((r - p.q)^2) over the test
+ * ratings into *sum_sq (one device double, caller zeroes); rmse = sqrt(sum_sq / test_n). */
+int mf_test_rmse(const mf_node* test, uint32_t test_n, const float* p, const float* q, int k,
+                 double* sum_sq, void* stream);
+/* Same, reading grouped storage directly (no host gather, no H2D of P and Q). */
+int mf_test_rmse_grouped(const mf_node* test, uint32_t test_n, void* const* p, void* const* q, int k,
+                         const uint32_t* user_group_end_idx, const uint32_t* item_group_end_idx,
+                         const uint8_t* user_group_prec_info, const uint8_t* item_group_prec_info,
+                         uint32_t user_group_num, uint32_t item_group_num, double* sum_sq, void* stream);
+
+/* ---- model init and preprocessing ----------------------------------------------------- */
+
+/* init_rand_state + init_rand_feature_single, model_init.cu:12-28: array[i] = (float)(N(0,1) * 0.01),
+ * from a counter-based generator keyed by (seed, stream_id, i) instead of clock()-seeded cuRAND states. */
+int mf_init_rand_feature(float* array, uint64_t n, uint64_t seed, uint64_t stream_id, void* stream);
+/* init_idx_arr, preprocess_utils.h:6-11. */
+int mf_init_idx_arr(uint32_t* arr, uint32_t n, void* stream);
+/* user_item_histogram, preprocess_utils.h:13-19 (caller zeroes the bins). */
+int mf_user_item_histogram(const mf_node* R, uint32_t n, uint32_t* user_bin, uint32_t* item_bin, void* stream);
+/* thrust::sort_by_key(cnt, idx), preprocess_utils.h:87-88: ascending stable sort of the counts carrying
+ * the ids, in place.  Allocates its temporary storage with hipMalloc and synchronises the stream. */
+int mf_sort_by_count(uint32_t* cnt, uint32_t* idx, uint32_t n, void* stream);
+/* matrix_reconst_gpu_triplet, preprocess_utils.h:28-36 (in place). */
+int mf_matrix_reconst_triplet(mf_node* R, const uint32_t* user2sorted_idx, const uint32_t* item2sorted_idx,
+                              uint32_t n, void* stream);
+/* Seeded replacement for srand(time(0)); std::random_shuffle(R, R+n) (mf_methods.cu:38-39): out = in
+ * permuted by ascending 64-bit key(seed, i).  Allocates temporaries with hipMalloc, synchronises. */
+int mf_shuffle_ratings(const mf_node* in, mf_node* out, uint32_t n, uint64_t seed, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,223 @@
+"""GPU parity of the five Hogwild update kernels against the CPU checker, through the C ABI.
+
+Schedules are conflict-free (each worker owns its users and items), so any interleaving of the
+wavefronts must equal the checker's sequential run.  Bar: bit-exact for every variant (the kernels
+reproduce the reference's order of roundings); sampled float sums that go through atomics are compared
+to 1e-5 relative."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import mfutil
+from mfutil import to_dev, from_dev
+
+pytestmark = pytest.mark.gpu
+
+LR, LAM = 0.01, 0.05
+
+
+def _run_dense(variant, k, R, starts, P, Q, uc, window, extra=()):
+    h = mfutil.hip()
+    W = starts.shape[1]
+    dR, dS, dP, dQ = to_dev(R), to_dev(starts), to_dev(P), to_dev(Q)
+    fn = getattr(h, "mf_%s_sgd_hogwild" % variant)
+    fn(dR.data_ptr(), R.size, dP.data_ptr(), dQ.data_ptr(), k, W, uc, window, *extra, 1234, 0, dS.data_ptr(), mfutil.stream_ptr())
+    import torch
+    torch.cuda.synchronize()
+    return from_dev(dP, np.float32, P.shape), from_dev(dQ, np.float32, Q.shape)
+
+
+@pytest.mark.parametrize("k", [64, 128])
+@pytest.mark.parametrize("W,uc,window", [(1, 1, 1), (6, 3, 128), (9, 2, 70), (64, 2, 128)])
+def test_sgd_fp32_bit_exact(orc, k, W, uc, window):
+    R, starts, P, Q = mfutil.conflict_free_problem(10 + k + W, k, W, uc, window)
+    gp, gq = _run_dense("single", k, R, starts, P, Q, uc, window, (LR, LAM))
+    orc.lib.orc_sgd_epoch(k, R.ctypes.data, R.size, P.ctypes.data, Q.ctypes.data, W, uc, window, LR, LAM, 0, 0, starts.ctypes.data, 1)
+    assert np.array_equal(gp.view(np.uint32), P.view(np.uint32))
+    assert np.array_equal(gq.view(np.uint32), Q.view(np.uint32))
+
+
+@pytest.mark.parametrize("k", [64, 128])
+@pytest.mark.parametrize("W,uc,window", [(1, 1, 1), (7, 3, 128), (64, 2, 128)])
+def test_mpt_bit_exact(orc, k, W, uc, window):
+    R, starts, P, Q = mfutil.conflict_free_problem(20 + k + W, k, W, uc, window)
+    # MPT's master copy starts from binary16-representable values (main.cu:152-153, mf_methods.cu:730-733)
+    P = orc.h2f(orc.f2h(P)); Q = orc.h2f(orc.f2h(Q))
+    lam_h = orc.lib.orc_float2half(np.float32(LAM) * np.float32(1000.0))
+    gp, gq = _run_dense("mpt", k, R, starts, P, Q, uc, window, (LR, lam_h, 1000.0))
+    orc.lib.orc_mpt_epoch(k, R.ctypes.data, R.size, P.ctypes.data, Q.ctypes.data, W, uc, window, LR, LAM, 1000.0, 0, 0, starts.ctypes.data, 1)
+    assert np.array_equal(gp.view(np.uint32), P.view(np.uint32))
+    assert np.array_equal(gq.view(np.uint32), Q.view(np.uint32))
+
+
+@pytest.mark.parametrize("k", [64, 128])
+@pytest.mark.parametrize("bits", [8, 12, 14, 16, 32])
+def test_muppet_bit_exact(orc, k, bits):
+    W, uc, window = 10, 2, 128
+    R, starts, P, Q = mfutil.conflict_free_problem(30 + k + bits, k, W, uc, window)
+    first_sample = window  # second window of every worker is sampled
+    import torch
+    h = mfutil.hip()
+    dR, dS, dP, dQ = to_dev(R), to_dev(starts), to_dev(P), to_dev(Q)
+    d_sum = torch.zeros(k, dtype=torch.float32, device="cuda")
+    d_norm = torch.full((W,), -7.0, dtype=torch.float32, device="cuda")
+    h.mf_muppet_sgd_hogwild(dR.data_ptr(), R.size, dP.data_ptr(), dQ.data_ptr(), k, W, uc, window, LR, LAM, first_sample,
+                            d_sum.data_ptr(), d_norm.data_ptr(), bits, bits, 0, 0, dS.data_ptr(), mfutil.stream_ptr())
+    torch.cuda.synchronize()
+    sum_ref = np.zeros(k, np.float32)
+    norm_ref = np.zeros(W, np.float32)
+    orc.lib.orc_muppet_epoch(k, R.ctypes.data, R.size, P.ctypes.data, Q.ctypes.data, W, uc, window, LR, LAM, first_sample,
+                             sum_ref.ctypes.data, norm_ref.ctypes.data, bits, bits, 0, 0, starts.ctypes.data, 1)
+    assert np.array_equal(from_dev(dP, np.float32, P.shape).view(np.uint32), P.view(np.uint32))
+    assert np.array_equal(from_dev(dQ, np.float32, Q.shape).view(np.uint32), Q.view(np.uint32))
+    assert np.array_equal(d_norm.cpu().numpy().view(np.uint32), norm_ref.view(np.uint32))
+    got = d_sum.cpu().numpy()
+    if bits == 32:
+        assert np.all(got == 0) and np.all(sum_ref == 0)
+    else:
+        scale = np.abs(sum_ref).max()
+        assert np.allclose(got, sum_ref, rtol=1e-5, atol=1e-5 * scale)
+
+
+@pytest.mark.parametrize("k", [64, 128])
+@pytest.mark.parametrize("afp_epoch", [0, 3])
+def test_afp_bit_exact(orc, k, afp_epoch):
+    W, uc, window = 10, 3, 128
+    R, starts, P, Q = mfutil.conflict_free_problem(40 + k + afp_epoch, k, W, uc, window)
+    gp, gq = _run_dense("afp", k, R, starts, P, Q, uc, window, (LR, LAM, afp_epoch))
+    orc.lib.orc_afp_epoch(k, R.ctypes.data, R.size, P.ctypes.data, Q.ctypes.data, W, uc, window, LR, LAM, afp_epoch, 0, 0, starts.ctypes.data, 1)
+    assert np.array_equal(gp.view(np.uint32), P.view(np.uint32))
+    assert np.array_equal(gq.view(np.uint32), Q.view(np.uint32))
+
+
+def _mascot_case(orc, k, W, uc, window, user_groups, item_groups, prec_mode, first_sample, seed):
+    import torch
+    h = mfutil.hip()
+    R, starts, P, Q = mfutil.conflict_free_problem(seed, k, W, uc, window)
+    n_users, n_items = P.shape[0], Q.shape[0]
+    uend, iend = mfutil.equal_end_idx(n_users, user_groups), mfutil.equal_end_idx(n_items, item_groups)
+    rng = np.random.default_rng(seed)
+    if prec_mode == "half":
+        uprec, iprec = np.zeros(user_groups, np.uint8), np.zeros(item_groups, np.uint8)
+    elif prec_mode == "float":
+        uprec, iprec = np.ones(user_groups, np.uint8), np.ones(item_groups, np.uint8)
+    else:
+        uprec, iprec = rng.integers(0, 2, user_groups).astype(np.uint8), rng.integers(0, 2, item_groups).astype(np.uint8)
+    gmp, gmq = mfutil.host_grouped(orc, k, P, uend, uprec), mfutil.host_grouped(orc, k, Q, iend, iprec)
+    dp, dq = mfutil.DeviceGrouped(gmp), mfutil.DeviceGrouped(gmq)
+    nb = h.mf_mascot_norm_blocks(W)
+    dR, dS = to_dev(R), to_dev(starts)
+    d_gsp = torch.zeros(user_groups * k, dtype=torch.float32, device="cuda")
+    d_gsq = torch.zeros(item_groups * k, dtype=torch.float32, device="cuda")
+    d_nsp = torch.full((user_groups * nb,), -3.0, dtype=torch.float32, device="cuda")
+    d_nsq = torch.full((item_groups * nb,), -3.0, dtype=torch.float32, device="cuda")
+    h.mf_mascot_sgd_hogwild(dR.data_ptr(), R.size, dp.ptrs.data_ptr(), dq.ptrs.data_ptr(), k, W, uc, window, LR, LAM,
+                            dp.end.data_ptr(), dq.end.data_ptr(), dp.prec.data_ptr(), dq.prec.data_ptr(),
+                            d_gsp.data_ptr(), d_gsq.data_ptr(), d_nsp.data_ptr(), d_nsq.data_ptr(),
+                            first_sample, user_groups, item_groups, 0, 0, dS.data_ptr(), mfutil.stream_ptr())
+    torch.cuda.synchronize()
+    gsp, gsq = np.zeros(user_groups * k, np.float32), np.zeros(item_groups * k, np.float32)
+    nsp, nsq = np.zeros(user_groups, np.float32), np.zeros(item_groups, np.float32)
+    orc.lib.orc_mascot_epoch(k, R.ctypes.data, R.size, gmp.ptrs, gmq.ptrs, gmp.end_idx.ctypes.data, gmq.end_idx.ctypes.data,
+                             gmp.prec.ctypes.data, gmq.prec.ctypes.data, user_groups, item_groups, W, uc, window, LR, LAM,
+                             first_sample, gsp.ctypes.data, gsq.ctypes.data, nsp.ctypes.data, nsq.ctypes.data,
+                             0, 0, starts.ctypes.data, 1)
+    for got, want in zip(dp.download() + dq.download(), gmp.arrays + gmq.arrays):
+        assert got.dtype == want.dtype
+        assert np.array_equal(got.view(np.uint8), want.view(np.uint8))
+    got_nsp = d_nsp.cpu().numpy().reshape(user_groups, nb).astype(np.float64).sum(1)
+    got_nsq = d_nsq.cpu().numpy().reshape(item_groups, nb).astype(np.float64).sum(1)
+    assert np.allclose(got_nsp, nsp, rtol=1e-5, atol=1e-7)
+    assert np.allclose(got_nsq, nsq, rtol=1e-5, atol=1e-7)
+    for got, want in ((d_gsp.cpu().numpy(), gsp), (d_gsq.cpu().numpy(), gsq)):
+        scale = max(np.abs(want).max(), 1e-6)
+        assert np.allclose(got, want, rtol=1e-5, atol=2e-5 * scale)
+    return nsp, nsq
+
+
+@pytest.mark.parametrize("k", [64, 128])
+@pytest.mark.parametrize("prec_mode", ["half", "float", "mixed"])
+def test_mascot_bit_exact(orc, k, prec_mode):
+    W, uc, window = 12, 3, 128
+    nsp, nsq = _mascot_case(orc, k, W, uc, window, 7, 5, prec_mode, first_sample=2 * window - 40, seed=50 + k)
+    if prec_mode == "half":
+        assert nsp.sum() > 0 and nsq.sum() > 0
+    if prec_mode == "float":
+        assert nsp.sum() == 0 and nsq.sum() == 0
+
+
+@pytest.mark.parametrize("k", [64, 128])
+def test_mascot_group_table_sizes(orc, k):
+    # one group per side, and more groups than a 64-lane compare could hold
+    _mascot_case(orc, k, 4, 1, 128, 1, 1, "half", first_sample=128, seed=61)
+    _mascot_case(orc, k, 40, 1, 64, 150, 101, "mixed", first_sample=0, seed=62)
+
+
+@pytest.mark.parametrize("k", [64, 128])
+def test_single_update_mascot_four_cases(orc, k):
+    for up in (0, 1):
+        for ip in (0, 1):
+            import torch
+            h = mfutil.hip()
+            rng = np.random.default_rng(70 + 2 * up + ip)
+            P = (rng.standard_normal((1, k)) * 0.1).astype(np.float32)
+            Q = (rng.standard_normal((1, k)) * 0.1).astype(np.float32)
+            R = np.zeros(1, mfutil.NODE); R["r"] = 4.0
+            gmp = mfutil.host_grouped(orc, k, P, np.array([0], np.uint32), np.array([up], np.uint8))
+            gmq = mfutil.host_grouped(orc, k, Q, np.array([0], np.uint32), np.array([ip], np.uint8))
+            dp, dq = mfutil.DeviceGrouped(gmp), mfutil.DeviceGrouped(gmq)
+            dR = to_dev(R); dS = to_dev(np.zeros((1, 1), np.uint32))
+            z = torch.zeros(4 * k, dtype=torch.float32, device="cuda")
+            h.mf_mascot_sgd_hogwild(dR.data_ptr(), 1, dp.ptrs.data_ptr(), dq.ptrs.data_ptr(), k, 1, 1, 1, LR, LAM,
+                                    dp.end.data_ptr(), dq.end.data_ptr(), dp.prec.data_ptr(), dq.prec.data_ptr(),
+                                    z.data_ptr(), z[k:].data_ptr(), z[2 * k:].data_ptr(), z[3 * k:].data_ptr(),
+                                    1, 1, 1, 0, 0, dS.data_ptr(), mfutil.stream_ptr())
+            torch.cuda.synchronize()
+            orc.lib.orc_mascot_update(k, gmp.arrays[0].ctypes.data, up, gmq.arrays[0].ctypes.data, ip, 4.0, LR, LAM, None, None, None, None)
+            assert np.array_equal(dp.download()[0].view(np.uint8), gmp.arrays[0].view(np.uint8)), (up, ip)
+            assert np.array_equal(dq.download()[0].view(np.uint8), gmq.arrays[0].view(np.uint8)), (up, ip)
+
+
+@pytest.mark.parametrize("k", [64, 128])
+def test_counter_rng_schedule_matches_checker(orc, k):
+    """window_start == NULL: the kernel's own generator must pick the windows the checker's twin picks."""
+    h = mfutil.hip()
+    rng = np.random.default_rng(80)
+    R = mfutil.make_ratings(81, 50, 40, 3000)
+    P = (rng.standard_normal((50, k)) * 0.1).astype(np.float32)
+    Q = (rng.standard_normal((40, k)) * 0.1).astype(np.float32)
+    for e in range(3):
+        for w in range(5):
+            assert h.mf_window_start(99, e, w, 7, R.size) == orc.lib.orc_window_start(99, e, w, 7, R.size)
+    import torch
+    dR, dP, dQ = to_dev(R), to_dev(P), to_dev(Q)
+    h.mf_single_sgd_hogwild(dR.data_ptr(), R.size, dP.data_ptr(), dQ.data_ptr(), k, 1, 6, 128, LR, LAM, 99, 2, None, mfutil.stream_ptr())
+    torch.cuda.synchronize()
+    orc.lib.orc_sgd_epoch(k, R.ctypes.data, R.size, P.ctypes.data, Q.ctypes.data, 1, 6, 128, LR, LAM, 99, 2, None, 1)
+    assert np.array_equal(from_dev(dP, np.float32, P.shape).view(np.uint32), P.view(np.uint32))
+    assert np.array_equal(from_dev(dQ, np.float32, Q.shape).view(np.uint32), Q.view(np.uint32))
+
+
+def test_window_wraps_past_end_of_ratings(orc):
+    """nnz smaller than the window: offset = (start + i) % nnz wraps several times (sgd_kernel.h:33)."""
+    k = 64
+    rng = np.random.default_rng(90)
+    R = mfutil.make_ratings(91, 6, 5, 50)
+    P = (rng.standard_normal((6, k)) * 0.1).astype(np.float32)
+    Q = (rng.standard_normal((5, k)) * 0.1).astype(np.float32)
+    starts = np.array([[47], [3]], np.uint32)
+    gp, gq = _run_dense("single", k, R, starts, P, Q, 2, 128, (LR, LAM))
+    orc.lib.orc_sgd_epoch(k, R.ctypes.data, R.size, P.ctypes.data, Q.ctypes.data, 1, 2, 128, LR, LAM, 0, 0, starts.ctypes.data, 1)
+    assert np.array_equal(gp.view(np.uint32), P.view(np.uint32))
+    assert np.array_equal(gq.view(np.uint32), Q.view(np.uint32))
+
+
+def test_argument_errors_launch_nothing():
+    h = mfutil.hip()
+    from importlib import import_module
+    MfError = import_module("icdm-2021_mascot_amd.capi").MfError
+    with pytest.raises(MfError, match="k must be 64 or 128"):
+        h.mf_single_sgd_hogwild(1, 1, 1, 1, 32, 1, 1, 1, LR, LAM, 0, 0, None, None)
+    with pytest.raises(MfError, match="empty rating array"):
+        h.mf_single_sgd_hogwild(None, 0, 1, 1, 64, 1, 1, 1, LR, LAM, 0, 0, None, None)
