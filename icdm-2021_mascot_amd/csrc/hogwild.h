@@ -1,19 +1,66 @@
 // The Hogwild driver loop shared by every update kernel (sgd/sgd_kernel.h:14-37 of the
-// reference, redesigned for wave64):
+// reference, redesigned for wave64 and for memory-level parallelism):
 //   * one wavefront = one worker; it walks update_count windows of update_vector_size ratings;
-//   * a window is consumed in chunks of 64 ratings: one coalesced streaming load puts rating j of
-//     the chunk in lane j, anything that can be computed per rating without the rows (group search,
-//     row addresses) is done once, vectorised across the 64 lanes, and the per-rating loop then
-//     broadcasts lane j's scalars with v_readlane;
-//   * the rows of rating j+1 are requested before rating j is reduced and stored, so one rating's
-//     memory latency hides behind the previous rating's arithmetic.  When consecutive ratings touch
-//     the same row the freshly computed row is forwarded in registers, so a worker's own updates
-//     are applied strictly in order (needed for bit-exact checks; other workers still race, that is
-//     Hogwild).
+//   * a window is consumed in chunks of up to 64 ratings: one coalesced streaming load puts rating j
+//     of the chunk in lane j (the next chunk's ratings are requested while the current chunk runs),
+//     everything that does not need the rows (group search, row addresses) is computed once,
+//     vectorised across the 64 lanes, and the per-rating loop broadcasts lane j's scalars with
+//     v_readlane;
+//   * the per-rating loop is a software pipeline over a ring of kRing register slots: the rows of
+//     rating j+kAhead are requested before rating j is reduced, updated and stored, so kAhead+1
+//     ratings of a wavefront are in flight and a row's latency hides behind kAhead updates;
+//   * a row requested early can be stale if one of the kAhead ratings in between updates the same
+//     row.  Row identities are wave-uniform scalars, so that is a scalar compare per older slot; on
+//     a match the freshly computed row is forwarded from that slot's registers.  A worker therefore
+//     applies its own updates strictly in order (what a bit-exact check needs); different workers
+//     still race on P and Q without atomics -- that is Hogwild.
 #pragma once
 #include "mf_device.h"
+#include <type_traits>
 
 namespace mf {
+
+template <int I, int N, class F> __device__ __forceinline__ void static_for(F&& f)
+{
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>());
+        static_for<I + 1, N>(f);
+    }
+}
+
+template <class Rule, int CLS>
+__device__ __forceinline__ void process_chunk(Rule& rule, const Rating& my, const typename Rule::Prep& prep, int n, uint32_t processed)
+{
+    constexpr int A = Rule::kAhead;
+    constexpr int S = Rule::kRing;
+    static_assert(S >= 2 * A + 1, "ring must keep kAhead finished rows next to kAhead+1 pending ones");
+    typename Rule::Row ring[S];
+    typename Rule::Info inf[S];
+    static_for<0, A>([&](auto D) {
+        constexpr int d = decltype(D)::value;
+        if (d < n) { inf[d] = rule.info(my, prep, d); rule.template load<CLS>(ring[d], inf[d]); }
+    });
+    for (int j0 = 0; j0 < n; j0 += S) {
+        static_for<0, S>([&](auto D) {
+            constexpr int d = decltype(D)::value;
+            const int j = j0 + d;
+            if (j < n) {
+                if (j + A < n) {
+                    constexpr int sl = (d + A) % S;
+                    inf[sl] = rule.info(my, prep, j + A);
+                    rule.template load<CLS>(ring[sl], inf[sl]);
+                }
+                // rows this rating shares with one of the previous kAhead ratings: newest wins
+                static_for<0, A>([&](auto H) {
+                    constexpr int h = A - decltype(H)::value;          // A, A-1, ..., 1
+                    constexpr int sh = (d - h + 2 * S) % S;
+                    if (j >= h) rule.forward(ring[d], inf[d], ring[sh], inf[sh]);
+                });
+                rule.template update<CLS>(ring[d], inf[d], processed + (uint32_t)j);
+            }
+        });
+    }
+}
 
 template <class Rule>
 __global__ __launch_bounds__(kBlock) void hogwild_kernel(Schedule s, typename Rule::Params prm)
@@ -23,42 +70,54 @@ __global__ __launch_bounds__(kBlock) void hogwild_kernel(Schedule s, typename Ru
     const uint32_t wid = (uint32_t)__builtin_amdgcn_readfirstlane((int)(blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6)));
     Rule rule;
     rule.init(prm, smem, lane, wid);                    // may synchronise the workgroup
-    if (wid < s.num_workers) {
-        uint32_t processed = 0;
-        for (uint32_t ite = 0; ite < s.update_count; ++ite) {
-            uint32_t start;
-            if (s.window_start) start = s.window_start[(size_t)ite * s.num_workers + wid] % s.nnz;
-            else start = window_start_rng(s.epoch_key, wid, ite, s.nnz);
-            start = (uint32_t)__builtin_amdgcn_readfirstlane((int)start);
-            for (uint32_t c = 0; c < s.update_vector_size; c += kWave) {
-                const uint32_t left = s.update_vector_size - c;
-                const int n = left < (uint32_t)kWave ? (int)left : kWave;
-                const bool valid = lane < n;
-                Rating my = {0.f, 0u, 0u};
-                if (valid) {
-                    uint32_t off = (c + (uint32_t)lane) % s.nnz;
-                    uint32_t idx = start + off;
-                    if (idx >= s.nnz || idx < start) idx -= s.nnz;
-                    my = load_rating(s.R, idx);
-                }
-                typename Rule::Prep prep = rule.prepare(my, valid);
-                typename Rule::Info ic = rule.info(my, prep, 0);
-                typename Rule::Row cur, nxt;
-                rule.load(cur, ic);
-                for (int j = 0; j < n; ++j) {
-                    const bool has_next = (j + 1) < n;
-                    typename Rule::Info in = ic;
-                    if (has_next) {
-                        in = rule.info(my, prep, j + 1);
-                        rule.load(nxt, in);
-                    }
-                    rule.update(cur, ic, processed);
-                    if (has_next) rule.forward(nxt, in, cur, ic);
-                    cur = nxt;
-                    ic = in;
-                    ++processed;
-                }
+    if (wid < s.num_workers && s.range_begin < s.range_end) {
+        // this worker handles ratings with processed index in [range_begin, range_end)
+        uint32_t processed = s.range_begin;
+        uint32_t ite = s.range_begin / s.update_vector_size;
+        uint32_t c = s.range_begin - ite * s.update_vector_size;
+        auto window_of = [&](uint32_t it) -> uint32_t {
+            uint32_t st;
+            if (s.window_start) st = s.window_start[(size_t)it * s.num_workers + wid] % s.nnz;
+            else st = window_start_rng(s.epoch_key, wid, it, s.nnz);
+            return (uint32_t)__builtin_amdgcn_readfirstlane((int)st);
+        };
+        auto chunk_len = [&](uint32_t cc, uint32_t pp) -> int {
+            uint32_t left = s.update_vector_size - cc;
+            if (left > s.range_end - pp) left = s.range_end - pp;
+            return left < (uint32_t)kWave ? (int)left : kWave;
+        };
+        auto fetch = [&](uint32_t st, uint32_t cc, int nn) -> Rating {
+            Rating x = {0.f, 0u, 0u};
+            if (lane < nn) {
+                uint32_t off = (cc + (uint32_t)lane) % s.nnz;
+                uint32_t idx = st + off;
+                if (idx >= s.nnz || idx < st) idx -= s.nnz;
+                x = load_rating(s.R, idx);
             }
+            return x;
+        };
+        uint32_t start = window_of(ite);
+        int n = chunk_len(c, processed);
+        Rating my = fetch(start, c, n);
+        while (true) {
+            // position of the chunk after this one, and its ratings, requested now
+            uint32_t nprocessed = processed + (uint32_t)n;
+            uint32_t nc = c + (uint32_t)n, nite = ite, nstart = start;
+            const bool more = nprocessed < s.range_end;
+            int nn = 0;
+            Rating nmy = {0.f, 0u, 0u};
+            if (more) {
+                if (nc >= s.update_vector_size) { nc = 0; ++nite; nstart = window_of(nite); }
+                nn = chunk_len(nc, nprocessed);
+                nmy = fetch(nstart, nc, nn);
+            }
+            const bool valid = lane < n;
+            typename Rule::Prep prep = rule.prepare(my, valid);
+            const int cls = rule.classify(prep, valid);
+            if (Rule::kClasses > 1 && cls == 1) process_chunk<Rule, 1>(rule, my, prep, n, processed);
+            else process_chunk<Rule, 0>(rule, my, prep, n, processed);
+            if (!more) break;
+            processed = nprocessed; c = nc; ite = nite; start = nstart; n = nn; my = nmy;
         }
     }
     rule.finish(prm, wid);                               // may synchronise the workgroup

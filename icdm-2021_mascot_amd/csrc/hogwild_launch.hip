@@ -33,7 +33,7 @@ static Schedule make_schedule(const mf_node* R, uint32_t nnz, uint32_t num_worke
 {
     Schedule s;
     s.R = R; s.nnz = nnz; s.num_workers = num_workers; s.update_count = update_count;
-    s.update_vector_size = update_vector_size; s.epoch_key = window_epoch_key(seed, epoch); s.window_start = window_start;
+    s.update_vector_size = update_vector_size; s.range_begin = 0; s.range_end = update_count * update_vector_size; s.epoch_key = window_epoch_key(seed, epoch); s.window_start = window_start;
     return s;
 }
 static inline uint32_t grid_for(uint32_t num_workers) { return (num_workers + kWavesPerBlock - 1) / kWavesPerBlock; }

@@ -122,6 +122,7 @@ struct Schedule {
     uint32_t num_workers;
     uint32_t update_count;
     uint32_t update_vector_size;
+    uint32_t range_begin, range_end;   // processed-index range [begin, end) every worker handles in this launch
     uint64_t epoch_key;
     const uint32_t* window_start;   // optional [update_count][num_workers]
 };

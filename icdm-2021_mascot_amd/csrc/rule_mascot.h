@@ -21,6 +21,10 @@ namespace mf {
 
 template <int K> struct MascotRule {
     static constexpr int E = K / 64;                        // elements per lane
+    static constexpr int kAhead = 3, kRing = 8;
+    // chunk classes: 0 = any mix of precisions (flag-driven), 1 = every rating of the chunk touches two
+    // binary16 rows (the state every group starts in): loads and arithmetic without any branching
+    static constexpr int kClasses = 2;
     using HV = typename std::conditional<E == 2, half2_t, half_t>::type;
 
     struct Params {
@@ -101,6 +105,10 @@ template <int K> struct MascotRule {
         }
         return pr;
     }
+    __device__ __forceinline__ int classify(const Prep& pr, bool valid) const
+    {
+        return __builtin_amdgcn_ballot_w64(valid && (pr.flags & 7u) != 0u) == 0ull ? 1 : 0;
+    }
     __device__ __forceinline__ Info info(const Rating& my, const Prep& pr, int j) const
     {
         Info i;
@@ -135,13 +143,18 @@ template <int K> struct MascotRule {
             else *reinterpret_cast<uint16_t*>(ptr + (uint64_t)lane * 2) = (uint16_t)r[0];
         }
     }
-    __device__ __forceinline__ void load(Row& row, const Info& i) const
+    template <int CLS> __device__ __forceinline__ void load(Row& row, const Info& i) const
     {
+        if constexpr (CLS == 1) {
+            load_side(row.p, i.pptr, false, lane);
+            load_side(row.q, i.qptr, false, lane);
+        } else {
 #pragma unroll
-        for (int e = 0; e < E; ++e) { row.p[e] = 0; row.q[e] = 0; }
-        if (i.flags & kSkip) return;
-        load_side(row.p, i.pptr, i.flags & 1u, lane);
-        load_side(row.q, i.qptr, i.flags & 2u, lane);
+            for (int e = 0; e < E; ++e) { row.p[e] = 0; row.q[e] = 0; }
+            if (i.flags & kSkip) return;
+            load_side(row.p, i.pptr, i.flags & 1u, lane);
+            load_side(row.q, i.qptr, i.flags & 2u, lane);
+        }
     }
     __device__ __forceinline__ void forward(Row& nxt, const Info& in, const Row& cur, const Info& ic) const
     {
@@ -204,10 +217,10 @@ template <int K> struct MascotRule {
         for (int e = 0; e < E; ++e) atomicAdd(dst + e, g[e]);
     }
 
-    __device__ __forceinline__ void update(Row& row, const Info& i, uint32_t processed) const
+    template <int CLS> __device__ __forceinline__ void update(Row& row, const Info& i, uint32_t processed) const
     {
-        if (i.flags & kSkip) return;
-        const bool up = i.flags & 1u, ip = i.flags & 2u;
+        if (CLS == 0 && (i.flags & kSkip)) return;
+        const bool up = CLS == 0 && (i.flags & 1u), ip = CLS == 0 && (i.flags & 2u);
         const bool sampled = processed >= first_sample;
         const uint32_t ug = (i.flags >> 3) & 0x3fffu, ig = (i.flags >> 17) & 0x3fffu;
         if (!up && !ip) {

@@ -74,12 +74,14 @@ template <int K> struct MuppetRule : DenseBase<K> {
     using typename Base::Info;
     static constexpr int E = Base::E;
     static constexpr int J = K / 32;
+    static constexpr int kAhead = 1, kRing = 4;
     struct Params {
         float* p; float* q; float lrate; float lambda; uint32_t first_sample;
         float* sum_updated_val; float* sum_norms; uint32_t num_workers; int fwd; int bwd;
     };
     float lrate, lambda; uint32_t first_sample; float* sum_updated_val; int fwd, bwd;
     float sum_norms_reg;
+    float grad_acc[K / 64];
     bool upper;
 
     __device__ __forceinline__ void init(const Params& a, uint8_t*, int lane_, uint32_t)
@@ -87,8 +89,10 @@ template <int K> struct MuppetRule : DenseBase<K> {
         this->P = a.p; this->Q = a.q; this->lane = lane_; lrate = a.lrate; lambda = a.lambda;
         first_sample = a.first_sample; sum_updated_val = a.sum_updated_val; fwd = a.fwd; bwd = a.bwd;
         sum_norms_reg = 0.f; upper = lane_ >= 32;
+#pragma unroll
+        for (int e = 0; e < E; ++e) grad_acc[e] = 0.f;
     }
-    __device__ __forceinline__ void update(Row& row, const Info& i, uint32_t processed)
+    template <int CLS> __device__ __forceinline__ void update(Row& row, const Info& i, uint32_t processed)
     {
         Mirror<K> p, q;
         p.build(row.p, upper); q.build(row.q, upper);
@@ -167,10 +171,8 @@ template <int K> struct MuppetRule : DenseBase<K> {
         }
 #pragma unroll
         for (int e = 0; e < E; ++e) {
-            const int j = 2 * e + (upper ? 1 : 0);
             float g = upper ? gp[2 * e + 1] : gp[2 * e];
             float h = upper ? gq[2 * e + 1] : gq[2 * e];
-            (void)j;
             row.p[e] = row.p[e] + lrate * g;
             row.q[e] = row.q[e] + lrate * h;
         }
@@ -189,13 +191,17 @@ template <int K> struct MuppetRule : DenseBase<K> {
             for (int e = 0; e < E; ++e) {
                 float g = upper ? gp[2 * e + 1] : gp[2 * e];
                 float h = upper ? gq[2 * e + 1] : gq[2 * e];
-                atomicAdd(sum_updated_val + this->lane + 64 * e, g + h);
+                grad_acc[e] += g + h;       // flushed once per worker in finish()
             }
         }
     }
     __device__ __forceinline__ void finish(const Params& a, uint32_t wid) const
     {
-        if (wid < a.num_workers && this->lane == 0) a.sum_norms[wid] = sum_norms_reg;
+        if (wid >= a.num_workers) return;
+        if (this->lane == 0) a.sum_norms[wid] = sum_norms_reg;
+#pragma unroll
+        for (int e = 0; e < E; ++e)
+            if (grad_acc[e] != 0.f) atomicAdd(a.sum_updated_val + this->lane + 64 * e, grad_acc[e]);
     }
 };
 
@@ -233,6 +239,7 @@ template <int K> struct AfpRule : DenseBase<K> {
     using typename Base::Info;
     static constexpr int E = Base::E;
     static constexpr int J = K / 32;
+    static constexpr int kAhead = 1, kRing = 4;
     struct Params { float* p; float* q; float lrate; float lambda; int afp_epoch; int init_threshold; };
     float lrate, lambda; int afp_epoch, init_threshold;
     AfpQ uq, iq, bq;
@@ -276,7 +283,7 @@ template <int K> struct AfpRule : DenseBase<K> {
         q.r = ufirst(q.r); q.n = ufirst(q.n); q.itv = ufirst(q.itv); q.mov_avg_range = ufirst(q.mov_avg_range);
         return q;
     }
-    __device__ __forceinline__ void update(Row& row, const Info& i, uint32_t)
+    template <int CLS> __device__ __forceinline__ void update(Row& row, const Info& i, uint32_t)
     {
         Mirror<K> p, q;
         p.build(row.p, upper); q.build(row.q, upper);

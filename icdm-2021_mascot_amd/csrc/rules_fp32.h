@@ -23,11 +23,13 @@ template <int K> struct DenseBase {
     using Row = DenseRow<K>;
     using Info = DenseInfo;
     using Prep = NoPrep;
+    static constexpr int kClasses = 1;
     float* P;
     float* Q;
     int lane;
 
     __device__ __forceinline__ Prep prepare(const Rating&, bool) const { return Prep(); }
+    __device__ __forceinline__ int classify(const Prep&, bool) const { return 0; }
     __device__ __forceinline__ Info info(const Rating& my, const Prep&, int j) const
     {
         Info i;
@@ -36,7 +38,7 @@ template <int K> struct DenseBase {
         i.v = bcast(my.v, j);
         return i;
     }
-    __device__ __forceinline__ void load(Row& row, const Info& i) const
+    template <int CLS> __device__ __forceinline__ void load(Row& row, const Info& i) const
     {
         const float* pp = P + (size_t)i.u * K + lane;
         const float* qq = Q + (size_t)i.v * K + lane;
@@ -82,6 +84,7 @@ template <int K> struct SgdRule : DenseBase<K> {
     using typename Base::Row;
     using typename Base::Info;
     static constexpr int E = Base::E;
+    static constexpr int kAhead = 3, kRing = 8;
     struct Params { float* p; float* q; float lrate; float lambda; };
     float lrate, lambda;
 
@@ -89,7 +92,7 @@ template <int K> struct SgdRule : DenseBase<K> {
     {
         this->P = a.p; this->Q = a.q; this->lane = lane_; lrate = a.lrate; lambda = a.lambda;
     }
-    __device__ __forceinline__ void update(Row& row, const Info& i, uint32_t) const
+    template <int CLS> __device__ __forceinline__ void update(Row& row, const Info& i, uint32_t) const
     {
         float m[E];
 #pragma unroll
@@ -113,6 +116,7 @@ template <int K> struct MptRule : DenseBase<K> {
     using typename Base::Row;
     using typename Base::Info;
     static constexpr int E = Base::E;
+    static constexpr int kAhead = 3, kRing = 8;
     struct Params { float* p; float* q; float lrate; uint16_t scaled_lambda_half; float scaling_factor; };
     float lrate, scaling_factor_rev;
     half_t lambda_h, scaling_factor_h;
@@ -124,7 +128,7 @@ template <int K> struct MptRule : DenseBase<K> {
         scaling_factor_h = (half_t)a.scaling_factor;
         lambda_h = from_bits<half_t>(a.scaled_lambda_half);
     }
-    __device__ __forceinline__ void update(Row& row, const Info& i, uint32_t) const
+    template <int CLS> __device__ __forceinline__ void update(Row& row, const Info& i, uint32_t) const
     {
         const half_t r_h = (half_t)i.r;
         half_t ph[E], qh[E], m[E];
