@@ -16,6 +16,10 @@ u8, u16, u32, u64, i32, f32, vp = C.c_uint8, C.c_uint16, C.c_uint32, C.c_uint64,
 SIGNATURES = {
     "mf_version": (i32, []),
     "mf_last_error": (C.c_char_p, []),
+    "mf_set_row_coherence": (i32, [i32]),
+    "mf_get_row_coherence": (i32, []),
+    "mf_set_epoch_splits": (i32, [u32]),
+    "mf_get_epoch_splits": (u32, []),
     "mf_mascot_norm_blocks": (u32, [u32]),
     "mf_update_count": (u32, [u32, u32, u32]),
     "mf_first_sample_rating_idx": (u32, [u32, u32, u32, u32, u32, f32]),
@@ -40,7 +44,32 @@ SIGNATURES = {
     "mf_sort_by_count": (i32, [vp, vp, u32, vp]),
     "mf_matrix_reconst_triplet": (i32, [vp, vp, vp, u32, vp]),
     "mf_shuffle_ratings": (i32, [vp, vp, u32, u64, vp]),
+    "mf_default_params": (None, [vp]),
+    "mf_init_model": (i32, [vp, vp, u32, u32, u32, u64, i32]),
+    "mf_train": (i32, [vp, vp, u32, u32, u32, vp, u32, vp, vp, vp]),
+    "mf_group_end_indices": (u32, [vp, u32, u32, vp]),
 }
+
+
+f64 = C.c_double
+
+
+class MfParams(C.Structure):
+    """mf_params of include/mascot_hip.h."""
+    _fields_ = [("lambda_", f32), ("learning_rate", f32), ("decay", f32), ("sample_ratio", f32), ("error_threshold", f32),
+                ("interval", u32), ("user_group_num", u32), ("item_group_num", u32), ("k", u32), ("num_workers", u32),
+                ("epoch", u32), ("thread_block_size", u32), ("version", u32), ("is_yahoo", u32), ("seed", u64),
+                ("verbose", u32), ("cached_rows", u32), ("epoch_splits", u32), ("reserved", u32)]
+
+
+class MfReport(C.Structure):
+    """mf_report of include/mascot_hip.h."""
+    _fields_ = [("rmse_per_epoch", vp), ("lr_per_epoch", vp), ("sgd_ms_per_epoch", vp),
+                ("user2sorted_idx", vp), ("item2sorted_idx", vp), ("user_group_end_idx", vp), ("item_group_end_idx", vp),
+                ("user_group_prec_info", vp), ("item_group_prec_info", vp),
+                ("user_group_num", u32), ("item_group_num", u32), ("test_reconst", vp),
+                ("preprocess_ms", f64), ("switching_ms", f64), ("error_ms", f64), ("sgd_ms", f64), ("total_ms", f64),
+                ("update_count", u32), ("muppet_final_bits", u32)]
 
 
 class MfError(RuntimeError):
@@ -80,10 +109,54 @@ class MascotHip:
     def __getattr__(self, name):
         if name.startswith("mf_"):
             fn = getattr(self.lib, name)
-            if SIGNATURES[name][0] is i32 and name != "mf_version":
+            if SIGNATURES[name][0] is i32 and name not in ("mf_version", "mf_get_row_coherence"):
                 return lambda *a: self.call(name, *a)
             return fn
         raise AttributeError(name)
+
+    # ---- host-level helpers over numpy arrays ----------------------------------------------
+    def default_params(self, **kw):
+        prm = MfParams()
+        self.lib.mf_default_params(C.byref(prm))
+        for key, val in kw.items():
+            setattr(prm, "lambda_" if key == "lambda_" or key == "lam" else key, val)
+        return prm
+
+    def init_model(self, n_users, n_items, k, seed, half_rounded=False):
+        p = np.empty((n_users, k), np.float32)
+        q = np.empty((n_items, k), np.float32)
+        self.call("mf_init_model", p.ctypes.data, q.ctypes.data, n_users, n_items, k, seed, int(half_rounded))
+        return p, q
+
+    def train(self, prm, R, n_users, n_items, test, p, q):
+        """Runs mf_train; returns a dict with the per-epoch figures and (MASCOT) the sorted-space tables."""
+        E = prm.epoch
+        out = dict(rmse=np.zeros(E, np.float64), lr=np.zeros(E, np.float32), sgd_ms=np.zeros(E, np.float32),
+                   user2sorted=np.zeros(n_users, np.uint32), item2sorted=np.zeros(n_items, np.uint32),
+                   user_end=np.zeros(max(prm.user_group_num, 1), np.uint32), item_end=np.zeros(max(prm.item_group_num, 1), np.uint32),
+                   user_prec=np.zeros(max(prm.user_group_num, 1), np.uint8), item_prec=np.zeros(max(prm.item_group_num, 1), np.uint8),
+                   test_reconst=np.zeros(test.size, NODE))
+        rep = MfReport()
+        rep.rmse_per_epoch = out["rmse"].ctypes.data
+        rep.lr_per_epoch = out["lr"].ctypes.data
+        rep.sgd_ms_per_epoch = out["sgd_ms"].ctypes.data
+        rep.user2sorted_idx = out["user2sorted"].ctypes.data
+        rep.item2sorted_idx = out["item2sorted"].ctypes.data
+        rep.user_group_end_idx = out["user_end"].ctypes.data
+        rep.item_group_end_idx = out["item_end"].ctypes.data
+        rep.user_group_prec_info = out["user_prec"].ctypes.data
+        rep.item_group_prec_info = out["item_prec"].ctypes.data
+        rep.test_reconst = out["test_reconst"].ctypes.data
+        R = np.ascontiguousarray(R)
+        test = np.ascontiguousarray(test)
+        self.call("mf_train", C.byref(prm), R.ctypes.data, R.size, n_users, n_items, test.ctypes.data, test.size,
+                  p.ctypes.data, q.ctypes.data, C.byref(rep))
+        out["report"] = rep
+        out["user_end"] = out["user_end"][:rep.user_group_num]
+        out["item_end"] = out["item_end"][:rep.item_group_num]
+        out["user_prec"] = out["user_prec"][:rep.user_group_num]
+        out["item_prec"] = out["item_prec"][:rep.item_group_num]
+        return out
 
 
 _handle = None

@@ -38,12 +38,45 @@ static Schedule make_schedule(const mf_node* R, uint32_t nnz, uint32_t num_worke
 }
 static inline uint32_t grid_for(uint32_t num_workers) { return (num_workers + kWavesPerBlock - 1) / kWavesPerBlock; }
 
+// 0: ordinary cached row accesses, 1: agent-scope coherent row accesses (see row_load in mf_device.h)
+static int g_row_coherence = 1;
+// number of consecutive kernel launches one call is cut into (each worker's windows are split evenly);
+// a kernel boundary writes back and invalidates the per-XCD L2s, which is how cached row copies of
+// different XCDs are reconciled during an epoch
+static uint32_t g_epoch_splits = 1;
+
 template <class Rule>
-static int launch(const char* who, const Schedule& s, const typename Rule::Params& prm, size_t lds, void* stream)
+static int launch(const char* who, const Schedule& s0, const typename Rule::Params& prm0, size_t lds, void* stream)
 {
-    if (s.update_count == 0 || s.update_vector_size == 0) return MF_OK;
-    hipLaunchKernelGGL((hogwild_kernel<Rule>), dim3(grid_for(s.num_workers)), dim3(kBlock), lds, as_stream(stream), s, prm);
-    return launch_status(who);
+    if (s0.update_count == 0 || s0.update_vector_size == 0) return MF_OK;
+    uint32_t splits = Rule::kSplittable ? g_epoch_splits : 1;
+    if (splits > s0.update_count) splits = s0.update_count;
+    const uint32_t total = s0.range_end;
+    for (uint32_t i = 0; i < splits; ++i) {
+        Schedule s = s0;
+        typename Rule::Params prm = prm0;
+        // cut on window boundaries
+        s.range_begin = (uint32_t)((uint64_t)s0.update_count * i / splits) * s0.update_vector_size;
+        s.range_end = i + 1 == splits ? total : (uint32_t)((uint64_t)s0.update_count * (i + 1) / splits) * s0.update_vector_size;
+        prm.accumulate = i != 0;
+        hipLaunchKernelGGL((hogwild_kernel<Rule>), dim3(grid_for(s.num_workers)), dim3(kBlock), lds, as_stream(stream), s, prm);
+        if (int rc = launch_status(who)) return rc;
+    }
+    return MF_OK;
+}
+
+// Instantiates Rule<K, COH> for the four (k, coherence) combinations; P is the parameter pack type,
+// identical across instantiations apart from the template arguments.
+template <template <int, bool> class Rule, class MakeParams>
+static int launch_k_coh(const char* who, int k, const Schedule& s, MakeParams make, size_t lds, void* stream)
+{
+    const bool coh = g_row_coherence != 0;
+    if (k == 128) {
+        if (coh) { auto a = make(typename Rule<128, true>::Params{}); return launch<Rule<128, true>>(who, s, a, lds, stream); }
+        auto a = make(typename Rule<128, false>::Params{}); return launch<Rule<128, false>>(who, s, a, lds, stream);
+    }
+    if (coh) { auto a = make(typename Rule<64, true>::Params{}); return launch<Rule<64, true>>(who, s, a, lds, stream); }
+    auto a = make(typename Rule<64, false>::Params{}); return launch<Rule<64, false>>(who, s, a, lds, stream);
 }
 
 }  // namespace mf
@@ -53,6 +86,20 @@ using namespace mf;
 extern "C" {
 
 int mf_version(void) { return 1; }
+int mf_set_row_coherence(int coherent)
+{
+    if (coherent != 0 && coherent != 1) return invalid("mf_set_row_coherence: 0 (cached) or 1 (device-coherent)");
+    g_row_coherence = coherent;
+    return MF_OK;
+}
+int mf_get_row_coherence(void) { return g_row_coherence; }
+int mf_set_epoch_splits(uint32_t splits)
+{
+    if (splits == 0 || splits > 65536) return invalid("mf_set_epoch_splits: between 1 and 65536");
+    g_epoch_splits = splits;
+    return MF_OK;
+}
+uint32_t mf_get_epoch_splits(void) { return g_epoch_splits; }
 const char* mf_last_error(void) { return g_error; }
 uint32_t mf_mascot_norm_blocks(uint32_t num_workers) { return grid_for(num_workers); }
 
@@ -90,9 +137,7 @@ int mf_single_sgd_hogwild(const mf_node* R, uint32_t nnz, float* p, float* q, in
     if (int rc = check_schedule("mf_single_sgd_hogwild", R, nnz, k, num_workers, update_count, update_vector_size)) return rc;
     if (!p || !q) return invalid("mf_single_sgd_hogwild: null model pointer");
     Schedule s = make_schedule(R, nnz, num_workers, update_count, update_vector_size, seed, epoch, window_start);
-    if (k == 128) { SgdRule<128>::Params a{p, q, lrate, lambda}; return launch<SgdRule<128>>("mf_single_sgd_hogwild", s, a, 0, stream); }
-    SgdRule<64>::Params a{p, q, lrate, lambda};
-    return launch<SgdRule<64>>("mf_single_sgd_hogwild", s, a, 0, stream);
+    return launch_k_coh<SgdRule>("mf_single_sgd_hogwild", k, s, [&](auto a) { a.p = p; a.q = q; a.lrate = lrate; a.lambda = lambda; return a; }, 0, stream);
 }
 
 int mf_mpt_sgd_hogwild(const mf_node* R, uint32_t nnz, float* p, float* q, int k,
@@ -104,9 +149,8 @@ int mf_mpt_sgd_hogwild(const mf_node* R, uint32_t nnz, float* p, float* q, int k
     if (!p || !q) return invalid("mf_mpt_sgd_hogwild: null model pointer");
     if (!(scaling_factor > 0)) return invalid("mf_mpt_sgd_hogwild: scaling_factor must be positive");
     Schedule s = make_schedule(R, nnz, num_workers, update_count, update_vector_size, seed, epoch, window_start);
-    if (k == 128) { MptRule<128>::Params a{p, q, lrate, scaled_lambda_half, scaling_factor}; return launch<MptRule<128>>("mf_mpt_sgd_hogwild", s, a, 0, stream); }
-    MptRule<64>::Params a{p, q, lrate, scaled_lambda_half, scaling_factor};
-    return launch<MptRule<64>>("mf_mpt_sgd_hogwild", s, a, 0, stream);
+    return launch_k_coh<MptRule>("mf_mpt_sgd_hogwild", k, s, [&](auto a) {
+        a.p = p; a.q = q; a.lrate = lrate; a.scaled_lambda_half = scaled_lambda_half; a.scaling_factor = scaling_factor; return a; }, 0, stream);
 }
 
 static bool muppet_precision_ok(uint8_t b) { return b == 8 || b == 12 || b == 14 || b == 16 || b == 32; }
@@ -125,12 +169,10 @@ int mf_muppet_sgd_hogwild(const mf_node* R, uint32_t nnz, float* p, float* q, in
     if ((forward_prop_precision == 32) != (backward_prop_precision == 32))
         return invalid("mf_muppet_sgd_hogwild: forward and backward precision must both be 32 or both below (the backward scale reuses forward statistics)");
     Schedule s = make_schedule(R, nnz, num_workers, update_count, update_vector_size, seed, epoch, window_start);
-    if (k == 128) {
-        MuppetRule<128>::Params a{p, q, lrate, lambda, first_sample_rating_idx, sum_updated_val, sum_norms, num_workers, forward_prop_precision, backward_prop_precision};
-        return launch<MuppetRule<128>>("mf_muppet_sgd_hogwild", s, a, 0, stream);
-    }
-    MuppetRule<64>::Params a{p, q, lrate, lambda, first_sample_rating_idx, sum_updated_val, sum_norms, num_workers, forward_prop_precision, backward_prop_precision};
-    return launch<MuppetRule<64>>("mf_muppet_sgd_hogwild", s, a, 0, stream);
+    return launch_k_coh<MuppetRule>("mf_muppet_sgd_hogwild", k, s, [&](auto a) {
+        a.p = p; a.q = q; a.lrate = lrate; a.lambda = lambda; a.first_sample = first_sample_rating_idx;
+        a.sum_updated_val = sum_updated_val; a.sum_norms = sum_norms; a.num_workers = num_workers;
+        a.fwd = forward_prop_precision; a.bwd = backward_prop_precision; return a; }, 0, stream);
 }
 
 int mf_afp_sgd_hogwild(const mf_node* R, uint32_t nnz, float* p, float* q, int k,
@@ -143,9 +185,8 @@ int mf_afp_sgd_hogwild(const mf_node* R, uint32_t nnz, float* p, float* q, int k
     Schedule s = make_schedule(R, nnz, num_workers, update_count, update_vector_size, seed, epoch, window_start);
     // afp_sgd_kernel.h:145: int initialization_threshold = (float)(update_count*update_vector_size)/10.0f
     const int init_threshold = (int)((float)(update_count * update_vector_size) / 10.0f);
-    if (k == 128) { AfpRule<128>::Params a{p, q, lrate, lambda, afp_epoch, init_threshold}; return launch<AfpRule<128>>("mf_afp_sgd_hogwild", s, a, 0, stream); }
-    AfpRule<64>::Params a{p, q, lrate, lambda, afp_epoch, init_threshold};
-    return launch<AfpRule<64>>("mf_afp_sgd_hogwild", s, a, 0, stream);
+    return launch_k_coh<AfpRule>("mf_afp_sgd_hogwild", k, s, [&](auto a) {
+        a.p = p; a.q = q; a.lrate = lrate; a.lambda = lambda; a.afp_epoch = afp_epoch; a.init_threshold = init_threshold; return a; }, 0, stream);
 }
 
 int mf_mascot_sgd_hogwild(const mf_node* R, uint32_t nnz, void* const* p, void* const* q, int k,
@@ -164,19 +205,15 @@ int mf_mascot_sgd_hogwild(const mf_node* R, uint32_t nnz, void* const* p, void* 
     if (!grad_sum_norm_p || !grad_sum_norm_q || !norm_sum_p || !norm_sum_q) return invalid("%s: null statistics buffer", who);
     if (user_group_num == 0 || item_group_num == 0) return invalid("%s: at least one group per side is required", who);
     if (user_group_num > 16383 || item_group_num > 16383) return invalid("%s: at most 16383 groups per side", who);
-    const size_t lds = MascotRule<128>::lds_bytes(user_group_num, item_group_num);
+    const size_t lds = MascotRule<128, true>::lds_bytes(user_group_num, item_group_num);
     if (lds > 64 * 1024) return invalid("%s: group tables need %zu bytes of LDS (limit 65536)", who, lds);
     Schedule s = make_schedule(R, nnz, num_workers, update_count, update_vector_size, seed, epoch, window_start);
-    if (k == 128) {
-        MascotRule<128>::Params a{p, q, user_group_end_idx, item_group_end_idx, user_group_prec_info, item_group_prec_info,
-                                  grad_sum_norm_p, grad_sum_norm_q, norm_sum_p, norm_sum_q,
-                                  first_sample_rating_idx, user_group_num, item_group_num, lrate, lambda};
-        return launch<MascotRule<128>>(who, s, a, lds, stream);
-    }
-    MascotRule<64>::Params a{p, q, user_group_end_idx, item_group_end_idx, user_group_prec_info, item_group_prec_info,
-                             grad_sum_norm_p, grad_sum_norm_q, norm_sum_p, norm_sum_q,
-                             first_sample_rating_idx, user_group_num, item_group_num, lrate, lambda};
-    return launch<MascotRule<64>>(who, s, a, lds, stream);
+    return launch_k_coh<MascotRule>(who, k, s, [&](auto a) {
+        a.p = p; a.q = q; a.user_end = user_group_end_idx; a.item_end = item_group_end_idx;
+        a.user_prec = user_group_prec_info; a.item_prec = item_group_prec_info;
+        a.grad_sum_p = grad_sum_norm_p; a.grad_sum_q = grad_sum_norm_q; a.norm_sum_p = norm_sum_p; a.norm_sum_q = norm_sum_q;
+        a.first_sample = first_sample_rating_idx; a.user_groups = user_group_num; a.item_groups = item_group_num;
+        a.lrate = lrate; a.lambda = lambda; return a; }, lds, stream);
 }
 
 }  // extern "C"

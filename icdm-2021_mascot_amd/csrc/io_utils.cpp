@@ -1,0 +1,208 @@
+#include "io_utils.h"
+#include <algorithm>
+#include <cerrno>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <fstream>
+#include <iostream>
+#include <sstream>
+
+namespace {
+
+std::vector<std::string> split(const std::string& s, char delim)
+{
+    std::vector<std::string> out;
+    std::stringstream ss(s);
+    std::string item;
+    while (std::getline(ss, item, delim)) out.push_back(item);
+    return out;
+}
+// column order from substrings of the path (io_utils.h:40-47)
+void column_order(const std::string& path, int& user_idx, int& item_idx)
+{
+    if (path.find("netflix") != std::string::npos || path.find("25M") != std::string::npos) { user_idx = 1; item_idx = 0; }
+    else { user_idx = 0; item_idx = 1; }
+}
+uint32_t dense_id(std::unordered_map<uint32_t, uint32_t>& map, std::vector<uint32_t>& orig, uint32_t& count, uint32_t id)
+{
+    auto it = map.find(id);
+    if (it != map.end()) return it->second;
+    map.emplace(id, count);
+    orig.push_back(id);
+    return count++;
+}
+float parse_rating(std::string s)
+{
+    s.erase(s.find_last_not_of(" \n\r\t") + 1);
+    return (float)std::atof(s.c_str());
+}
+std::string parent_dir(const std::string& path)
+{
+    const size_t pos = path.find_last_of('/');
+    return pos == std::string::npos ? std::string() : path.substr(0, pos);
+}
+std::string file_name(const std::string& path)
+{
+    const size_t pos = path.find_last_of('/');
+    return pos == std::string::npos ? path : path.substr(pos + 1);
+}
+
+}  // namespace
+
+bool read_training_dataset(Dataset& d, const std::string& path)
+{
+    std::ifstream file(path);
+    if (!file) return false;
+    int user_idx, item_idx;
+    column_order(path, user_idx, item_idx);
+    std::string line;
+    if (path.find("Yahoo") != std::string::npos) {           // io_utils.h:49-79: "user|count" then count lines "item\trating"
+        while (std::getline(file, line)) {
+            std::vector<std::string> head = split(line, '|');
+            if (head.size() < 2) continue;
+            const uint32_t user = (uint32_t)std::stoi(head[0]);
+            const uint32_t cnt = (uint32_t)std::stoi(head[1]);
+            const uint32_t u = dense_id(d.user_map, d.user_orig, d.max_user, user);
+            for (uint32_t i = 0; i < cnt; ++i) {
+                if (!std::getline(file, line)) break;
+                std::vector<std::string> tok = split(line, '\t');
+                if (tok.size() < 2) continue;
+                const uint32_t it = dense_id(d.item_map, d.item_orig, d.max_item, (uint32_t)std::stoi(tok[0]));
+                const float rating = (float)std::atof(tok[1].c_str());
+                d.R.push_back({(rating / 25.f) + 1.0f, u, it});
+            }
+        }
+    } else {
+        while (std::getline(file, line)) {
+            std::vector<std::string> tok = split(line, '\t');
+            if (tok.size() != 3) continue;
+            const uint32_t user = (uint32_t)std::stoi(tok[user_idx]);
+            const uint32_t item = (uint32_t)std::stoi(tok[item_idx]);
+            const float rating = parse_rating(tok[2]);
+            const uint32_t u = dense_id(d.user_map, d.user_orig, d.max_user, user);
+            const uint32_t it = dense_id(d.item_map, d.item_orig, d.max_item, item);
+            d.R.push_back({rating, u, it});
+        }
+    }
+    return true;
+}
+
+bool read_test_dataset(Dataset& d, const std::string& path)
+{
+    std::vector<uint32_t> remove_user, remove_item;
+    uint32_t missing = 0;
+    std::ifstream file(path);
+    int user_idx, item_idx;
+    column_order(path, user_idx, item_idx);
+    // test_R[user][item] = rating: later duplicates overwrite earlier ones (io_utils.h:186)
+    std::vector<std::map<uint32_t, float>> test_R(d.max_user);
+    std::string line;
+    if (file) {
+        if (path.find("Yahoo") != std::string::npos) {
+            while (std::getline(file, line)) {
+                std::vector<std::string> head = split(line, '|');
+                if (head.size() < 2) continue;
+                const uint32_t cnt = (uint32_t)std::stoi(head[1]);
+                auto itu = d.user_map.find((uint32_t)std::stoi(head[0]));
+                if (itu == d.user_map.end()) {
+                    // the reference counts the block as missing and moves on without consuming its lines
+                    // (io_utils.h:153-156); consume them here so the following blocks parse
+                    missing += cnt;
+                    for (uint32_t i = 0; i < cnt; ++i) std::getline(file, line);
+                    continue;
+                }
+                for (uint32_t i = 0; i < cnt; ++i) {
+                    if (!std::getline(file, line)) break;
+                    std::vector<std::string> tok = split(line, '\t');
+                    if (tok.size() < 2) continue;
+                    auto iti = d.item_map.find((uint32_t)std::stoi(tok[0]));
+                    if (iti == d.item_map.end()) { missing += 1; continue; }
+                    test_R[itu->second][iti->second] = ((float)std::atof(tok[1].c_str()) / 25.f) + 1.0f;
+                    d.test_lines_kept++;
+                }
+            }
+        } else {
+            while (std::getline(file, line)) {
+                std::vector<std::string> tok = split(line, '\t');
+                if (tok.size() != 3) continue;
+                const uint32_t user = (uint32_t)std::stoi(tok[user_idx]);
+                const uint32_t item = (uint32_t)std::stoi(tok[item_idx]);
+                const float rating = parse_rating(tok[2]);
+                auto itu = d.user_map.find(user);
+                auto iti = d.item_map.find(item);
+                if (itu != d.user_map.end() && iti != d.item_map.end()) { test_R[itu->second][iti->second] = rating; d.test_lines_kept++; }
+                else if (itu == d.user_map.end()) { missing++; remove_user.push_back(user); }
+                else { missing++; remove_item.push_back(item); }
+            }
+        }
+    }
+    std::cout << "Missing the number of ratings : " << missing << std::endl;
+    // test_set_preprocess, preprocess_utils.h:38-52: users ascending (dense id), items ascending within a user
+    for (uint32_t u = 0; u < d.max_user; ++u)
+        for (const auto& kv : test_R[u]) d.test.push_back({kv.second, u, kv.first});
+
+    const std::string dir = parent_dir(path);
+    for (int which = 0; which < 2; ++which) {
+        const std::string out = dir + (which ? "/remove_item.txt" : "/remove_user.txt");
+        std::ofstream f(out);
+        if (f.fail()) { std::cout << "fail to write file named " << out << std::endl; return true; }
+        for (uint32_t v : (which ? remove_item : remove_user)) f << v << std::endl;
+    }
+    return true;
+}
+
+bool save_trained_model(const Dataset& d, const float* p, const float* q, uint32_t k, const std::string& outfile)
+{
+    std::cout << "Save trained model..." << std::endl;
+    const std::string outpath = outfile + ".txt";
+    std::ofstream f(outpath);
+    if (f.fail()) { std::cout << "fail to write file named " << outpath << std::endl; std::cerr << "Error: " << std::strerror(errno); return false; }
+    auto sorted_by_orig = [](const std::unordered_map<uint32_t, uint32_t>& m) {
+        std::vector<std::pair<uint32_t, uint32_t>> v(m.begin(), m.end());
+        std::sort(v.begin(), v.end());
+        return v;
+    };
+    const auto users = sorted_by_orig(d.user_map), items = sorted_by_orig(d.item_map);
+    f << users.back().first + 1 << " " << items.back().first + 1 << " " << k << std::endl;
+    auto dump = [&](const std::vector<std::pair<uint32_t, uint32_t>>& ids, const float* m) {
+        int prev = 0;
+        for (const auto& kv : ids) {
+            const int orig = (int)kv.first;
+            for (int c = prev; c <= orig - 1; ++c) for (uint32_t j = 0; j < k; ++j) f << 0 << " ";
+            for (uint32_t j = 0; j < k; ++j) f << m[(size_t)kv.second * k + j] << " ";
+            prev = orig + 1;
+        }
+    };
+    dump(users, p);
+    f << std::endl;
+    dump(items, q);
+    return true;
+}
+
+bool save_trained_model_reconst(uint32_t n_users, uint32_t n_items, const float* p, const float* q, uint32_t k, const std::string& outfile)
+{
+    std::cout << "Save trained reconst model..." << std::endl;
+    const std::string outpath = outfile + "_reconst.txt";
+    std::ofstream f(outpath);
+    if (f.fail()) { std::cout << "fail to write file named " << outpath << std::endl; std::cerr << "Error: " << std::strerror(errno); return false; }
+    f << n_users << " " << n_items << " " << k << std::endl;
+    for (size_t i = 0; i < (size_t)n_users * k; ++i) f << p[i] << " ";
+    f << std::endl;
+    for (size_t i = 0; i < (size_t)n_items * k; ++i) f << q[i] << " ";
+    return true;
+}
+
+bool save_reconst_testset(const std::vector<mf_node>& test, const std::string& testfile)
+{
+    std::cout << "Save reconst mat.." << std::endl;
+    const std::string out = parent_dir(testfile) + "/reconst_" + file_name(testfile);
+    std::ofstream f(out);
+    if (f.fail()) { std::cout << "fail to write file named " << out << std::endl; return false; }
+    const bool user_first = !(out.find("netflix") != std::string::npos || out.find("25M") != std::string::npos);
+    for (const mf_node& t : test) {
+        if (user_first) f << t.u << "\t" << t.i << "\t" << t.r << std::endl;
+        else f << t.i << "\t" << t.u << "\t" << t.r << std::endl;
+    }
+    return true;
+}

@@ -1,0 +1,29 @@
+// Host I/O of the quantized_mf command line: rating readers and model writers with the file layouts
+// of the reference's io_utils.h.
+#pragma once
+#include <cstdint>
+#include <map>
+#include <string>
+#include <unordered_map>
+#include <vector>
+#include "../../include/mascot_hip.h"
+
+struct Dataset {
+    std::vector<mf_node> R;                       // training ratings, dense first-seen ids
+    std::vector<mf_node> test;                    // test ratings ordered by (user, item), duplicates folded
+    std::unordered_map<uint32_t, uint32_t> user_map, item_map;   // original id -> dense id
+    std::vector<uint32_t> user_orig, item_orig;   // dense id -> original id
+    uint32_t max_user = 0, max_item = 0;          // number of distinct users / items
+    uint32_t test_lines_kept = 0;                 // the reference's test_n (counts duplicates, io_utils.h:187)
+};
+
+// read_training_dataset, io_utils.h:30-120
+bool read_training_dataset(Dataset& d, const std::string& path);
+// read_test_dataset, io_utils.h:122-240 (also writes remove_user.txt / remove_item.txt next to the file)
+bool read_test_dataset(Dataset& d, const std::string& path);
+// save_trained_model, io_utils.h:242-303: <out>.txt, rows by original id, zero rows for absent ids
+bool save_trained_model(const Dataset& d, const float* p, const float* q, uint32_t k, const std::string& outfile);
+// save_trained_model_reconst, io_utils.h:305-332: <out>_reconst.txt, rows in the order given
+bool save_trained_model_reconst(uint32_t n_users, uint32_t n_items, const float* p, const float* q, uint32_t k, const std::string& outfile);
+// save_reconst_testset, io_utils.h:374-405: reconst_<testfile> next to the test file
+bool save_reconst_testset(const std::vector<mf_node>& test, const std::string& testfile);

@@ -1,0 +1,121 @@
+// quantized_mf: the reference's command line (main.cu:15-175) over libmascot_hip.
+// Same flags, same stdout lines, same model files.  Additions: `-seed <n>` (the reference seeds from
+// time(0) and clock(), so two of its runs never agree; here the default seed is fixed), `-cached <0|1>`
+// and `-split <n>` (row access policy and kernel launches per epoch, see include/mascot_hip.h).
+#include <sys/stat.h>
+#include <cstdlib>
+#include <iostream>
+#include <string>
+#include <vector>
+#include "io_utils.h"
+
+static bool exists(const std::string& name) { struct stat b; return stat(name.c_str(), &b) == 0; }
+
+int main(int argc, const char* argv[])
+{
+    std::string infile, outfile, testfile = "None";
+    mf_params prm;
+    mf_default_params(&prm);
+    unsigned reconst_save = 0;
+    const char* usage = " [-t <threads> -p <predictions/user> -o <output-tsv>] <input-tsv>";
+    if (argc < 2) { std::cout << argv[0] << usage << std::endl; return 0; }
+    if (argc == 2) infile = argv[1];
+    else {
+        for (int i = 0; i < argc; ++i) {
+            const std::string a = argv[i];
+            const bool has = i < argc - 1;
+            if (a == "-i" && has) infile = argv[i + 1];
+            if (a == "-o" && has) outfile = argv[i + 1];
+            if (a == "-y" && has) testfile = argv[i + 1];
+            if (a == "-l" && has) prm.epoch = std::atoi(argv[i + 1]);
+            if (a == "-k" && has) prm.k = std::atoi(argv[i + 1]);
+            if (a == "-b" && has) prm.lambda = std::atof(argv[i + 1]);
+            if (a == "-a" && has) prm.learning_rate = std::atof(argv[i + 1]);
+            if (a == "-wg" && has) prm.num_workers = std::atoi(argv[i + 1]);
+            if (a == "-d" && has) prm.decay = std::atof(argv[i + 1]);
+            if (a == "-bl" && has) prm.thread_block_size = std::atoi(argv[i + 1]);
+            if (a == "-v" && has) prm.version = std::atoi(argv[i + 1]);
+            if (a == "-r" && has) prm.sample_ratio = std::atof(argv[i + 1]);
+            if (a == "-ug" && has) prm.user_group_num = std::atoi(argv[i + 1]);
+            if (a == "-ig" && has) prm.item_group_num = std::atoi(argv[i + 1]);
+            if (a == "-e" && has) prm.error_threshold = std::atof(argv[i + 1]);
+            if (a == "-s" && has) prm.sample_ratio = std::atof(argv[i + 1]);
+            if (a == "-it" && has) prm.interval = std::atoi(argv[i + 1]);
+            if (a == "-rc" && has) reconst_save = std::atoi(argv[i + 1]);
+            if (a == "-seed" && has) prm.seed = std::strtoull(argv[i + 1], nullptr, 10);
+            if (a == "-cached" && has) prm.cached_rows = std::atoi(argv[i + 1]);
+            if (a == "-split" && has) prm.epoch_splits = std::atoi(argv[i + 1]);
+            if (a == "-h") { std::cout << argv[0] << usage << std::endl; return 0; }
+        }
+    }
+    if (!exists(infile)) { std::cout << infile << " doesn't exist!" << std::endl; return 0; }
+
+    std::cout << std::endl;
+    std::cout << "Input file                  : " << infile << std::endl;
+    std::cout << "Test file                   : " << testfile << std::endl;
+    std::cout << "Output file                 : " << outfile << std::endl;
+    std::cout << "Latent features             : " << prm.k << std::endl;
+    std::cout << "Learning rate               : " << prm.learning_rate << std::endl;
+    std::cout << "Decay                       : " << prm.decay << std::endl;
+    std::cout << "Lambda                      : " << prm.lambda << std::endl;
+    std::cout << "Iteration                   : " << prm.epoch << std::endl;
+    std::cout << "Num of workers              : " << prm.num_workers << std::endl;
+    std::cout << "Thread block size           : " << prm.thread_block_size << std::endl;
+    std::cout << "Sample ratio                : " << prm.sample_ratio << std::endl;
+    std::cout << "Error threshold             : " << prm.error_threshold << std::endl;
+    std::cout << "Interval                    : " << prm.interval << std::endl;
+    std::cout << "Seed                        : " << prm.seed << std::endl;
+
+    Dataset d;
+    read_training_dataset(d, infile);
+    read_test_dataset(d, testfile);
+    std::cout << "The number of nonzeros      : " << d.R.size() << std::endl;
+    std::cout << "The number of users         : " << d.max_user << std::endl;
+    std::cout << "The number of items         : " << d.max_item << std::endl;
+    std::cout << "The number of test nonzeros : " << d.test.size() << std::endl;
+
+    prm.is_yahoo = infile.find("Yahoo") != std::string::npos;
+    prm.verbose = 1;
+    if (prm.version == 0) prm.version = 5;          // "-v 0" is accepted as plain fp32 SGD
+    const size_t pn = (size_t)d.max_user * prm.k, qn = (size_t)d.max_item * prm.k;
+    std::vector<float> p(pn), q(qn);
+    // init_model_half for the variants that start from binary16-representable values (main.cu:152-153)
+    const int half_init = prm.version == 4 || prm.version == 7 || prm.version == 8;
+    if (int rc = mf_init_model(p.data(), q.data(), d.max_user, d.max_item, prm.k, prm.seed, half_init)) {
+        std::cerr << "quantized_mf: " << mf_last_error() << std::endl;
+        return rc > 0 ? rc : 1;
+    }
+    mf_report rep = {};
+    std::vector<float> ms(prm.epoch);
+    std::vector<mf_node> test_reconst(d.test.size());
+    rep.sgd_ms_per_epoch = ms.data();
+    rep.test_reconst = test_reconst.data();
+    if (int rc = mf_train(&prm, d.R.data(), (uint32_t)d.R.size(), d.max_user, d.max_item, d.test.data(), (uint32_t)d.test.size(),
+                          p.data(), q.data(), &rep)) {
+        std::cerr << "quantized_mf: " << mf_last_error() << std::endl;
+        return rc > 0 ? rc : 1;
+    }
+    // timing summary in the reference's units (micro seconds unless stated), mf_methods.cu:401-418
+    if (prm.version == 1) {
+        std::cout << "\n<Preprocessing time (micro sec)>" << std::endl;
+        std::cout << "Total preprocessing time         : " << rep.preprocess_ms * 1000 << std::endl;
+        std::cout << "\n<User & item parameter copy exec time (micro sec)>" << std::endl;
+        std::cout << "Precision switching              : " << rep.switching_ms * 1000 / prm.epoch << std::endl;
+        std::cout << "Total precision switching time   : " << rep.switching_ms * 1000 << std::endl;
+        std::cout << "\n<User & item group error comp exec time (micro sec)>" << std::endl;
+        std::cout << "Error computation time           : " << rep.error_ms * 1000 / prm.epoch << std::endl;
+        std::cout << "Total error computation time     : " << rep.error_ms * 1000 << std::endl;
+        std::cout << "\n<User & item parameter update exec time (micro sec)>" << std::endl;
+    }
+    std::cout << "Parameters update per epoch      : " << rep.sgd_ms * 1000 / prm.epoch << std::endl;
+    std::cout << "Total parameters update          : " << rep.sgd_ms * 1000 << std::endl;
+    std::cout << "Total MF time(ms)                : " << (rep.preprocess_ms + rep.switching_ms + rep.error_ms + rep.sgd_ms) << std::endl;
+    std::cout << "Ratings per second (update kernel): " << (double)d.R.size() * prm.epoch / (rep.sgd_ms / 1000.0) << std::endl;
+
+    if (!outfile.empty()) {
+        if (prm.version == 1) save_trained_model_reconst(d.max_user, d.max_item, p.data(), q.data(), prm.k, outfile);
+        else save_trained_model(d, p.data(), q.data(), prm.k, outfile);
+    }
+    if (prm.version == 1 && reconst_save == 1) save_reconst_testset(test_reconst, testfile);
+    return 0;
+}

@@ -90,6 +90,29 @@ __device__ __forceinline__ uint64_t bcast(uint64_t v, int lane)
     return (uint64_t)bcast((uint32_t)v, lane) | ((uint64_t)bcast((uint32_t)(v >> 32), lane) << 32);
 }
 
+// ---- device-coherent row accesses -----------------------------------------------------------
+// MI355X has one L2 per XCD and the L2s do not snoop each other for ordinary loads and stores: a row
+// cached in one XCD's L2 would not see the updates other XCDs make to it during the same kernel, and
+// each XCD would train its own private copy of every hot row.  Hogwild needs the opposite (the latest
+// value any worker wrote), so P and Q rows are read and written with agent-scope relaxed atomics: plain
+// global_load/global_store instructions with the sc1 cache policy, no fences and no read-modify-write.
+//
+// The price: every access to a row goes to the memory side, and all accesses to one row serialise
+// there.  With a row that takes a large share of all ratings (Zipf-like synthetic data) that single row
+// bounds the epoch.  COH = false keeps ordinary cached accesses instead: each XCD then works on its own
+// L2-resident copy of a hot row between evictions (a row that is not re-used while cached behaves the
+// same either way).  The host picks per run (mf_set_row_coherence).
+template <bool COH, class T> __device__ __forceinline__ T row_load(const T* p)
+{
+    if constexpr (COH) return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    else return *p;
+}
+template <bool COH, class T> __device__ __forceinline__ void row_store(T* p, T v)
+{
+    if constexpr (COH) __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    else *p = v;
+}
+
 // ---- counter-based generator -----------------------------------------------------------
 __host__ __device__ __forceinline__ uint64_t mix64(uint64_t z)
 {

@@ -19,7 +19,7 @@
 
 namespace mf {
 
-template <int K> struct MascotRule {
+template <int K, bool COH> struct MascotRule {
     static constexpr int E = K / 64;                        // elements per lane
     static constexpr int kAhead = 3, kRing = 8;
     // chunk classes: 0 = any mix of precisions (flag-driven), 1 = every rating of the chunk touches two
@@ -33,8 +33,9 @@ template <int K> struct MascotRule {
         const uint8_t* user_prec; const uint8_t* item_prec;
         float* grad_sum_p; float* grad_sum_q; float* norm_sum_p; float* norm_sum_q;
         uint32_t first_sample; uint32_t user_groups; uint32_t item_groups;
-        float lrate; float lambda;
+        float lrate; float lambda; bool accumulate;
     };
+    static constexpr bool kSplittable = true;
     // raw row registers: binary16 rows use r[0] only
     struct Row { uint32_t p[E], q[E]; };
     struct Prep { uint64_t pptr, qptr; uint32_t flags; };
@@ -123,24 +124,24 @@ template <int K> struct MascotRule {
     {
         if (fp32) {
             if constexpr (E == 2) {
-                const uint2 v = *reinterpret_cast<const uint2*>(ptr + (uint64_t)lane * 8);
-                r[0] = v.x; r[1] = v.y;
+                const uint64_t v = row_load<COH>(reinterpret_cast<const uint64_t*>(ptr + (uint64_t)lane * 8));
+                r[0] = (uint32_t)v; r[1] = (uint32_t)(v >> 32);
             } else {
-                r[0] = *reinterpret_cast<const uint32_t*>(ptr + (uint64_t)lane * 4);
+                r[0] = row_load<COH>(reinterpret_cast<const uint32_t*>(ptr + (uint64_t)lane * 4));
             }
         } else {
-            if constexpr (E == 2) r[0] = *reinterpret_cast<const uint32_t*>(ptr + (uint64_t)lane * 4);
-            else r[0] = *reinterpret_cast<const uint16_t*>(ptr + (uint64_t)lane * 2);
+            if constexpr (E == 2) r[0] = row_load<COH>(reinterpret_cast<const uint32_t*>(ptr + (uint64_t)lane * 4));
+            else r[0] = row_load<COH>(reinterpret_cast<const uint16_t*>(ptr + (uint64_t)lane * 2));
         }
     }
     static __device__ __forceinline__ void store_side(const uint32_t* r, uint64_t ptr, bool fp32, int lane)
     {
         if (fp32) {
-            if constexpr (E == 2) *reinterpret_cast<uint2*>(ptr + (uint64_t)lane * 8) = make_uint2(r[0], r[1]);
-            else *reinterpret_cast<uint32_t*>(ptr + (uint64_t)lane * 4) = r[0];
+            if constexpr (E == 2) row_store<COH>(reinterpret_cast<uint64_t*>(ptr + (uint64_t)lane * 8), (uint64_t)r[0] | ((uint64_t)r[1] << 32));
+            else row_store<COH>(reinterpret_cast<uint32_t*>(ptr + (uint64_t)lane * 4), r[0]);
         } else {
-            if constexpr (E == 2) *reinterpret_cast<uint32_t*>(ptr + (uint64_t)lane * 4) = r[0];
-            else *reinterpret_cast<uint16_t*>(ptr + (uint64_t)lane * 2) = (uint16_t)r[0];
+            if constexpr (E == 2) row_store<COH>(reinterpret_cast<uint32_t*>(ptr + (uint64_t)lane * 4), r[0]);
+            else row_store<COH>(reinterpret_cast<uint16_t*>(ptr + (uint64_t)lane * 2), (uint16_t)r[0]);
         }
     }
     template <int CLS> __device__ __forceinline__ void load(Row& row, const Info& i) const
@@ -279,8 +280,15 @@ template <int K> struct MascotRule {
     __device__ __forceinline__ void finish(const Params& a, uint32_t) const
     {
         __syncthreads();
-        for (uint32_t g = threadIdx.x; g < user_groups; g += blockDim.x) a.norm_sum_p[(size_t)gridDim.x * g + blockIdx.x] = unorm_s[g];
-        for (uint32_t g = threadIdx.x; g < item_groups; g += blockDim.x) a.norm_sum_q[(size_t)gridDim.x * g + blockIdx.x] = inorm_s[g];
+        // a launch that continues an epoch (accumulate) adds to what the earlier launches of the epoch left
+        for (uint32_t g = threadIdx.x; g < user_groups; g += blockDim.x) {
+            float* dst = &a.norm_sum_p[(size_t)gridDim.x * g + blockIdx.x];
+            *dst = a.accumulate ? *dst + unorm_s[g] : unorm_s[g];
+        }
+        for (uint32_t g = threadIdx.x; g < item_groups; g += blockDim.x) {
+            float* dst = &a.norm_sum_q[(size_t)gridDim.x * g + blockIdx.x];
+            *dst = a.accumulate ? *dst + inorm_s[g] : inorm_s[g];
+        }
     }
 };
 

@@ -68,8 +68,8 @@ __device__ __forceinline__ uint32_t muppet_scale_index(unsigned bitwidth, float 
 }
 __device__ __forceinline__ half_t grid_h(float v, float s, float s_rev) { return (half_t)(roundf(v * s) * s_rev); }
 
-template <int K> struct MuppetRule : DenseBase<K> {
-    using Base = DenseBase<K>;
+template <int K, bool COH> struct MuppetRule : DenseBase<K, COH> {
+    using Base = DenseBase<K, COH>;
     using typename Base::Row;
     using typename Base::Info;
     static constexpr int E = Base::E;
@@ -77,8 +77,9 @@ template <int K> struct MuppetRule : DenseBase<K> {
     static constexpr int kAhead = 1, kRing = 4;
     struct Params {
         float* p; float* q; float lrate; float lambda; uint32_t first_sample;
-        float* sum_updated_val; float* sum_norms; uint32_t num_workers; int fwd; int bwd;
+        float* sum_updated_val; float* sum_norms; uint32_t num_workers; int fwd; int bwd; bool accumulate;
     };
+    static constexpr bool kSplittable = false;     // per-worker statistics span the whole launch
     float lrate, lambda; uint32_t first_sample; float* sum_updated_val; int fwd, bwd;
     float sum_norms_reg;
     float grad_acc[K / 64];
@@ -233,14 +234,15 @@ __device__ __forceinline__ int afp_sat8(float t) { return (int)(t > 127.0f ? 127
 __device__ __forceinline__ float ufirst(float x) { return from_bits<float>((uint32_t)__builtin_amdgcn_readfirstlane((int)bits(x))); }
 __device__ __forceinline__ int ufirst(int x) { return __builtin_amdgcn_readfirstlane(x); }
 
-template <int K> struct AfpRule : DenseBase<K> {
-    using Base = DenseBase<K>;
+template <int K, bool COH> struct AfpRule : DenseBase<K, COH> {
+    using Base = DenseBase<K, COH>;
     using typename Base::Row;
     using typename Base::Info;
     static constexpr int E = Base::E;
     static constexpr int J = K / 32;
     static constexpr int kAhead = 1, kRing = 4;
-    struct Params { float* p; float* q; float lrate; float lambda; int afp_epoch; int init_threshold; };
+    static constexpr bool kSplittable = false;    // the per-worker quantiser state lives for one launch
+    struct Params { float* p; float* q; float lrate; float lambda; int afp_epoch; int init_threshold; bool accumulate; };
     float lrate, lambda; int afp_epoch, init_threshold;
     AfpQ uq, iq, bq;
     int upd_u, upd_i, upd_b, cur_iter;

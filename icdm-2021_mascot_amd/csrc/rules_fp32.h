@@ -18,7 +18,7 @@ template <int K> struct DenseRow {
 struct DenseInfo { float r; uint32_t u, v; };
 struct NoPrep {};
 
-template <int K> struct DenseBase {
+template <int K, bool COH> struct DenseBase {
     static constexpr int E = K / 64;
     using Row = DenseRow<K>;
     using Info = DenseInfo;
@@ -43,14 +43,14 @@ template <int K> struct DenseBase {
         const float* pp = P + (size_t)i.u * K + lane;
         const float* qq = Q + (size_t)i.v * K + lane;
 #pragma unroll
-        for (int e = 0; e < E; ++e) { row.p[e] = pp[64 * e]; row.q[e] = qq[64 * e]; }
+        for (int e = 0; e < E; ++e) { row.p[e] = row_load<COH>(pp + 64 * e); row.q[e] = row_load<COH>(qq + 64 * e); }
     }
     __device__ __forceinline__ void store(const Row& row, const Info& i) const
     {
         float* pp = P + (size_t)i.u * K + lane;
         float* qq = Q + (size_t)i.v * K + lane;
 #pragma unroll
-        for (int e = 0; e < E; ++e) { pp[64 * e] = row.p[e]; qq[64 * e] = row.q[e]; }
+        for (int e = 0; e < E; ++e) { row_store<COH>(pp + 64 * e, row.p[e]); row_store<COH>(qq + 64 * e, row.q[e]); }
     }
     __device__ __forceinline__ void forward(Row& nxt, const Info& in, const Row& cur, const Info& ic) const
     {
@@ -79,13 +79,14 @@ template <int E, class T> __device__ __forceinline__ T dot_reference_order(const
 }
 
 // single_sgd_k128/k64_hogwild_kernel, sgd/sgd_kernel.h:55-76.
-template <int K> struct SgdRule : DenseBase<K> {
-    using Base = DenseBase<K>;
+template <int K, bool COH> struct SgdRule : DenseBase<K, COH> {
+    using Base = DenseBase<K, COH>;
     using typename Base::Row;
     using typename Base::Info;
     static constexpr int E = Base::E;
     static constexpr int kAhead = 3, kRing = 8;
-    struct Params { float* p; float* q; float lrate; float lambda; };
+    static constexpr bool kSplittable = true;
+    struct Params { float* p; float* q; float lrate; float lambda; bool accumulate; };
     float lrate, lambda;
 
     __device__ __forceinline__ void init(const Params& a, uint8_t*, int lane_, uint32_t)
@@ -111,13 +112,14 @@ template <int K> struct SgdRule : DenseBase<K> {
 };
 
 // mpt_sgd_k128/k64_hogwild_kernel, mpt/mpt_sgd_kernel.h:15-16,38-91.
-template <int K> struct MptRule : DenseBase<K> {
-    using Base = DenseBase<K>;
+template <int K, bool COH> struct MptRule : DenseBase<K, COH> {
+    using Base = DenseBase<K, COH>;
     using typename Base::Row;
     using typename Base::Info;
     static constexpr int E = Base::E;
     static constexpr int kAhead = 3, kRing = 8;
-    struct Params { float* p; float* q; float lrate; uint16_t scaled_lambda_half; float scaling_factor; };
+    static constexpr bool kSplittable = true;
+    struct Params { float* p; float* q; float lrate; uint16_t scaled_lambda_half; float scaling_factor; bool accumulate; };
     float lrate, scaling_factor_rev;
     half_t lambda_h, scaling_factor_h;
 

@@ -39,6 +39,22 @@ typedef struct { float r; uint32_t u; uint32_t i; } mf_node;
 
 int mf_version(void);
 const char* mf_last_error(void);
+/* How the update kernels read and write P/Q rows (process-wide, takes effect at the next launch):
+ *   1 (default)  device-coherent: every row access bypasses the per-XCD L2 (agent-scope relaxed atomics),
+ *                so a worker always sees the latest row any other worker stored -- the semantics the
+ *                reference gets from a GPU with one L2.  All accesses to one row serialise at the
+ *                memory side, which bounds the epoch when a single row takes percents of all ratings.
+ *   0            cached: ordinary loads and stores; each of the 8 XCDs works on its own L2-resident copy
+ *                of a hot row until it is evicted, copies are merged last-writer-wins.
+ * No counterpart in the reference (one L2, nothing to choose).  mf_train picks per run, see there. */
+int mf_set_row_coherence(int coherent);
+int mf_get_row_coherence(void);
+/* Cuts every fp32-SGD / MPT / MASCOT update call into `splits` consecutive kernel launches (each worker's
+ * windows are divided evenly).  A kernel boundary writes back and invalidates the per-XCD L2s, so with
+ * cached row accesses the XCDs' copies of hot rows are reconciled `splits` times per epoch instead of once.
+ * Default 1.  No counterpart in the reference. */
+int mf_set_epoch_splits(uint32_t splits);
+uint32_t mf_get_epoch_splits(void);
 /* Number of per-block columns mf_mascot_sgd_hogwild writes into norm_sum_p / norm_sum_q
  * (the reference's `block_num`, mf_methods.cu:109). */
 uint32_t mf_mascot_norm_blocks(uint32_t num_workers);
@@ -155,6 +171,68 @@ int mf_matrix_reconst_triplet(mf_node* R, const uint32_t* user2sorted_idx, const
 /* Seeded replacement for srand(time(0)); std::random_shuffle(R, R+n) (mf_methods.cu:38-39): out = in
  * permuted by ascending 64-bit key(seed, i).  Allocates temporaries with hipMalloc, synchronises. */
 int mf_shuffle_ratings(const mf_node* in, mf_node* out, uint32_t n, uint64_t seed, void* stream);
+
+/* ---- host training drivers (the reference's mf_methods.h:4-11 surface) -------------------
+ * These take HOST pointers, allocate and free their own device memory with hipMalloc, run on
+ * the current device's default stream and block until the run is finished.  One host thread. */
+
+/* Parameter + the run-level fields of Mf_info, common_struct.h:19-35,87-91; defaults main.cu:19-32. */
+typedef struct {
+    float lambda;             /* -b  */
+    float learning_rate;      /* -a  */
+    float decay;              /* -d  */
+    float sample_ratio;       /* -r / -s */
+    float error_threshold;    /* -e  */
+    uint32_t interval;        /* -it */
+    uint32_t user_group_num;  /* -ug (requested; the grouping may return fewer, preprocess_utils.h:189-190) */
+    uint32_t item_group_num;  /* -ig */
+    uint32_t k;               /* -k  */
+    uint32_t num_workers;     /* -wg */
+    uint32_t epoch;           /* -l  */
+    uint32_t thread_block_size; /* -bl: accepted for compatibility; workgroups are always 4 wavefronts here */
+    uint32_t version;         /* -v: 1 MASCOT, 2 AFP, 3 MuPPET, 4 MPT, 5 fp32 SGD (0 = alias of 5) */
+    uint32_t is_yahoo;        /* MuPPET starts at 12 bit (mf_methods.cu:600) */
+    uint64_t seed;            /* replaces time(0) / clock() seeding */
+    uint32_t verbose;         /* 1: print the reference's stdout lines (mf_methods.cu:396 etc.) */
+    uint32_t cached_rows;     /* 0: device-coherent row accesses (default), 1: cached, see mf_set_row_coherence */
+    uint32_t epoch_splits;    /* kernel launches per epoch, 0 or 1 = one, see mf_set_epoch_splits */
+    uint32_t reserved;
+} mf_params;
+
+/* What a run reports back; every pointer is optional host memory owned by the caller. */
+typedef struct {
+    double* rmse_per_epoch;        /* [epoch] test RMSE after each epoch (mf_methods.cu:395-396) */
+    float* lr_per_epoch;           /* [epoch] */
+    float* sgd_ms_per_epoch;       /* [epoch] hipEvent time of the update kernel(s) (mf_methods.cu:187-241) */
+    uint32_t* user2sorted_idx;     /* [n_users] MASCOT only: dense id -> popularity-sorted row */
+    uint32_t* item2sorted_idx;     /* [n_items] */
+    uint32_t* user_group_end_idx;  /* [requested user_group_num] MASCOT only */
+    uint32_t* item_group_end_idx;  /* [requested item_group_num] */
+    uint8_t* user_group_prec_info; /* [requested user_group_num] final precision per group */
+    uint8_t* item_group_prec_info;
+    uint32_t user_group_num;       /* actual number of groups (out) */
+    uint32_t item_group_num;
+    mf_node* test_reconst;         /* [test_n] MASCOT only: the test set in sorted index space (io_utils.h:374-405) */
+    double preprocess_ms, switching_ms, error_ms, sgd_ms, total_ms;   /* mf_methods.cu:401-418 */
+    uint32_t update_count;
+    uint32_t muppet_final_bits;
+} mf_report;
+
+void mf_default_params(mf_params* out);
+/* init_model_single / init_model_half, model_init.cu:138-173: p [n_users*k], q [n_items*k] on the host,
+ * N(0,1)*0.01 from the seeded generator; `half_rounded` != 0 rounds every value through binary16. */
+int mf_init_model(float* p, float* q, uint32_t n_users, uint32_t n_items, uint32_t k, uint64_t seed, int half_rounded);
+/* mascot_training_mf / adaptive_fixed_point_training_mf / muppet_training_mf / mixed_precision_training_mf /
+ * training_single_mf, mf_methods.cu:36-434,436-527,529-711,713-818,820-924, selected by params->version.
+ *   R, test        host COO arrays in dense (first-seen) id space; R is shuffled on the device with
+ *                  params->seed, the caller's array is left untouched
+ *   p, q           host [n_users*k], [n_items*k]: initial model in, trained model out.  For version 1 the
+ *                  rows come back in popularity-sorted order (as save_trained_model_reconst expects). */
+int mf_train(const mf_params* params, const mf_node* R, uint32_t n, uint32_t n_users, uint32_t n_items,
+             const mf_node* test, uint32_t test_n, float* p, float* q, mf_report* report);
+/* Host grouping, split_group_based_equal_size_not_strict_ret_end_idx, preprocess_utils.h:101-190:
+ * sorted_cnt ascending rating counts; writes inclusive end indices (capacity n) and returns their number. */
+uint32_t mf_group_end_indices(const uint32_t* sorted_cnt, uint32_t n, uint32_t requested_groups, uint32_t* end_idx_out);
 
 #ifdef __cplusplus
 }

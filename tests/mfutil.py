@@ -128,3 +128,98 @@ class DeviceGrouped:
     def download(self):
         host = self.arena.cpu().numpy()
         return [host[o:o + s].view(dt).copy() for o, s, dt in zip(self.offs, self.sizes, self.dtypes)]
+
+
+# ---- the checker's end-to-end drivers (restating mf_methods.cu on the CPU) -------------------------
+def test_set_order(test):
+    """test_set_preprocess, preprocess_utils.h:38-52: by user then item, last duplicate wins."""
+    key = test["u"].astype(np.int64) * (1 << 32) + test["i"].astype(np.int64)
+    order = np.argsort(key, kind="stable")
+    t = test[order]
+    key = key[order]
+    last = np.ones(t.size, bool)
+    last[:-1] = key[1:] != key[:-1]
+    return np.ascontiguousarray(t[last])
+
+
+def oracle_train_dense(orc, version, R, test, P, Q, k, W, epochs, lr, lam, decay, seed, threads=8, sample_ratio=0.01):
+    """training_single_mf / mixed_precision_training_mf / muppet_training_mf / adaptive_fixed_point_training_mf
+    (mf_methods.cu:820-924, 713-818, 529-711, 436-527) on the CPU; returns per-epoch test RMSE."""
+    Rs = orc.shuffle(seed, R)
+    uc = orc.lib.orc_update_count(Rs.size, W, 128)
+    rmse = []
+    bits_ladder = [8, 12, 14, 16, 32]
+    pidx, switched, viol, maxdiv = 0, C.c_int(-1), C.c_int(0), C.c_float(-1.0)
+    pidx_c = C.c_int(0)
+    norms_hist = np.zeros(epochs, np.float32)
+    upd_hist = np.zeros((epochs, k), np.float32)
+    first_sample = uc * 128 - int(np.float32(uc * 128) * np.float32(sample_ratio))
+    for e in range(epochs):
+        lre = orc.lib.orc_lr_schedule(lr, decay, e)
+        if version == 5:
+            orc.lib.orc_sgd_epoch(k, Rs.ctypes.data, Rs.size, P.ctypes.data, Q.ctypes.data, W, uc, 128, lre, lam, seed, e, None, threads)
+        elif version == 4:
+            orc.lib.orc_mpt_epoch(k, Rs.ctypes.data, Rs.size, P.ctypes.data, Q.ctypes.data, W, uc, 128, lre, lam, 1000.0, seed, e, None, threads)
+        elif version == 3:
+            s = np.zeros(k, np.float32)
+            nrm = np.zeros(W, np.float32)
+            b = bits_ladder[min(pidx_c.value, 4)]
+            orc.lib.orc_muppet_epoch(k, Rs.ctypes.data, Rs.size, P.ctypes.data, Q.ctypes.data, W, uc, 128, lre, lam, first_sample,
+                                     s.ctypes.data, nrm.ctypes.data, b, b, seed, e, None, 1)
+            norms_hist[e] = np.float32(nrm.sum(dtype=np.float32))
+            upd_hist[e] = s
+            orc.lib.orc_muppet_ladder_step(k, e, C.byref(switched), C.byref(pidx_c), C.byref(maxdiv), C.byref(viol),
+                                           norms_hist.ctypes.data, upd_hist.ctypes.data)
+        elif version == 2:
+            orc.lib.orc_afp_epoch(k, Rs.ctypes.data, Rs.size, P.ctypes.data, Q.ctypes.data, W, uc, 128, lre, lam, e, seed, e, None, 1)
+        rmse.append(orc.rmse(k, test, P, Q))
+    return np.array(rmse), dict(final_bits=bits_ladder[min(pidx_c.value, 4)])
+
+
+def oracle_train_mascot(orc, R, test, P, Q, k, W, epochs, lr, lam, decay, seed, ug, ig, sample_ratio, interval, threshold, threads=8):
+    """mascot_training_mf, mf_methods.cu:36-434, on the CPU: shuffle, histogram, sort, grouping, re-index,
+    scatter into binary16 groups, epochs with sampled error estimation and precision switching."""
+    n_users, n_items = P.shape[0], Q.shape[0]
+    Rs = orc.shuffle(seed, R)
+    ucnt, icnt = orc.histogram(Rs, n_users, n_items)
+    suc, sui = orc.sort_by_count(ucnt)
+    sic, sii = orc.sort_by_count(icnt)
+    uend, iend = orc.grouping(suc, ug), orc.grouping(sic, ig)
+    u2s, u2g, usz = orc.reindex_tables(sui, uend)
+    i2s, i2g, isz = orc.reindex_tables(sii, iend)
+    test = test.copy()
+    orc.lib.orc_reindex(Rs.ctypes.data, Rs.size, u2s.ctypes.data, i2s.ctypes.data)
+    orc.lib.orc_reindex(test.ctypes.data, test.size, u2s.ctypes.data, i2s.ctypes.data)
+    Ps = np.empty_like(P); Ps[u2s] = P
+    Qs = np.empty_like(Q); Qs[i2s] = Q
+    gu = host_grouped(orc, k, Ps, uend, np.zeros(uend.size, np.uint8))
+    gi = host_grouped(orc, k, Qs, iend, np.zeros(iend.size, np.uint8))
+    uc = orc.lib.orc_update_count(Rs.size, W, 128)
+    init_u, init_i = np.ones(uend.size, np.float32), np.ones(iend.size, np.float32)
+    rmse, switches = [], []
+    for e in range(epochs):
+        lre = orc.lib.orc_lr_schedule(lr, decay, e)
+        first = orc.lib.orc_first_sample_rating_idx(e, interval, epochs, uc, 128, sample_ratio)
+        check = bool(orc.lib.orc_is_error_check_epoch(e, interval, epochs))
+        gsp, gsq = np.zeros(uend.size * k, np.float32), np.zeros(iend.size * k, np.float32)
+        nsp, nsq = np.zeros(uend.size, np.float32), np.zeros(iend.size, np.float32)
+        orc.lib.orc_mascot_epoch(k, Rs.ctypes.data, Rs.size, gu.ptrs, gi.ptrs, gu.end_idx.ctypes.data, gi.end_idx.ctypes.data,
+                                 gu.prec.ctypes.data, gi.prec.ctypes.data, gu.groups, gi.groups, W, uc, 128, lre, lam, first,
+                                 gsp.ctypes.data, gsq.ctypes.data, nsp.ctypes.data, nsq.ctypes.data, seed, e, None, threads)
+        if check:
+            eu, ei = np.zeros(uend.size, np.float32), np.zeros(iend.size, np.float32)
+            orc.lib.orc_group_error(k, gu.groups, gsp.ctypes.data, nsp.ctypes.data, 1, gu.prec.ctypes.data, init_u.ctypes.data, eu.ctypes.data)
+            orc.lib.orc_group_error(k, gi.groups, gsq.ctypes.data, nsq.ctypes.data, 1, gi.prec.ctypes.data, init_i.ctypes.data, ei.ctypes.data)
+            if e == 5:
+                init_u, init_i = eu.copy(), ei.copy()
+            if e > 5:       # precision_switching_by_groups_grad_diversity, precision_switching.h:8-51
+                for gm, err in ((gu, eu), (gi, ei)):
+                    for g in range(gm.groups):
+                        if err[g] > threshold and gm.prec[g] == 0:
+                            gm.arrays[g] = orc.h2f(gm.arrays[g])
+                            gm.prec[g] = 1
+                    gm.refresh()
+            switches.append((e, eu.copy(), ei.copy()))
+        rmse.append(orc.lib.orc_rmse_grouped(k, test.ctypes.data, test.size, gu.ptrs, gi.ptrs, gu.end_idx.ctypes.data, gi.end_idx.ctypes.data,
+                                             gu.prec.ctypes.data, gi.prec.ctypes.data, gu.groups, gi.groups))
+    return np.array(rmse), dict(gu=gu, gi=gi, uend=uend, iend=iend, u2s=u2s, i2s=i2s, test=test, errors=switches)

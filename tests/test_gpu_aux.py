@@ -1,0 +1,223 @@
+"""GPU parity of the kernels around the update loop (conversion, grouped storage, g-switching error,
+RMSE, init, histogram/sort/reindex/shuffle) against the CPU checker, through the C ABI."""
+import numpy as np
+import pytest
+
+import mfutil
+from mfutil import to_dev, from_dev
+
+pytestmark = pytest.mark.gpu
+
+
+def _sync():
+    import torch
+    torch.cuda.synchronize()
+
+
+def test_float2half_exhaustive_halves_and_midpoints(orc):
+    """Bit-exact RN-even conversion: every binary16 value, every tie and its neighbours, random floats."""
+    import torch
+    h = mfutil.hip()
+    hb = np.arange(65536, dtype=np.uint16)
+    f = hb.view(np.float16).astype(np.float32)
+    pos = np.arange(0, 0x7C00, dtype=np.uint16)
+    lo = pos.view(np.float16).astype(np.float64)
+    hi = (pos + 1).astype(np.uint16).view(np.float16).astype(np.float64)
+    hi[-1] = 65536.0
+    mid = ((lo + hi) / 2).astype(np.float32)
+    rng = np.random.default_rng(1)
+    rnd = rng.integers(0, 2 ** 32, 1_000_001, dtype=np.uint64).astype(np.uint32).view(np.float32)   # odd length: tail path
+    x = np.concatenate([f[np.isfinite(f)], mid, np.nextafter(mid, np.float32(np.inf)), np.nextafter(mid, np.float32(-np.inf)), -mid, rnd])
+    x = x[~np.isnan(x)]
+    if x.size % 2 == 0:
+        x = x[:-1]
+    dx = to_dev(x)
+    dout = torch.zeros(x.size + 1, dtype=torch.int16, device="cuda")
+    h.mf_transform_float2half(dx.data_ptr(), dout.data_ptr(), x.size, mfutil.stream_ptr())
+    _sync()
+    got = dout.cpu().numpy().view(np.uint16)[:x.size]
+    assert np.array_equal(got, orc.f2h(x))
+    with np.errstate(over="ignore"):
+        assert np.array_equal(got, x.astype(np.float16).view(np.uint16))
+
+
+def test_half2float_exhaustive(orc):
+    import torch
+    h = mfutil.hip()
+    hb = np.arange(65535, dtype=np.uint16)     # odd count on purpose
+    dx = to_dev(hb)
+    dout = torch.zeros(hb.size, dtype=torch.float32, device="cuda")
+    h.mf_transform_half2float(dx.data_ptr(), dout.data_ptr(), hb.size, mfutil.stream_ptr())
+    _sync()
+    got = dout.cpu().numpy()
+    want = orc.h2f(hb)
+    nan = np.isnan(want)
+    assert np.array_equal(got[~nan].view(np.uint32), want[~nan].view(np.uint32))
+    assert np.all(np.isnan(got[nan]))
+
+
+def test_empty_inputs_are_no_ops():
+    h = mfutil.hip()
+    assert h.mf_transform_float2half(None, None, 0, None) == 0
+    assert h.mf_test_rmse(None, 0, None, None, 64, None, None) == 0
+    assert h.mf_user_item_histogram(None, 0, None, None, None) == 0
+    assert h.mf_sort_by_count(None, None, 0, None) == 0
+    assert h.mf_shuffle_ratings(None, None, 0, 1, None) == 0
+
+
+def _preprocess_reference(orc, R, n_users, n_items, ug_req, ig_req):
+    uc, ic = orc.histogram(R, n_users, n_items)
+    suc, sui = orc.sort_by_count(uc)
+    sic, sii = orc.sort_by_count(ic)
+    uend, iend = orc.grouping(suc, ug_req), orc.grouping(sic, ig_req)
+    u2s, u2g, usz = orc.reindex_tables(sui, uend)
+    i2s, i2g, isz = orc.reindex_tables(sii, iend)
+    return dict(uc=uc, ic=ic, suc=suc, sui=sui, sic=sic, sii=sii, uend=uend, iend=iend, u2s=u2s, u2g=u2g, i2s=i2s, i2g=i2g)
+
+
+def test_histogram_sort_reindex(orc):
+    import torch
+    h = mfutil.hip()
+    n_users, n_items = 3000, 700
+    R = mfutil.make_ratings(5, n_users, n_items, 200_000, alpha=1.0)
+    ref = _preprocess_reference(orc, R, n_users, n_items, 20, 10)
+    dR = to_dev(R)
+    ub = torch.zeros(n_users, dtype=torch.int32, device="cuda")
+    ib = torch.zeros(n_items, dtype=torch.int32, device="cuda")
+    st = mfutil.stream_ptr()
+    h.mf_user_item_histogram(dR.data_ptr(), R.size, ub.data_ptr(), ib.data_ptr(), st)
+    _sync()
+    assert np.array_equal(ub.cpu().numpy().view(np.uint32), ref["uc"])
+    assert np.array_equal(ib.cpu().numpy().view(np.uint32), ref["ic"])
+    uidx = torch.zeros(n_users, dtype=torch.int32, device="cuda")
+    iidx = torch.zeros(n_items, dtype=torch.int32, device="cuda")
+    h.mf_init_idx_arr(uidx.data_ptr(), n_users, st)
+    h.mf_init_idx_arr(iidx.data_ptr(), n_items, st)
+    h.mf_sort_by_count(ub.data_ptr(), uidx.data_ptr(), n_users, st)
+    h.mf_sort_by_count(ib.data_ptr(), iidx.data_ptr(), n_items, st)
+    assert np.array_equal(ub.cpu().numpy().view(np.uint32), ref["suc"])
+    assert np.array_equal(uidx.cpu().numpy().view(np.uint32), ref["sui"])      # stable: ties keep id order
+    assert np.array_equal(iidx.cpu().numpy().view(np.uint32), ref["sii"])
+    du2s, di2s = to_dev(ref["u2s"]), to_dev(ref["i2s"])
+    h.mf_matrix_reconst_triplet(dR.data_ptr(), du2s.data_ptr(), di2s.data_ptr(), R.size, st)
+    _sync()
+    want = R.copy()
+    orc.lib.orc_reindex(want.ctypes.data, want.size, ref["u2s"].ctypes.data, ref["i2s"].ctypes.data)
+    assert np.array_equal(from_dev(dR, np.uint8), want.view(np.uint8).reshape(-1))
+
+
+def test_shuffle_is_the_checkers_permutation(orc):
+    import torch
+    h = mfutil.hip()
+    R = mfutil.make_ratings(6, 500, 300, 123_457)
+    dR = to_dev(R)
+    dOut = torch.zeros(R.size * 12, dtype=torch.uint8, device="cuda")
+    h.mf_shuffle_ratings(dR.data_ptr(), dOut.data_ptr(), R.size, 77, mfutil.stream_ptr())
+    got = from_dev(dOut, mfutil.NODE)
+    want = orc.shuffle(77, R)
+    assert np.array_equal(got.view(np.uint8), want.view(np.uint8))
+    # a permutation of the input, and not the identity
+    assert np.array_equal(np.sort(got.view(np.uint8).reshape(-1, 12).view("V12").ravel()), np.sort(R.view("V12").ravel()))
+    assert not np.array_equal(got.view(np.uint8), R.view(np.uint8))
+
+
+def test_init_normal_bit_exact_and_distribution(orc):
+    import torch
+    from scipy import stats
+    h = mfutil.hip()
+    n = 1_000_003
+    d = torch.zeros(n, dtype=torch.float32, device="cuda")
+    h.mf_init_rand_feature(d.data_ptr(), n, 42, 1, mfutil.stream_ptr())
+    _sync()
+    got = d.cpu().numpy()
+    want = orc.init_normal(42, 1, n)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    # model_init.cu:25: N(0,1) * 0.01
+    assert abs(got.mean()) < 5e-5 and abs(got.std() - 0.01) < 5e-5
+    assert stats.kstest(got[:200000] / 0.01, "norm").pvalue > 1e-3
+    other = orc.init_normal(42, 0, 1000)
+    assert not np.array_equal(other, want[:1000])
+
+
+@pytest.mark.parametrize("k", [64, 128])
+def test_scatter_gather_rmse_grouped(orc, k):
+    import torch
+    h = mfutil.hip()
+    st = mfutil.stream_ptr()
+    n_users, n_items = 900, 400
+    R = mfutil.make_ratings(7 + k, n_users, n_items, 60_000)
+    test = mfutil.make_ratings(8 + k, n_users, n_items, 10_001)
+    ref = _preprocess_reference(orc, R, n_users, n_items, 12, 9)
+    P = orc.init_normal(1, 0, n_users * k).reshape(n_users, k) * 10
+    Q = orc.init_normal(1, 1, n_items * k).reshape(n_items, k) * 10
+    # dense RMSE in original id space
+    dT, dP, dQ = to_dev(test), to_dev(P), to_dev(Q)
+    acc = torch.zeros(1, dtype=torch.float64, device="cuda")
+    h.mf_test_rmse(dT.data_ptr(), test.size, dP.data_ptr(), dQ.data_ptr(), k, acc.data_ptr(), st)
+    _sync()
+    rm = float(np.sqrt(acc.cpu().numpy()[0] / test.size))
+    assert abs(rm - orc.rmse(k, test, P, Q)) <= 1e-6 * rm
+    # scatter rows into grouped binary16 storage (model_init.cu:30-56)
+    sizes_u = np.diff(np.concatenate([[-1], ref["uend"].astype(np.int64)]))
+    sizes_i = np.diff(np.concatenate([[-1], ref["iend"].astype(np.int64)]))
+    gu = orc_grouped_zero(k, ref["uend"], sizes_u)
+    gi = orc_grouped_zero(k, ref["iend"], sizes_i)
+    du, di = mfutil.DeviceGrouped(gu), mfutil.DeviceGrouped(gi)
+    d_u2g, d_u2s, d_i2g, d_i2s = to_dev(ref["u2g"]), to_dev(ref["u2s"]), to_dev(ref["i2g"]), to_dev(ref["i2s"])
+    h.mf_cpyparams2grouped_params(dP.data_ptr(), du.ptrs.data_ptr(), du.end.data_ptr(), d_u2g.data_ptr(), d_u2s.data_ptr(), k, n_users, du.groups, st)
+    h.mf_cpyparams2grouped_params(dQ.data_ptr(), di.ptrs.data_ptr(), di.end.data_ptr(), d_i2g.data_ptr(), d_i2s.data_ptr(), k, n_items, di.groups, st)
+    _sync()
+    Ps = np.empty_like(P); Ps[ref["u2s"]] = P          # rows in sorted order
+    Qs = np.empty_like(Q); Qs[ref["i2s"]] = Q
+    want_u = mfutil.host_grouped(orc, k, Ps, ref["uend"], np.zeros(du.groups, np.uint8))
+    want_i = mfutil.host_grouped(orc, k, Qs, ref["iend"], np.zeros(di.groups, np.uint8))
+    for got, want in zip(du.download() + di.download(), want_u.arrays + want_i.arrays):
+        assert np.array_equal(got, want)
+    # gather back to dense (sorted order), widening exactly
+    dense = torch.zeros(n_users * k, dtype=torch.float32, device="cuda")
+    h.mf_grouped_params2dense(du.ptrs.data_ptr(), du.end.data_ptr(), du.prec.data_ptr(), dense.data_ptr(), k, n_users, du.groups, st)
+    _sync()
+    assert np.array_equal(dense.cpu().numpy().reshape(n_users, k), orc.h2f(orc.f2h(Ps)))
+    # RMSE straight from grouped storage on the re-indexed test set
+    tr = test.copy()
+    orc.lib.orc_reindex(tr.ctypes.data, tr.size, ref["u2s"].ctypes.data, ref["i2s"].ctypes.data)
+    dTr = to_dev(tr)
+    acc.zero_()
+    h.mf_test_rmse_grouped(dTr.data_ptr(), tr.size, du.ptrs.data_ptr(), di.ptrs.data_ptr(), k, du.end.data_ptr(), di.end.data_ptr(),
+                           du.prec.data_ptr(), di.prec.data_ptr(), du.groups, di.groups, acc.data_ptr(), st)
+    _sync()
+    rm_g = float(np.sqrt(acc.cpu().numpy()[0] / tr.size))
+    want_g = orc.lib.orc_rmse_grouped(k, tr.ctypes.data, tr.size, want_u.ptrs, want_i.ptrs, want_u.end_idx.ctypes.data, want_i.end_idx.ctypes.data,
+                                      want_u.prec.ctypes.data, want_i.prec.ctypes.data, want_u.groups, want_i.groups)
+    assert abs(rm_g - want_g) <= 1e-6 * want_g
+    assert abs(rm_g - rm) < 5e-3        # binary16 storage of the same model: close to the fp32 figure
+
+
+def orc_grouped_zero(k, end_idx, sizes):
+    from oracle import oracle as om
+    arrays = [np.zeros(int(s) * k, np.uint16) for s in sizes]
+    return om.GroupedModel(k, end_idx, np.zeros(len(sizes), np.uint8), arrays)
+
+
+@pytest.mark.parametrize("k", [64, 128])
+def test_group_error_matches_host_formula(orc, k):
+    import torch
+    h = mfutil.hip()
+    rng = np.random.default_rng(9)
+    G, nb = 37, 513
+    gs = rng.standard_normal(G * k).astype(np.float32) * 3
+    ns = rng.random(G * nb).astype(np.float32)
+    prec = (rng.random(G) < 0.3).astype(np.uint8)
+    init = (rng.random(G).astype(np.float32) + 0.5)
+    want = np.zeros(G, np.float32)
+    orc.lib.orc_group_error(k, G, gs.ctypes.data, ns.ctypes.data, nb, prec.ctypes.data, init.ctypes.data, want.ctypes.data)
+    dgs, dns, dpr, din = to_dev(gs), to_dev(ns), to_dev(prec), to_dev(init)
+    out = torch.zeros(G, dtype=torch.float32, device="cuda")
+    h.mf_group_error(dgs.data_ptr(), dns.data_ptr(), nb, dpr.data_ptr(), din.data_ptr(), out.data_ptr(), k, G, mfutil.stream_ptr())
+    _sync()
+    got = out.cpu().numpy()
+    assert np.array_equal(got[prec == 1], np.full(int(prec.sum()), -1, np.float32))
+    assert np.allclose(got[prec == 0], want[prec == 0], rtol=1e-5)
+    # the accumulators of binary16 groups are cleared for the next check epoch (mf_methods.cu:333)
+    left = from_dev(dgs, np.float32).reshape(G, k)
+    assert np.all(left[prec == 0] == 0)

@@ -1,0 +1,168 @@
+"""End-to-end parity of the host training drivers (mf_train through the C ABI) and the quantized_mf
+command line against the checker's CPU runs on the same seeded data, shuffle and initial model.
+Hogwild races make trajectories differ run to run, so the bar is the north-star tolerance: final test
+RMSE within 0.005 of the reference rule.  The runs use device-coherent row accesses and a few dozen
+workers: with Zipf(1.0) popularity a handful of rows take percents of all ratings, and the number of
+updates in flight decides how many of a hot row's updates survive (on the GPU as on the CPU)."""
+import os
+import subprocess
+
+import numpy as np
+import pytest
+
+import mfutil
+
+pytestmark = pytest.mark.gpu
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CLI = os.path.join(os.path.dirname(HERE), "icdm-2021_mascot_amd", "quantized_mf")
+
+
+def _split(R, n_train):
+    return np.ascontiguousarray(R[:n_train]), mfutil.test_set_order(R[n_train:])
+
+
+def test_config1_fp32_sgd_k64(orc):
+    """BASELINE config 1: 5,000 x 2,000, 500k ratings (80/20), Zipf(1.0), rank-8 truth, integers 1-5;
+    fp32 SGD, k=64, 10 epochs, lr 0.01, lambda 0.05, decay 0.1."""
+    h = mfutil.hip()
+    R = mfutil.make_ratings(2021, 5000, 2000, 500_000, rank=8, alpha=1.0, step=1.0, lo=1, hi=5, mean=3.5, noise=0.5)
+    train, test = _split(R, 400_000)
+    k, W, E = 64, 8, 10
+    prm = h.default_params(k=k, num_workers=W, epoch=E, learning_rate=0.01, lam=0.05, decay=0.1, version=5, seed=11)
+    p, q = h.init_model(5000, 2000, k, 11)
+    p0, q0 = orc.init_normal(11, 0, 5000 * k).reshape(5000, k), orc.init_normal(11, 1, 2000 * k).reshape(2000, k)
+    assert np.array_equal(p, p0) and np.array_equal(q, q0)
+    out = h.train(prm, train, 5000, 2000, test, p, q)
+    ref, _ = mfutil.oracle_train_dense(orc, 5, train, test, p0, q0, k, W, E, 0.01, 0.05, 0.1, 11)
+    print("gpu", out["rmse"], "\ncpu", ref)
+    assert np.all(np.diff(out["rmse"]) < 0)
+    assert abs(out["rmse"][-1] - ref[-1]) < 0.005
+    assert np.max(np.abs(out["rmse"] - ref)[2:]) < 0.01      # the first two epochs are the steep part of the curve
+    # the model that comes back is the one the RMSE was measured on
+    assert abs(orc.rmse(k, test, p, q) - out["rmse"][-1]) < 1e-6
+    assert np.allclose(out["lr"], [orc.lib.orc_lr_schedule(0.01, 0.1, e) for e in range(E)], rtol=0, atol=0)
+
+
+@pytest.mark.parametrize("version,k", [(4, 128), (3, 64), (2, 128)])
+def test_dense_variants_track_the_checker(orc, version, k):
+    h = mfutil.hip()
+    n_users, n_items = 3000, 1200
+    R = mfutil.make_ratings(77 + version, n_users, n_items, 250_000, rank=8, alpha=1.0)
+    train, test = _split(R, 200_000)
+    W, E = 4, 10
+    prm = h.default_params(k=k, num_workers=W, epoch=E, learning_rate=0.01, lam=0.05, decay=0.1, version=version, seed=5, sample_ratio=0.05)
+    half = version == 4
+    p, q = h.init_model(n_users, n_items, k, 5, half_rounded=half)
+    p0, q0 = orc.init_normal(5, 0, n_users * k).reshape(n_users, k), orc.init_normal(5, 1, n_items * k).reshape(n_items, k)
+    if half:
+        p0, q0 = orc.h2f(orc.f2h(p0)), orc.h2f(orc.f2h(q0))
+    assert np.array_equal(p, p0) and np.array_equal(q, q0)
+    out = h.train(prm, train, n_users, n_items, test, p, q)
+    ref, info = mfutil.oracle_train_dense(orc, version, train, test, p0, q0, k, W, E, 0.01, 0.05, 0.1, 5, sample_ratio=0.05)
+    print("gpu", out["rmse"], "\ncpu", ref)
+    assert out["rmse"][-1] < out["rmse"][0]
+    assert abs(out["rmse"][-1] - ref[-1]) < 0.005
+    if version == 3:
+        assert out["report"].muppet_final_bits in (8, 12, 14, 16, 32)
+
+
+def test_mascot_reduced_config2(orc):
+    """BASELINE config 2 at one tenth: Zipf(0.9), rank-16 truth, ratings 0.5-5.0 in half steps; MASCOT k=128,
+    sample ratio 0.05, period 2; a low threshold so that groups do switch to binary32 within 12 epochs."""
+    h = mfutil.hip()
+    n_users, n_items = 7000, 1070
+    R = mfutil.make_ratings(2, n_users, n_items, 1_000_000, rank=16, alpha=0.9, step=0.5, lo=0.5, hi=5.0, mean=3.5, noise=0.8)
+    train, test = _split(R, 800_000)
+    k, W, E = 128, 8, 12
+    kw = dict(k=k, num_workers=W, epoch=E, learning_rate=0.01, lam=0.015, decay=0.1, version=1, seed=3,
+              user_group_num=20, item_group_num=20, sample_ratio=0.05, interval=2, error_threshold=1.5)
+    prm = h.default_params(**kw)
+    p, q = h.init_model(n_users, n_items, k, 3)
+    p0, q0 = p.copy(), q.copy()
+    out = h.train(prm, train, n_users, n_items, test, p, q)
+    ref, info = mfutil.oracle_train_mascot(orc, train, test, p0, q0, k, W, E, 0.01, 0.015, 0.1, 3, 20, 20, 0.05, 2, 1.5)
+    print("gpu", out["rmse"], "\ncpu", ref)
+    print("gpu prec", out["user_prec"], out["item_prec"], "\ncpu prec", info["gu"].prec, info["gi"].prec)
+    # integer pre-processing is bit-exact
+    assert np.array_equal(out["user_end"], info["uend"]) and np.array_equal(out["item_end"], info["iend"])
+    assert np.array_equal(out["user2sorted"], info["u2s"]) and np.array_equal(out["item2sorted"], info["i2s"])
+    assert np.array_equal(out["test_reconst"].view(np.uint8), info["test"].view(np.uint8))
+    assert abs(out["rmse"][-1] - ref[-1]) < 0.005
+    assert np.max(np.abs(out["rmse"] - ref)[2:]) < 0.01
+    # model returned in sorted row order reproduces the reported RMSE on the sorted-space test set
+    assert abs(orc.rmse(k, out["test_reconst"], p, q) - out["rmse"][-1]) < 1e-6
+    # switching decisions: the error estimate is a noisy statistic of a racy trajectory (its device-side
+    # arithmetic is pinned exactly in test_gpu_hogwild / test_gpu_aux); here only groups whose estimate is
+    # far above the threshold on the CPU run must also have switched on the GPU, and both runs must switch
+    errs = {e: (eu, ei) for e, eu, ei in info["errors"]}
+    for got_prec, ref_gm, idx in ((out["user_prec"], info["gu"], 0), (out["item_prec"], info["gi"], 1)):
+        decided = np.zeros(ref_gm.groups, bool)
+        for e, pair in errs.items():
+            if e > 5:
+                decided |= (pair[idx] > 1.5 * 3)
+        assert np.all(got_prec[decided] == 1)
+        assert got_prec.sum() >= 1 and ref_gm.prec.sum() >= 1
+
+
+def _write_tsv(path, R, offset=0):
+    with open(path, "w") as f:
+        for r, u, i in zip(R["r"].tolist(), R["u"].tolist(), R["i"].tolist()):
+            f.write("%d\t%d\t%g\n" % (u * 3 + 1 + offset, i * 2 + 5, r))
+
+
+@pytest.mark.parametrize("version", [1, 5])
+def test_quantized_mf_command_line(orc, tmp_path, version):
+    """The C++ command line: reference flags in, per-epoch "<epoch> <lr> <rmse>" lines and the reference's
+    model-file layout out (io_utils.h:242-332)."""
+    assert os.path.exists(CLI), "quantized_mf is not built"
+    n_users, n_items, k = 400, 150, 64
+    R = mfutil.make_ratings(31, n_users, n_items, 40_000)
+    train, test = R[:32_000], R[32_000:]
+    tr, te = str(tmp_path / "train.tsv"), str(tmp_path / "test.tsv")
+    _write_tsv(tr, train)
+    _write_tsv(te, test)
+    with open(te, "a") as f:
+        f.write("999999\t5\t3\n")          # unseen user: dropped and listed in remove_user.txt (io_utils.h:191-193)
+    out = str(tmp_path / "model")
+    cmd = [CLI, "-i", tr, "-y", te, "-o", out, "-v", str(version), "-k", str(k), "-l", "7", "-wg", "64", "-a", "0.01", "-b", "0.05",
+           "-d", "0.1", "-ug", "5", "-ig", "4", "-s", "0.05", "-it", "1", "-e", "2", "-rc", "1", "-seed", "9"]
+    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=300)
+    assert res.returncode == 0, res.stderr
+    lines = [l.split() for l in res.stdout.splitlines()]
+    epochs = [l for l in lines if len(l) == 3 and l[0].isdigit()]
+    assert [int(l[0]) for l in epochs] == list(range(1, 8))
+    rm = np.array([float(l[2]) for l in epochs])
+    assert rm[-1] < rm[0]
+    assert "Missing the number of ratings : 1" in res.stdout
+    assert open(str(tmp_path / "remove_user.txt")).read().split() == ["999999"]
+    n_tr_users = np.unique(train["u"]).size
+    n_tr_items = np.unique(train["i"]).size
+    if version == 1:
+        model = out + "_reconst.txt"
+        head = open(model).readline().split()
+        assert head == [str(n_tr_users), str(n_tr_items), str(k)]
+        rows = open(model).read().split("\n")
+        assert len(rows[1].split()) == n_tr_users * k and len(rows[2].split()) == n_tr_items * k
+        P = np.array(rows[1].split(), np.float32).reshape(n_tr_users, k)
+        Q = np.array(rows[2].split(), np.float32).reshape(n_tr_items, k)
+        rt = np.loadtxt(str(tmp_path / "reconst_test.tsv"), dtype=np.float64)
+        tn = np.empty(rt.shape[0], mfutil.NODE)
+        tn["u"], tn["i"], tn["r"] = rt[:, 0], rt[:, 1], rt[:, 2]
+        # 6 significant digits in the text file (default ostream precision)
+        assert abs(orc.rmse(k, tn, P, Q) - rm[-1]) < 2e-4
+    else:
+        model = out + ".txt"
+        head = open(model).readline().split()
+        max_u = int(train["u"].max()) * 3 + 1
+        max_i = int(train["i"].max()) * 2 + 5
+        assert head == [str(max_u + 1), str(max_i + 1), str(k)]
+        rows = open(model).read().split("\n")
+        P = np.array(rows[1].split(), np.float32).reshape(max_u + 1, k)
+        Q = np.array(rows[2].split(), np.float32).reshape(max_i + 1, k)
+        assert np.all(P[0] == 0) and np.all(Q[0] == 0)          # absent original ids are zero rows
+        keep = np.isin(test["u"], train["u"]) & np.isin(test["i"], train["i"])
+        tn = mfutil.test_set_order(test[keep])
+        tn["u"] = tn["u"] * 3 + 1
+        tn["i"] = tn["i"] * 2 + 5
+        assert abs(orc.rmse(k, tn, P, Q) - rm[-1]) < 2e-4
