@@ -1,0 +1,274 @@
+#!/usr/bin/env python3
+"""Benchmark of the MASCOT SGD hot path on one MI355X.
+
+A step is one epoch's update launch of MASCOT (k=128, ug=ig=100, sample ratio 0.05, period 2) over the
+synthetic 480,000 x 17,800 matrix with 100M training ratings (item popularity Zipf(1.1), integers 1-5 from a
+rank-32 truth plus N(0,0.9) noise) -- the fourth configuration of BASELINE.json.  Inputs are resident in HBM
+before the timed region.  Everything goes through the C ABI of libmascot_hip.so; torch only owns the device
+memory and the stream.  One JSON line on stdout.
+"""
+import argparse
+import ctypes as C
+import importlib
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+PEAK_HBM_GBS = 8000.0
+
+
+def zipf_ranks(torch, count, size, alpha, gen, dev):
+    w = 1.0 / torch.arange(1, count + 1, device=dev, dtype=torch.float64) ** alpha
+    cdf = torch.cumsum(w, 0)
+    cdf = cdf / cdf[-1]
+    out = torch.empty(size, dtype=torch.int64, device=dev)
+    step = 20_000_000
+    for s in range(0, size, step):
+        r = torch.rand(min(step, size - s), device=dev, generator=gen, dtype=torch.float64)
+        out[s:s + r.numel()] = torch.searchsorted(cdf, r).clamp_(max=count - 1)
+    return out
+
+
+def make_workload(torch, n_users, n_items, n, seed, dev, user_alpha, item_alpha, rank, noise, mean):
+    """COO ratings [n][3] int32 (float bits, user, item) on the device, ids in random (unsorted) order."""
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(seed)
+    uperm = torch.randperm(n_users, device=dev, generator=gen)
+    iperm = torch.randperm(n_items, device=dev, generator=gen)
+    u = uperm[zipf_ranks(torch, n_users, n, user_alpha, gen, dev)]
+    i = iperm[zipf_ranks(torch, n_items, n, item_alpha, gen, dev)]
+    U = torch.randn(n_users, rank, device=dev, generator=gen) * 0.5
+    V = torch.randn(n_items, rank, device=dev, generator=gen) * 0.5
+    R = torch.empty((n, 3), dtype=torch.int32, device=dev)
+    step = 10_000_000
+    for s in range(0, n, step):
+        e = min(n, s + step)
+        val = (U[u[s:e]] * V[i[s:e]]).sum(1) + mean + torch.randn(e - s, device=dev, generator=gen) * noise
+        R[s:e, 0] = val.round_().clamp_(1, 5).to(torch.float32).view(torch.int32)
+    R[:, 1] = u.to(torch.int32)
+    R[:, 2] = i.to(torch.int32)
+    return R
+
+
+class MascotProblem:
+    """Device-resident MASCOT training state built with the library's own pre-processing kernels."""
+
+    def __init__(self, torch, h, R, n_users, n_items, k, ug, ig, seed, test=None):
+        self.torch, self.h, self.k = torch, h, k
+        dev = R.device
+        st = torch.cuda.current_stream().cuda_stream
+        n = R.shape[0]
+        self.n, self.n_users, self.n_items = n, n_users, n_items
+        # seeded shuffle (mf_methods.cu:38-39)
+        self.R = torch.empty_like(R)
+        h.mf_shuffle_ratings(R.data_ptr(), self.R.data_ptr(), n, seed, st)
+        # histogram -> sort -> grouping -> re-index (preprocess_utils.h:54-255)
+        ucnt = torch.zeros(n_users, dtype=torch.int32, device=dev)
+        icnt = torch.zeros(n_items, dtype=torch.int32, device=dev)
+        h.mf_user_item_histogram(self.R.data_ptr(), n, ucnt.data_ptr(), icnt.data_ptr(), st)
+        self.sides = []
+        for cnt, num, req in ((ucnt, n_users, ug), (icnt, n_items, ig)):
+            idx = torch.empty(num, dtype=torch.int32, device=dev)
+            h.mf_init_idx_arr(idx.data_ptr(), num, st)
+            h.mf_sort_by_count(cnt.data_ptr(), idx.data_ptr(), num, st)
+            sorted_cnt = cnt.cpu().numpy().view(np.uint32)
+            sorted_id = idx.cpu().numpy().view(np.uint32)
+            end = np.zeros(num, np.uint32)
+            g = h.mf_group_end_indices(sorted_cnt.ctypes.data, num, req, end.ctypes.data)
+            end = end[:g].copy()
+            id2sorted = np.empty(num, np.uint32)
+            id2sorted[sorted_id] = np.arange(num, dtype=np.uint32)
+            id2group = np.searchsorted(end, id2sorted).astype(np.uint32)
+            self.sides.append(dict(end=end, id2sorted=id2sorted, id2group=id2group, groups=g, num=num))
+        du2s = torch.from_numpy(self.sides[0]["id2sorted"].view(np.int32)).to(dev)
+        di2s = torch.from_numpy(self.sides[1]["id2sorted"].view(np.int32)).to(dev)
+        h.mf_matrix_reconst_triplet(self.R.data_ptr(), du2s.data_ptr(), di2s.data_ptr(), n, st)
+        self.test = None
+        if test is not None:
+            self.test = test.clone()
+            h.mf_matrix_reconst_triplet(self.test.data_ptr(), du2s.data_ptr(), di2s.data_ptr(), self.test.shape[0], st)
+        # model init (model_init.cu:114-173) and scatter into binary16 groups (model_init.cu:175-222)
+        for side, (s, d_id2sorted) in enumerate(zip(self.sides, (du2s, di2s))):
+            num, g, end = s["num"], s["groups"], s["end"]
+            dense = torch.empty(num * k, dtype=torch.float32, device=dev)
+            h.mf_init_rand_feature(dense.data_ptr(), num * k, seed, side, st)
+            sizes = np.diff(np.concatenate([[-1], end.astype(np.int64)]))
+            offs = np.concatenate([[0], np.cumsum((sizes * k * 2 + 255) // 256 * 256)[:-1]])
+            arena = torch.zeros(int((sizes * k * 2 + 255).sum() // 1 + 256 * g), dtype=torch.uint8, device=dev)
+            ptrs = torch.tensor([arena.data_ptr() + int(o) for o in offs], dtype=torch.int64, device=dev)
+            d_end = torch.from_numpy(end.view(np.int32)).to(dev)
+            d_prec = torch.zeros(g, dtype=torch.uint8, device=dev)
+            d_id2group = torch.from_numpy(s["id2group"].view(np.int32)).to(dev)
+            h.mf_cpyparams2grouped_params(dense.data_ptr(), ptrs.data_ptr(), d_end.data_ptr(), d_id2group.data_ptr(),
+                                          d_id2sorted.data_ptr(), k, num, g, st)
+            s.update(arena=arena, ptrs=ptrs, d_end=d_end, d_prec=d_prec, sizes=sizes, offs=offs)
+            torch.cuda.synchronize()
+            s["initial"] = arena.clone()
+        self.stats = None
+
+    def reset(self):
+        for s in self.sides:
+            s["arena"].copy_(s["initial"])
+
+    def alloc_stats(self, W):
+        torch, h, k = self.torch, self.h, self.k
+        nb = h.mf_mascot_norm_blocks(W)
+        U, I = self.sides
+        dev = self.R.device
+        self.stats = dict(W=W, nb=nb,
+                          gsp=torch.zeros(U["groups"] * k, device=dev), gsq=torch.zeros(I["groups"] * k, device=dev),
+                          nsp=torch.zeros(U["groups"] * nb, device=dev), nsq=torch.zeros(I["groups"] * nb, device=dev))
+
+    def epoch(self, e, W, epochs, lr0, decay, lam, sample_ratio, interval, seed):
+        h, U, I, s = self.h, self.sides[0], self.sides[1], self.stats
+        st = self.torch.cuda.current_stream().cuda_stream
+        uc = h.mf_update_count(self.n, W, 128)
+        first = h.mf_first_sample_rating_idx(e, interval, epochs, uc, 128, sample_ratio)
+        if first < uc * 128:
+            s["gsp"].zero_()
+            s["gsq"].zero_()
+        h.mf_mascot_sgd_hogwild(self.R.data_ptr(), self.n, U["ptrs"].data_ptr(), I["ptrs"].data_ptr(), self.k, W, uc, 128,
+                                h.mf_lr_schedule(lr0, decay, e), lam, U["d_end"].data_ptr(), I["d_end"].data_ptr(),
+                                U["d_prec"].data_ptr(), I["d_prec"].data_ptr(), s["gsp"].data_ptr(), s["gsq"].data_ptr(),
+                                s["nsp"].data_ptr(), s["nsq"].data_ptr(), first, U["groups"], I["groups"], seed, e, None, st)
+        return uc
+
+    def rmse(self):
+        torch, h, U, I = self.torch, self.h, self.sides[0], self.sides[1]
+        acc = torch.zeros(1, dtype=torch.float64, device=self.R.device)
+        h.mf_test_rmse_grouped(self.test.data_ptr(), self.test.shape[0], U["ptrs"].data_ptr(), I["ptrs"].data_ptr(), self.k,
+                               U["d_end"].data_ptr(), I["d_end"].data_ptr(), U["d_prec"].data_ptr(), I["d_prec"].data_ptr(),
+                               U["groups"], I["groups"], acc.data_ptr(), torch.cuda.current_stream().cuda_stream)
+        return float(np.sqrt(acc.item() / self.test.shape[0]))
+
+    def host_grouped(self):
+        """Host mirror of the grouped model for the CPU checker."""
+        from oracle import oracle as om
+        out = []
+        for s in self.sides:
+            host = s["arena"].cpu().numpy()
+            arrays = [host[int(o):int(o) + int(sz) * self.k * 2].view(np.uint16).copy() for o, sz in zip(s["offs"], s["sizes"])]
+            out.append(om.GroupedModel(self.k, s["end"], np.zeros(s["groups"], np.uint8), arrays))
+        return out
+
+
+def time_steps(torch, prob, W, warmup, steps, cfg, seed):
+    """W untimed epochs, then K epochs each bracketed by events on the launch stream."""
+    prob.reset()
+    prob.alloc_stats(W)
+    for e in range(warmup):
+        prob.epoch(e, W, cfg["epochs"], cfg["lr"], cfg["decay"], cfg["lam"], cfg["sample_ratio"], cfg["interval"], seed)
+    torch.cuda.synchronize()
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    t0 = time.perf_counter()
+    uc = 0
+    for i in range(steps):
+        ev[i][0].record()
+        uc = prob.epoch(warmup + i, W, cfg["epochs"], cfg["lr"], cfg["decay"], cfg["lam"], cfg["sample_ratio"], cfg["interval"], seed)
+        ev[i][1].record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    per = np.array([a.elapsed_time(b) for a, b in ev])
+    return per, wall, uc
+
+
+def cpu_baseline(prob, cfg, seed, threads, target_updates):
+    """The checker's MASCOT epoch (reference update rule, binary16 through F16C) as a Hogwild CPU loop."""
+    from oracle import oracle as om
+    orc = om.get()
+    R = prob.R.cpu().numpy().view(np.uint8).reshape(-1).view(om.NODE)
+    gu, gi = prob.host_grouped()
+    W = threads * 8
+    uc = max(1, target_updates // (W * 128))
+    z = [np.zeros(n, np.float32) for n in (gu.groups * prob.k, gi.groups * prob.k, gu.groups, gi.groups)]
+    t0 = time.perf_counter()
+    orc.lib.orc_mascot_epoch(prob.k, R.ctypes.data, R.size, gu.ptrs, gi.ptrs, gu.end_idx.ctypes.data, gi.end_idx.ctypes.data,
+                             gu.prec.ctypes.data, gi.prec.ctypes.data, gu.groups, gi.groups, W, uc, 128,
+                             cfg["lr"], cfg["lam"], uc * 128, z[0].ctypes.data, z[1].ctypes.data, z[2].ctypes.data, z[3].ctypes.data,
+                             seed, 0, None, threads)
+    dt = time.perf_counter() - t0
+    done = W * uc * 128
+    return done / dt, done, dt
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--ratings", type=int, default=100_000_000)
+    ap.add_argument("--workers", type=int, default=2048, help="-wg of the measured run (reference default for k=128)")
+    ap.add_argument("--cached-workers", type=int, default=16384)
+    ap.add_argument("--cpu-updates", type=int, default=6_000_000, help="size of the CPU baseline sample")
+    ap.add_argument("--skip-cpu", action="store_true")
+    ap.add_argument("--skip-cached", action="store_true")
+    ap.add_argument("--seed", type=int, default=2021)
+    a = ap.parse_args()
+    if a.gpus != 1:
+        print("bench.py: this build runs on one GPU only (every box has one; the multi-GPU sharding is a design note "
+              "in DESIGN.md); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    h = importlib.import_module("icdm-2021_mascot_amd").load()
+    dev = torch.device("cuda:0")
+    n_users, n_items, k = 480_000, 17_800, 128
+    cfg = dict(epochs=50, lr=0.01, decay=0.1, lam=0.015, sample_ratio=0.05, interval=2, ug=100, ig=100)
+    t0 = time.perf_counter()
+    R = make_workload(torch, n_users, n_items, a.ratings, a.seed, dev, user_alpha=0.8, item_alpha=1.1, rank=32, noise=0.9, mean=3.6)
+    prob = MascotProblem(torch, h, R, n_users, n_items, k, cfg["ug"], cfg["ig"], a.seed)
+    del R
+    torch.cuda.synchronize()
+    setup_s = time.perf_counter() - t0
+    bytes_per_update = 12 + 2 * k * (2 + 2)          # all groups still binary16 in the measured epochs: 1036 B
+
+    def leg(coherent, W):
+        h.mf_set_row_coherence(1 if coherent else 0)
+        per, wall, uc = time_steps(torch, prob, W, a.warmup, a.steps, cfg, a.seed)
+        updates = W * uc * 128
+        ms = float(per.mean())
+        return dict(ms_per_step=ms, ms_steps=[round(float(x), 3) for x in per], wall_s=wall, updates_per_step=updates,
+                    ratings_per_s=a.ratings / (ms / 1e3), gbs=updates * bytes_per_update / (ms / 1e3) / 1e9, workers=W)
+
+    main_leg = leg(True, a.workers)
+    out = {
+        "metric": "SGD ratings/sec/epoch & % HBM roofline at k=128 on 1 MI355X; test RMSE delta",
+        "value": main_leg["ratings_per_s"], "unit": "ratings/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": main_leg["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16", "data": "synthetic",
+        "config": {"workload": "config 4: 480000 users x 17800 items, %d train ratings, item Zipf(1.1), user Zipf(0.8), "
+                               "ints 1-5 from rank-32 truth + N(0,0.9); MASCOT -v 1 -k 128 -ug 100 -ig 100 -s 0.05 -it 2 -e 20" % a.ratings,
+                   "workers": a.workers, "row_access": "device-coherent", "update_vector_size": 128,
+                   "epochs_timed": "%d..%d of 50" % (a.warmup, a.warmup + a.steps - 1), "seed": a.seed,
+                   "user_groups": int(prob.sides[0]["groups"]), "item_groups": int(prob.sides[1]["groups"]), "setup_s": round(setup_s, 1)},
+        "roofline": {"bound": "hbm", "achieved": main_leg["gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": main_leg["gbs"] / PEAK_HBM_GBS, "traffic": None,
+                     "kernel": "hogwild_kernel<MascotRule<128,true>>", "bytes_per_update": bytes_per_update,
+                     "updates_per_launch": main_leg["updates_per_step"]},
+        "ms_steps": main_leg["ms_steps"],
+    }
+    if not a.skip_cached:
+        c = leg(False, a.cached_workers)
+        out["cached_rows"] = {"note": "same workload with ordinary cached row accesses (each XCD trains its own L2-resident copy of hot "
+                                      "rows; faster, converges worse, see DESIGN.md)",
+                              "value": c["ratings_per_s"], "unit": "ratings/s", "ms_per_step": c["ms_per_step"], "workers": c["workers"],
+                              "roofline": {"bound": "hbm", "achieved": c["gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": c["gbs"] / PEAK_HBM_GBS,
+                                           "kernel": "hogwild_kernel<MascotRule<128,false>>"},
+                              "ms_steps": c["ms_steps"]}
+        h.mf_set_row_coherence(1)
+    if not a.skip_cpu:
+        threads = min(os.cpu_count() or 1, 16)
+        prob.reset()
+        rate, done, dt = cpu_baseline(prob, cfg, a.seed, threads, a.cpu_updates)
+        out["cpu_baseline"] = {"value": rate, "unit": "ratings/s", "cores": threads, "kind": "port",
+                               "sample": "%d updates of the same shuffled ratings and binary16 model (%d workers x %d windows of 128), "
+                                         "%.1f s, OpenMP Hogwild loop of the checker" % (done, threads * 8, done // (threads * 8 * 128), dt)}
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

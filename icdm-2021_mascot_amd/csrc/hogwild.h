@@ -63,14 +63,18 @@ __device__ __forceinline__ void process_chunk(Rule& rule, const Rating& my, cons
 }
 
 template <class Rule>
-__global__ __launch_bounds__(kBlock) void hogwild_kernel(Schedule s, typename Rule::Params prm)
+__global__ __launch_bounds__(kMaxBlock) void hogwild_kernel(Schedule s, typename Rule::Params prm)
 {
     extern __shared__ __align__(16) uint8_t smem[];
     const int lane = threadIdx.x & (kWave - 1);
-    const uint32_t wid = (uint32_t)__builtin_amdgcn_readfirstlane((int)(blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6)));
+    const uint32_t waves_per_block = blockDim.x >> 6;
+    const uint32_t total_waves = gridDim.x * waves_per_block;
+    const uint32_t first_wid = (uint32_t)__builtin_amdgcn_readfirstlane((int)(blockIdx.x * waves_per_block + (threadIdx.x >> 6)));
     Rule rule;
-    rule.init(prm, smem, lane, wid);                    // may synchronise the workgroup
-    if (wid < s.num_workers && s.range_begin < s.range_end) {
+    rule.init(prm, smem, lane, first_wid);              // may synchronise the workgroup
+    // a launch normally has one wavefront per worker; a launch with fewer wavefronts (the sampled tail of
+    // a MASCOT epoch, which keeps per-workgroup statistics in LDS) lets each wavefront play several workers
+    for (uint32_t wid = first_wid; wid < s.num_workers && s.range_begin < s.range_end; wid += total_waves) {
         // this worker handles ratings with processed index in [range_begin, range_end)
         uint32_t processed = s.range_begin;
         uint32_t ite = s.range_begin / s.update_vector_size;
@@ -120,7 +124,7 @@ __global__ __launch_bounds__(kBlock) void hogwild_kernel(Schedule s, typename Ru
             processed = nprocessed; c = nc; ite = nite; start = nstart; n = nn; my = nmy;
         }
     }
-    rule.finish(prm, wid);                               // may synchronise the workgroup
+    rule.finish(prm, first_wid);                         // may synchronise the workgroup
 }
 
 }  // namespace mf

@@ -5,6 +5,7 @@
 #include "rules_fixed_point.h"
 #include <cmath>
 #include <cstring>
+#include <vector>
 
 namespace mf {
 
@@ -45,21 +46,48 @@ static int g_row_coherence = 1;
 // different XCDs are reconciled during an epoch
 static uint32_t g_epoch_splits = 1;
 
+struct Segment { uint32_t begin, end; bool tail; };
+template <class P> static auto set_tail(P& p, bool v) -> decltype(p.lds_stats, void()) { p.lds_stats = v; }
+static void set_tail(...) {}
+
 template <class Rule>
-static int launch(const char* who, const Schedule& s0, const typename Rule::Params& prm0, size_t lds, void* stream)
+static int launch(const char* who, const Schedule& s0, const typename Rule::Params& prm0, size_t lds, void* stream,
+                  uint32_t tail_begin = 0xffffffffu, size_t tail_lds = 0)
 {
     if (s0.update_count == 0 || s0.update_vector_size == 0) return MF_OK;
-    uint32_t splits = Rule::kSplittable ? g_epoch_splits : 1;
-    if (splits > s0.update_count) splits = s0.update_count;
     const uint32_t total = s0.range_end;
+    // [0, body_end) runs as ordinary launches (cut into g_epoch_splits pieces on window boundaries);
+    // [body_end, total) -- the sampled tail of a MASCOT check epoch -- runs as one launch of large workgroups
+    // that keep their gradient sums in LDS
+    const bool has_tail = tail_begin < total;
+    const uint32_t body_end = has_tail ? tail_begin : total;
+    std::vector<Segment> seg;
+    uint32_t splits = Rule::kSplittable ? g_epoch_splits : 1;
+    const uint32_t body_windows = body_end / s0.update_vector_size;
+    if (splits > body_windows) splits = body_windows ? body_windows : 1;
     for (uint32_t i = 0; i < splits; ++i) {
+        const uint32_t b = (uint32_t)((uint64_t)body_windows * i / splits) * s0.update_vector_size;
+        const uint32_t e = i + 1 == splits ? body_end : (uint32_t)((uint64_t)body_windows * (i + 1) / splits) * s0.update_vector_size;
+        if (b < e || !has_tail) seg.push_back({b, e, false});
+    }
+    if (has_tail) seg.push_back({body_end, total, true});
+    bool first = true;
+    for (const Segment& sg : seg) {
         Schedule s = s0;
         typename Rule::Params prm = prm0;
-        // cut on window boundaries
-        s.range_begin = (uint32_t)((uint64_t)s0.update_count * i / splits) * s0.update_vector_size;
-        s.range_end = i + 1 == splits ? total : (uint32_t)((uint64_t)s0.update_count * (i + 1) / splits) * s0.update_vector_size;
-        prm.accumulate = i != 0;
-        hipLaunchKernelGGL((hogwild_kernel<Rule>), dim3(grid_for(s.num_workers)), dim3(kBlock), lds, as_stream(stream), s, prm);
+        s.range_begin = sg.begin; s.range_end = sg.end;
+        prm.accumulate = !first;
+        first = false;
+        if (sg.tail) {
+            uint32_t blocks = (s.num_workers + 15) / 16;
+            if (blocks > 256) blocks = 256;
+            if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&hogwild_kernel<Rule>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)tail_lds),
+                                   "hipFuncSetAttribute(MaxDynamicSharedMemorySize)")) return rc;
+            set_tail(prm, true);
+            hipLaunchKernelGGL((hogwild_kernel<Rule>), dim3(blocks), dim3(kMaxBlock), tail_lds, as_stream(stream), s, prm);
+        } else {
+            hipLaunchKernelGGL((hogwild_kernel<Rule>), dim3(grid_for(s.num_workers)), dim3(kBlock), lds, as_stream(stream), s, prm);
+        }
         if (int rc = launch_status(who)) return rc;
     }
     return MF_OK;
@@ -68,15 +96,16 @@ static int launch(const char* who, const Schedule& s0, const typename Rule::Para
 // Instantiates Rule<K, COH> for the four (k, coherence) combinations; P is the parameter pack type,
 // identical across instantiations apart from the template arguments.
 template <template <int, bool> class Rule, class MakeParams>
-static int launch_k_coh(const char* who, int k, const Schedule& s, MakeParams make, size_t lds, void* stream)
+static int launch_k_coh(const char* who, int k, const Schedule& s, MakeParams make, size_t lds, void* stream,
+                        uint32_t tail_begin = 0xffffffffu, size_t tail_lds = 0)
 {
     const bool coh = g_row_coherence != 0;
     if (k == 128) {
-        if (coh) { auto a = make(typename Rule<128, true>::Params{}); return launch<Rule<128, true>>(who, s, a, lds, stream); }
-        auto a = make(typename Rule<128, false>::Params{}); return launch<Rule<128, false>>(who, s, a, lds, stream);
+        if (coh) { auto a = make(typename Rule<128, true>::Params{}); return launch<Rule<128, true>>(who, s, a, lds, stream, tail_begin, tail_lds); }
+        auto a = make(typename Rule<128, false>::Params{}); return launch<Rule<128, false>>(who, s, a, lds, stream, tail_begin, tail_lds);
     }
-    if (coh) { auto a = make(typename Rule<64, true>::Params{}); return launch<Rule<64, true>>(who, s, a, lds, stream); }
-    auto a = make(typename Rule<64, false>::Params{}); return launch<Rule<64, false>>(who, s, a, lds, stream);
+    if (coh) { auto a = make(typename Rule<64, true>::Params{}); return launch<Rule<64, true>>(who, s, a, lds, stream, tail_begin, tail_lds); }
+    auto a = make(typename Rule<64, false>::Params{}); return launch<Rule<64, false>>(who, s, a, lds, stream, tail_begin, tail_lds);
 }
 
 }  // namespace mf
@@ -208,12 +237,19 @@ int mf_mascot_sgd_hogwild(const mf_node* R, uint32_t nnz, void* const* p, void* 
     const size_t lds = MascotRule<128, true>::lds_bytes(user_group_num, item_group_num);
     if (lds > 64 * 1024) return invalid("%s: group tables need %zu bytes of LDS (limit 65536)", who, lds);
     Schedule s = make_schedule(R, nnz, num_workers, update_count, update_vector_size, seed, epoch, window_start);
+    // sampled tail: its own launch with the gradient sums in LDS when they fit (160 KB per workgroup)
+    uint32_t tail_begin = 0xffffffffu;
+    size_t tail_lds = 0;
+    if (first_sample_rating_idx < update_count * update_vector_size) {
+        const size_t need = lds + (size_t)(user_group_num + item_group_num) * (size_t)k * sizeof(float);
+        if (need <= 160 * 1024) { tail_begin = first_sample_rating_idx; tail_lds = need; }
+    }
     return launch_k_coh<MascotRule>(who, k, s, [&](auto a) {
         a.p = p; a.q = q; a.user_end = user_group_end_idx; a.item_end = item_group_end_idx;
         a.user_prec = user_group_prec_info; a.item_prec = item_group_prec_info;
         a.grad_sum_p = grad_sum_norm_p; a.grad_sum_q = grad_sum_norm_q; a.norm_sum_p = norm_sum_p; a.norm_sum_q = norm_sum_q;
         a.first_sample = first_sample_rating_idx; a.user_groups = user_group_num; a.item_groups = item_group_num;
-        a.lrate = lrate; a.lambda = lambda; return a; }, lds, stream);
+        a.lrate = lrate; a.lambda = lambda; a.norm_stride = grid_for(num_workers); a.lds_stats = false; return a; }, lds, stream, tail_begin, tail_lds);
 }
 
 }  // extern "C"

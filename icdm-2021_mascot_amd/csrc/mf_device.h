@@ -14,6 +14,7 @@ typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 constexpr int kWave = 64;
 constexpr int kBlock = 256;              // 4 wavefronts per workgroup
 constexpr int kWavesPerBlock = kBlock / kWave;
+constexpr int kMaxBlock = 1024;          // the sampled tail of a MASCOT epoch runs 16 wavefronts per workgroup
 
 // ---- bit casts -----------------------------------------------------------------------
 __device__ __forceinline__ uint32_t bits(float x) { return __builtin_bit_cast(uint32_t, x); }

@@ -34,6 +34,8 @@ template <int K, bool COH> struct MascotRule {
         float* grad_sum_p; float* grad_sum_q; float* norm_sum_p; float* norm_sum_q;
         uint32_t first_sample; uint32_t user_groups; uint32_t item_groups;
         float lrate; float lambda; bool accumulate;
+        uint32_t norm_stride;     // columns per group in norm_sum_* (workgroups of an ordinary launch)
+        bool lds_stats;           // sampled gradient sums are kept per workgroup in LDS and flushed once
     };
     static constexpr bool kSplittable = true;
     // raw row registers: binary16 rows use r[0] only
@@ -49,11 +51,13 @@ template <int K, bool COH> struct MascotRule {
     uint32_t* uend_s; uint32_t* iend_s;
     uint8_t* uprec_s; uint8_t* iprec_s;
     float* grad_sum_p; float* grad_sum_q;
+    float* ugrad_s; float* igrad_s;      // per-workgroup [groups][K] sums in LDS, or null
     uint32_t first_sample, user_groups, item_groups;
     float lrate, lambda;
     int lane;
 
-    static size_t lds_bytes(uint32_t ug, uint32_t ig) { return (size_t)(ug + ig) * (8 + 4 + 4 + 1) + 16; }
+    static __host__ __device__ size_t lds_bytes(uint32_t ug, uint32_t ig) { return ((size_t)(ug + ig) * (8 + 4 + 4 + 1) + 31) / 16 * 16; }
+    static size_t lds_stats_bytes(uint32_t ug, uint32_t ig) { return (size_t)(ug + ig) * K * sizeof(float); }
 
     __device__ __forceinline__ void init(const Params& a, uint8_t* smem, int lane_, uint32_t)
     {
@@ -77,6 +81,12 @@ template <int K, bool COH> struct MascotRule {
         }
         grad_sum_p = a.grad_sum_p; grad_sum_q = a.grad_sum_q;
         first_sample = a.first_sample; lrate = a.lrate; lambda = a.lambda;
+        ugrad_s = nullptr; igrad_s = nullptr;
+        if (a.lds_stats) {
+            ugrad_s = reinterpret_cast<float*>(smem + lds_bytes(user_groups, item_groups));
+            igrad_s = ugrad_s + (size_t)user_groups * K;
+            for (uint32_t i = threadIdx.x; i < (user_groups + item_groups) * K; i += blockDim.x) ugrad_s[i] = 0.f;
+        }
         __syncthreads();
     }
 
@@ -207,13 +217,13 @@ template <int K, bool COH> struct MascotRule {
         if constexpr (E == 2) { HV h; h.x = v; h.y = v; return h; } else return v;
     }
     // sampled statistics of one binary16 side: ||g||^2 into the block's LDS slot, g into the global sums
-    __device__ __forceinline__ void sample(const float* g, uint32_t group, float* norm_s, float* grad_sum) const
+    __device__ __forceinline__ void sample(const float* g, uint32_t group, float* norm_s, float* grad_sum, float* grad_s) const
     {
         float n = g[0] * g[0];
         if constexpr (E == 2) n = n + g[1] * g[1];
         n = reduce_wave(n, OpAdd());
         if (lane == 0) atomicAdd(&norm_s[group], n);
-        float* dst = grad_sum + (size_t)group * K + (size_t)lane * E;
+        float* dst = (grad_s ? grad_s : grad_sum) + (size_t)group * K + (size_t)lane * E;
 #pragma unroll
         for (int e = 0; e < E; ++e) atomicAdd(dst + e, g[e]);
     }
@@ -241,10 +251,10 @@ template <int K, bool COH> struct MascotRule {
                 float g[E];
 #pragma unroll
                 for (int e = 0; e < E; ++e) g[e] = widen(gp, e);
-                sample(g, ug, unorm_s, grad_sum_p);
+                sample(g, ug, unorm_s, grad_sum_p, ugrad_s);
 #pragma unroll
                 for (int e = 0; e < E; ++e) g[e] = widen(gq, e);
-                sample(g, ig, inorm_s, grad_sum_q);
+                sample(g, ig, inorm_s, grad_sum_q, igrad_s);
             }
         } else {
             float pf[E], qf[E], m[E];
@@ -270,24 +280,34 @@ template <int K, bool COH> struct MascotRule {
             store_side(row.p, i.pptr, up, lane);
             store_side(row.q, i.qptr, ip, lane);
             if (sampled) {
-                if (!up) sample(gp, ug, unorm_s, grad_sum_p);
-                if (!ip) sample(gq, ig, inorm_s, grad_sum_q);
+                if (!up) sample(gp, ug, unorm_s, grad_sum_p, ugrad_s);
+                if (!ip) sample(gq, ig, inorm_s, grad_sum_q, igrad_s);
             }
         }
     }
 
-    // mascot_sgd_kernel.h:448-456: per-block norm sums, layout [group][block]
+    // mascot_sgd_kernel.h:448-456: per-block norm sums, layout [group][norm_stride]
     __device__ __forceinline__ void finish(const Params& a, uint32_t) const
     {
         __syncthreads();
         // a launch that continues an epoch (accumulate) adds to what the earlier launches of the epoch left
         for (uint32_t g = threadIdx.x; g < user_groups; g += blockDim.x) {
-            float* dst = &a.norm_sum_p[(size_t)gridDim.x * g + blockIdx.x];
+            float* dst = &a.norm_sum_p[(size_t)a.norm_stride * g + blockIdx.x];
             *dst = a.accumulate ? *dst + unorm_s[g] : unorm_s[g];
         }
         for (uint32_t g = threadIdx.x; g < item_groups; g += blockDim.x) {
-            float* dst = &a.norm_sum_q[(size_t)gridDim.x * g + blockIdx.x];
+            float* dst = &a.norm_sum_q[(size_t)a.norm_stride * g + blockIdx.x];
             *dst = a.accumulate ? *dst + inorm_s[g] : inorm_s[g];
+        }
+        if (!a.accumulate) {   // columns no workgroup of this launch owns (a launch of fewer, larger workgroups)
+            for (uint32_t col = gridDim.x + blockIdx.x; col < a.norm_stride; col += gridDim.x) {
+                for (uint32_t g = threadIdx.x; g < user_groups; g += blockDim.x) a.norm_sum_p[(size_t)a.norm_stride * g + col] = 0.f;
+                for (uint32_t g = threadIdx.x; g < item_groups; g += blockDim.x) a.norm_sum_q[(size_t)a.norm_stride * g + col] = 0.f;
+            }
+        }
+        if (ugrad_s) {     // single flush of the workgroup's gradient sums
+            for (uint32_t i = threadIdx.x; i < user_groups * K; i += blockDim.x) { const float v = ugrad_s[i]; if (v != 0.f) atomicAdd(grad_sum_p + i, v); }
+            for (uint32_t i = threadIdx.x; i < item_groups * K; i += blockDim.x) { const float v = igrad_s[i]; if (v != 0.f) atomicAdd(grad_sum_q + i, v); }
         }
     }
 };
