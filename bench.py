@@ -207,6 +207,9 @@ def main():
     ap.add_argument("--cpu-updates", type=int, default=6_000_000, help="size of the CPU baseline sample")
     ap.add_argument("--skip-cpu", action="store_true")
     ap.add_argument("--skip-cached", action="store_true")
+    ap.add_argument("--skip-coherent", action="store_true", help="profiling aid: time only the cached-rows leg")
+    ap.add_argument("--pmc-copy", action="store_true",
+                    help="profiling aid: also run three 1 GiB device copies, the known-size kernel that FETCH_SIZE / WRITE_SIZE are scaled by")
     ap.add_argument("--seed", type=int, default=2021)
     a = ap.parse_args()
     if a.gpus != 1:
@@ -234,7 +237,16 @@ def main():
         return dict(ms_per_step=ms, ms_steps=[round(float(x), 3) for x in per], wall_s=wall, updates_per_step=updates,
                     ratings_per_s=a.ratings / (ms / 1e3), gbs=updates * bytes_per_update / (ms / 1e3) / 1e9, workers=W)
 
-    main_leg = leg(True, a.workers)
+    if a.pmc_copy:
+        src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+    main_leg = leg(False, a.cached_workers) if a.skip_coherent else leg(True, a.workers)
+    if a.skip_coherent:
+        a.skip_cached = True
     out = {
         "metric": "SGD ratings/sec/epoch & % HBM roofline at k=128 on 1 MI355X; test RMSE delta",
         "value": main_leg["ratings_per_s"], "unit": "ratings/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
@@ -242,11 +254,14 @@ def main():
         "dtype": "f16", "data": "synthetic",
         "config": {"workload": "config 4: 480000 users x 17800 items, %d train ratings, item Zipf(1.1), user Zipf(0.8), "
                                "ints 1-5 from rank-32 truth + N(0,0.9); MASCOT -v 1 -k 128 -ug 100 -ig 100 -s 0.05 -it 2 -e 20" % a.ratings,
-                   "workers": a.workers, "row_access": "device-coherent", "update_vector_size": 128,
+                   "workers": main_leg["workers"], "row_access": "cached" if a.skip_coherent else "device-coherent", "update_vector_size": 128,
                    "epochs_timed": "%d..%d of 50" % (a.warmup, a.warmup + a.steps - 1), "seed": a.seed,
                    "user_groups": int(prob.sides[0]["groups"]), "item_groups": int(prob.sides[1]["groups"]), "setup_s": round(setup_s, 1)},
         "roofline": {"bound": "hbm", "achieved": main_leg["gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                     "frac": main_leg["gbs"] / PEAK_HBM_GBS, "traffic": None,
+                     "frac": main_leg["gbs"] / PEAK_HBM_GBS,
+                     # HBM bytes per plain-epoch launch at 100M ratings from rocprofv3 FETCH_SIZE (x2.0) + WRITE_SIZE (x1.0),
+                     # see profiles/hogwild_mascot_k128_config4_hbm_traffic.md; only valid for the default workload
+                     "traffic": (53.4e9 if a.skip_coherent else 99.2e9) if a.ratings == 100_000_000 else None,
                      "kernel": "hogwild_kernel<MascotRule<128,true>>", "bytes_per_update": bytes_per_update,
                      "updates_per_launch": main_leg["updates_per_step"]},
         "ms_steps": main_leg["ms_steps"],
