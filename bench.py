@@ -84,7 +84,7 @@ class MascotProblem:
             id2sorted = np.empty(num, np.uint32)
             id2sorted[sorted_id] = np.arange(num, dtype=np.uint32)
             id2group = np.searchsorted(end, id2sorted).astype(np.uint32)
-            self.sides.append(dict(end=end, id2sorted=id2sorted, id2group=id2group, groups=g, num=num))
+            self.sides.append(dict(end=end, id2sorted=id2sorted, id2group=id2group, groups=g, num=num, sorted_cnt=sorted_cnt.copy()))
         du2s = torch.from_numpy(self.sides[0]["id2sorted"].view(np.int32)).to(dev)
         di2s = torch.from_numpy(self.sides[1]["id2sorted"].view(np.int32)).to(dev)
         h.mf_matrix_reconst_triplet(self.R.data_ptr(), du2s.data_ptr(), di2s.data_ptr(), n, st)
@@ -114,6 +114,25 @@ class MascotProblem:
     def reset(self):
         for s in self.sides:
             s["arena"].copy_(s["initial"])
+
+    def set_thinning(self, W, inflight_cap):
+        """Hot-row thinning tables from the rating counts (rows are in popularity-sorted order), as mf_train builds them."""
+        torch, h = self.torch, self.h
+        if not inflight_cap:
+            h.mf_set_hot_row_thinning(None, None)
+            self.keep = None
+            return 1.0
+        F = min(W, 8192) * 4.0
+        tabs, kept = [], 0.0
+        for s in self.sides:
+            inflight = F * s["sorted_cnt"].astype(np.float64) / self.n
+            keep = np.where(inflight > inflight_cap, inflight_cap / np.maximum(inflight, 1e-30), 1.0)
+            t = np.clip(np.floor(keep * 256.0) - 1, 0, 255).astype(np.uint8)
+            kept += float((s["sorted_cnt"].astype(np.float64) * (t.astype(np.float64) + 1) / 256.0).sum()) / self.n
+            tabs.append(torch.from_numpy(t).to(self.R.device))
+        self.keep = tabs
+        h.mf_set_hot_row_thinning(tabs[0].data_ptr(), tabs[1].data_ptr())
+        return kept / 2
 
     def alloc_stats(self, W):
         torch, h, k = self.torch, self.h, self.k
@@ -208,6 +227,8 @@ def main():
     ap.add_argument("--skip-cpu", action="store_true")
     ap.add_argument("--skip-cached", action="store_true")
     ap.add_argument("--skip-coherent", action="store_true", help="profiling aid: time only the cached-rows leg")
+    ap.add_argument("--skip-exact", action="store_true", help="skip the leg with every row update carried out (no thinning)")
+    ap.add_argument("--hot-row-inflight", type=float, default=16.0, help="hot-row thinning cap of the measured run (0 = off)")
     ap.add_argument("--pmc-copy", action="store_true",
                     help="profiling aid: also run three 1 GiB device copies, the known-size kernel that FETCH_SIZE / WRITE_SIZE are scaled by")
     ap.add_argument("--seed", type=int, default=2021)
@@ -222,20 +243,25 @@ def main():
     n_users, n_items, k = 480_000, 17_800, 128
     cfg = dict(epochs=50, lr=0.01, decay=0.1, lam=0.015, sample_ratio=0.05, interval=2, ug=100, ig=100)
     t0 = time.perf_counter()
-    R = make_workload(torch, n_users, n_items, a.ratings, a.seed, dev, user_alpha=0.8, item_alpha=1.1, rank=32, noise=0.9, mean=3.6)
-    prob = MascotProblem(torch, h, R, n_users, n_items, k, cfg["ug"], cfg["ig"], a.seed)
+    n_test = 1_400_000
+    R = make_workload(torch, n_users, n_items, a.ratings + n_test, a.seed, dev, user_alpha=0.8, item_alpha=1.1, rank=32, noise=0.9, mean=3.6)
+    prob = MascotProblem(torch, h, R[:a.ratings].contiguous(), n_users, n_items, k, cfg["ug"], cfg["ig"], a.seed, test=R[a.ratings:].contiguous())
     del R
     torch.cuda.synchronize()
     setup_s = time.perf_counter() - t0
     bytes_per_update = 12 + 2 * k * (2 + 2)          # all groups still binary16 in the measured epochs: 1036 B
 
-    def leg(coherent, W):
+    def leg(coherent, W, inflight_cap=0.0):
         h.mf_set_row_coherence(1 if coherent else 0)
+        kept = prob.set_thinning(W, inflight_cap)
         per, wall, uc = time_steps(torch, prob, W, a.warmup, a.steps, cfg, a.seed)
+        rmse = prob.rmse()
+        prob.set_thinning(W, 0.0)
         updates = W * uc * 128
         ms = float(per.mean())
         return dict(ms_per_step=ms, ms_steps=[round(float(x), 3) for x in per], wall_s=wall, updates_per_step=updates,
-                    ratings_per_s=a.ratings / (ms / 1e3), gbs=updates * bytes_per_update / (ms / 1e3) / 1e9, workers=W)
+                    ratings_per_s=a.ratings / (ms / 1e3), gbs=updates * bytes_per_update / (ms / 1e3) / 1e9, workers=W,
+                    rmse=rmse, row_updates_kept=kept)
 
     if a.pmc_copy:
         src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
@@ -244,7 +270,7 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
-    main_leg = leg(False, a.cached_workers) if a.skip_coherent else leg(True, a.workers)
+    main_leg = leg(False, a.cached_workers) if a.skip_coherent else leg(True, a.workers, a.hot_row_inflight)
     if a.skip_coherent:
         a.skip_cached = True
     out = {
@@ -256,16 +282,23 @@ def main():
                                "ints 1-5 from rank-32 truth + N(0,0.9); MASCOT -v 1 -k 128 -ug 100 -ig 100 -s 0.05 -it 2 -e 20" % a.ratings,
                    "workers": main_leg["workers"], "row_access": "cached" if a.skip_coherent else "device-coherent", "update_vector_size": 128,
                    "epochs_timed": "%d..%d of 50" % (a.warmup, a.warmup + a.steps - 1), "seed": a.seed,
+                   "hot_row_inflight": 0.0 if a.skip_coherent else a.hot_row_inflight,
+                   "row_updates_carried_out": round(main_leg["row_updates_kept"], 4),
                    "user_groups": int(prob.sides[0]["groups"]), "item_groups": int(prob.sides[1]["groups"]), "setup_s": round(setup_s, 1)},
         "roofline": {"bound": "hbm", "achieved": main_leg["gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
                      "frac": main_leg["gbs"] / PEAK_HBM_GBS,
-                     # HBM bytes per plain-epoch launch at 100M ratings from rocprofv3 FETCH_SIZE (x2.0) + WRITE_SIZE (x1.0),
-                     # see profiles/hogwild_mascot_k128_config4_hbm_traffic.md; only valid for the default workload
-                     "traffic": (53.4e9 if a.skip_coherent else 99.2e9) if a.ratings == 100_000_000 else None,
+                     "traffic": None,
                      "kernel": "hogwild_kernel<MascotRule<128,true>>", "bytes_per_update": bytes_per_update,
                      "updates_per_launch": main_leg["updates_per_step"]},
         "ms_steps": main_leg["ms_steps"],
+        "test_rmse_after_timed_epochs": {"value": main_leg["rmse"], "epochs": a.warmup + a.steps, "test_ratings": n_test},
     }
+    if not a.skip_coherent and not a.skip_exact and a.hot_row_inflight:
+        e = leg(True, a.workers, 0.0)
+        out["exact_coherent"] = {"note": "same workload, device-coherent rows, every row update carried out (no hot-row thinning): bound by "
+                                         "the serialisation of accesses to the hottest row at the memory side",
+                                 "value": e["ratings_per_s"], "unit": "ratings/s", "ms_per_step": e["ms_per_step"], "workers": e["workers"],
+                                 "roofline_frac": e["gbs"] / PEAK_HBM_GBS, "test_rmse_after_timed_epochs": e["rmse"]}
     if not a.skip_cached:
         c = leg(False, a.cached_workers)
         out["cached_rows"] = {"note": "same workload with ordinary cached row accesses (each XCD trains its own L2-resident copy of hot "
@@ -273,7 +306,7 @@ def main():
                               "value": c["ratings_per_s"], "unit": "ratings/s", "ms_per_step": c["ms_per_step"], "workers": c["workers"],
                               "roofline": {"bound": "hbm", "achieved": c["gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": c["gbs"] / PEAK_HBM_GBS,
                                            "kernel": "hogwild_kernel<MascotRule<128,false>>"},
-                              "ms_steps": c["ms_steps"]}
+                              "ms_steps": c["ms_steps"], "test_rmse_after_timed_epochs": c["rmse"]}
         h.mf_set_row_coherence(1)
     if not a.skip_cpu:
         threads = min(os.cpu_count() or 1, 16)

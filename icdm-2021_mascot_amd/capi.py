@@ -20,6 +20,7 @@ SIGNATURES = {
     "mf_get_row_coherence": (i32, []),
     "mf_set_epoch_splits": (i32, [u32]),
     "mf_get_epoch_splits": (u32, []),
+    "mf_set_hot_row_thinning": (i32, [vp, vp]),
     "mf_mascot_norm_blocks": (u32, [u32]),
     "mf_update_count": (u32, [u32, u32, u32]),
     "mf_first_sample_rating_idx": (u32, [u32, u32, u32, u32, u32, f32]),
@@ -59,7 +60,7 @@ class MfParams(C.Structure):
     _fields_ = [("lambda_", f32), ("learning_rate", f32), ("decay", f32), ("sample_ratio", f32), ("error_threshold", f32),
                 ("interval", u32), ("user_group_num", u32), ("item_group_num", u32), ("k", u32), ("num_workers", u32),
                 ("epoch", u32), ("thread_block_size", u32), ("version", u32), ("is_yahoo", u32), ("seed", u64),
-                ("verbose", u32), ("cached_rows", u32), ("epoch_splits", u32), ("reserved", u32)]
+                ("verbose", u32), ("cached_rows", u32), ("epoch_splits", u32), ("hot_row_inflight", f32)]
 
 
 class MfReport(C.Structure):

@@ -91,12 +91,17 @@ __global__ __launch_bounds__(kMaxBlock) void hogwild_kernel(Schedule s, typename
             return left < (uint32_t)kWave ? (int)left : kWave;
         };
         auto fetch = [&](uint32_t st, uint32_t cc, int nn) -> Rating {
-            Rating x = {0.f, 0u, 0u};
+            Rating x = {0.f, 0u, 0u, 0u};
             if (lane < nn) {
                 uint32_t off = (cc + (uint32_t)lane) % s.nnz;
                 uint32_t idx = st + off;
                 if (idx >= s.nnz || idx < st) idx -= s.nnz;
                 x = load_rating(s.R, idx);
+                if (s.keep_u) {
+                    const uint32_t rnd = (uint32_t)(mix64(s.epoch_key ^ (((uint64_t)idx << 20) ^ (uint64_t)wid ^ 0x7468696eull)) >> 40);
+                    if ((rnd & 255u) > (uint32_t)s.keep_u[x.u]) x.thin |= 1u;
+                    if (((rnd >> 8) & 255u) > (uint32_t)s.keep_v[x.v]) x.thin |= 2u;
+                }
             }
             return x;
         };
@@ -109,7 +114,7 @@ __global__ __launch_bounds__(kMaxBlock) void hogwild_kernel(Schedule s, typename
             uint32_t nc = c + (uint32_t)n, nite = ite, nstart = start;
             const bool more = nprocessed < s.range_end;
             int nn = 0;
-            Rating nmy = {0.f, 0u, 0u};
+            Rating nmy = {0.f, 0u, 0u, 0u};
             if (more) {
                 if (nc >= s.update_vector_size) { nc = 0; ++nite; nstart = window_of(nite); }
                 nn = chunk_len(nc, nprocessed);

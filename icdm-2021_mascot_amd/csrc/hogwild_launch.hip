@@ -9,6 +9,9 @@
 
 namespace mf {
 
+// hot-row thinning tables (device pointers, see Schedule::keep_u); null = off
+static const uint8_t* g_keep_u = nullptr;
+static const uint8_t* g_keep_v = nullptr;
 static thread_local char g_error[512] = "";
 void set_error(const char* fmt, ...)
 {
@@ -34,7 +37,7 @@ static Schedule make_schedule(const mf_node* R, uint32_t nnz, uint32_t num_worke
 {
     Schedule s;
     s.R = R; s.nnz = nnz; s.num_workers = num_workers; s.update_count = update_count;
-    s.update_vector_size = update_vector_size; s.range_begin = 0; s.range_end = update_count * update_vector_size; s.epoch_key = window_epoch_key(seed, epoch); s.window_start = window_start;
+    s.update_vector_size = update_vector_size; s.range_begin = 0; s.range_end = update_count * update_vector_size; s.epoch_key = window_epoch_key(seed, epoch); s.window_start = window_start; s.keep_u = g_keep_u; s.keep_v = g_keep_v;
     return s;
 }
 static inline uint32_t grid_for(uint32_t num_workers) { return (num_workers + kWavesPerBlock - 1) / kWavesPerBlock; }
@@ -129,6 +132,12 @@ int mf_set_epoch_splits(uint32_t splits)
     return MF_OK;
 }
 uint32_t mf_get_epoch_splits(void) { return g_epoch_splits; }
+int mf_set_hot_row_thinning(const uint8_t* user_keep, const uint8_t* item_keep)
+{
+    if ((user_keep == nullptr) != (item_keep == nullptr)) return invalid("mf_set_hot_row_thinning: pass both tables or neither");
+    g_keep_u = user_keep; g_keep_v = item_keep;
+    return MF_OK;
+}
 const char* mf_last_error(void) { return g_error; }
 uint32_t mf_mascot_norm_blocks(uint32_t num_workers) { return grid_for(num_workers); }
 

@@ -45,6 +45,7 @@ int main(int argc, const char* argv[])
             if (a == "-seed" && has) prm.seed = std::strtoull(argv[i + 1], nullptr, 10);
             if (a == "-cached" && has) prm.cached_rows = std::atoi(argv[i + 1]);
             if (a == "-split" && has) prm.epoch_splits = std::atoi(argv[i + 1]);
+            if (a == "-hot" && has) prm.hot_row_inflight = std::atof(argv[i + 1]);
             if (a == "-h") { std::cout << argv[0] << usage << std::endl; return 0; }
         }
     }

@@ -103,10 +103,13 @@ __device__ __forceinline__ uint64_t bcast(uint64_t v, int lane)
 // bounds the epoch.  COH = false keeps ordinary cached accesses instead: each XCD then works on its own
 // L2-resident copy of a hot row between evictions (a row that is not re-used while cached behaves the
 // same either way).  The host picks per run (mf_set_row_coherence).
-template <bool COH, class T> __device__ __forceinline__ T row_load(const T* p)
+// `coherent == false` (a thinned access, see Schedule::keep_u) falls back to the cached path.
+template <bool COH, class T> __device__ __forceinline__ T row_load(const T* p, bool coherent = true)
 {
-    if constexpr (COH) return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    else return *p;
+    if constexpr (COH) {
+        if (coherent) return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        return *p;
+    } else return *p;
 }
 template <bool COH, class T> __device__ __forceinline__ void row_store(T* p, T v)
 {
@@ -149,10 +152,17 @@ struct Schedule {
     uint32_t range_begin, range_end;   // processed-index range [begin, end) every worker handles in this launch
     uint64_t epoch_key;
     const uint32_t* window_start;   // optional [update_count][num_workers]
+    // Hot-row thinning (optional, both null = off).  keep_u[row] / keep_v[row] in 0..255: the update of
+    // that row is carried out with probability (keep+1)/256; otherwise the row is only read (through the
+    // caches) for the other side's update and is not written.  Under Hogwild a row with C updates in
+    // flight keeps one of them anyway; thinning such rows to about one update in flight removes the
+    // wasted traffic, which with device-coherent rows is what serialises at the memory side.
+    const uint8_t* keep_u;
+    const uint8_t* keep_v;
 };
 
 // One lane's rating of a 64-rating chunk; the stream is read once per epoch, so bypass-style loads.
-struct Rating { float r; uint32_t u; uint32_t v; };
+struct Rating { float r; uint32_t u; uint32_t v; uint32_t thin; };   // thin: bit0 skip the P update, bit1 skip the Q update
 __device__ __forceinline__ Rating load_rating(const mf_node* R, uint32_t idx)
 {
     const uint32_t* w = reinterpret_cast<const uint32_t*>(R + idx);
@@ -160,6 +170,7 @@ __device__ __forceinline__ Rating load_rating(const mf_node* R, uint32_t idx)
     x.r = from_bits<float>(__builtin_nontemporal_load(w));
     x.u = __builtin_nontemporal_load(w + 1);
     x.v = __builtin_nontemporal_load(w + 2);
+    x.thin = 0u;
     return x;
 }
 

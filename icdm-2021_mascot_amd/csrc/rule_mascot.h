@@ -41,7 +41,7 @@ template <int K, bool COH> struct MascotRule {
     // raw row registers: binary16 rows use r[0] only
     struct Row { uint32_t p[E], q[E]; };
     struct Prep { uint64_t pptr, qptr; uint32_t flags; };
-    struct Info { float r; uint64_t pptr, qptr; uint32_t flags; };
+    struct Info { float r; uint64_t pptr, qptr; uint32_t flags, thin; };
     // flags: bit0 user row is fp32, bit1 item row is fp32, bit2 rating is skipped (index outside the
     // group table), bits 3..16 user group, bits 17..30 item group
     static constexpr uint32_t kSkip = 4u;
@@ -127,21 +127,22 @@ template <int K, bool COH> struct MascotRule {
         i.pptr = bcast(pr.pptr, j);
         i.qptr = bcast(pr.qptr, j);
         i.flags = bcast(pr.flags, j);
+        i.thin = bcast(my.thin, j);
         return i;
     }
 
-    static __device__ __forceinline__ void load_side(uint32_t* r, uint64_t ptr, bool fp32, int lane)
+    static __device__ __forceinline__ void load_side(uint32_t* r, uint64_t ptr, bool fp32, int lane, bool coh)
     {
         if (fp32) {
             if constexpr (E == 2) {
-                const uint64_t v = row_load<COH>(reinterpret_cast<const uint64_t*>(ptr + (uint64_t)lane * 8));
+                const uint64_t v = row_load<COH>(reinterpret_cast<const uint64_t*>(ptr + (uint64_t)lane * 8), coh);
                 r[0] = (uint32_t)v; r[1] = (uint32_t)(v >> 32);
             } else {
-                r[0] = row_load<COH>(reinterpret_cast<const uint32_t*>(ptr + (uint64_t)lane * 4));
+                r[0] = row_load<COH>(reinterpret_cast<const uint32_t*>(ptr + (uint64_t)lane * 4), coh);
             }
         } else {
-            if constexpr (E == 2) r[0] = row_load<COH>(reinterpret_cast<const uint32_t*>(ptr + (uint64_t)lane * 4));
-            else r[0] = row_load<COH>(reinterpret_cast<const uint16_t*>(ptr + (uint64_t)lane * 2));
+            if constexpr (E == 2) r[0] = row_load<COH>(reinterpret_cast<const uint32_t*>(ptr + (uint64_t)lane * 4), coh);
+            else r[0] = row_load<COH>(reinterpret_cast<const uint16_t*>(ptr + (uint64_t)lane * 2), coh);
         }
     }
     static __device__ __forceinline__ void store_side(const uint32_t* r, uint64_t ptr, bool fp32, int lane)
@@ -157,14 +158,14 @@ template <int K, bool COH> struct MascotRule {
     template <int CLS> __device__ __forceinline__ void load(Row& row, const Info& i) const
     {
         if constexpr (CLS == 1) {
-            load_side(row.p, i.pptr, false, lane);
-            load_side(row.q, i.qptr, false, lane);
+            load_side(row.p, i.pptr, false, lane, !(i.thin & 1u));
+            load_side(row.q, i.qptr, false, lane, !(i.thin & 2u));
         } else {
 #pragma unroll
             for (int e = 0; e < E; ++e) { row.p[e] = 0; row.q[e] = 0; }
             if (i.flags & kSkip) return;
-            load_side(row.p, i.pptr, i.flags & 1u, lane);
-            load_side(row.q, i.qptr, i.flags & 2u, lane);
+            load_side(row.p, i.pptr, i.flags & 1u, lane, !(i.thin & 1u));
+            load_side(row.q, i.qptr, i.flags & 2u, lane, !(i.thin & 2u));
         }
     }
     __device__ __forceinline__ void forward(Row& nxt, const Info& in, const Row& cur, const Info& ic) const
@@ -243,10 +244,8 @@ template <int K, bool COH> struct MascotRule {
             const HV ruv = splat(r_h - dot);
             const HV gp = ruv * Q - lam_h * P;
             const HV gq = ruv * P - lam_h * Q;
-            row.p[0] = bits(HV(__builtin_elementwise_fma(lr_h, gp, P)));
-            row.q[0] = bits(HV(__builtin_elementwise_fma(lr_h, gq, Q)));
-            store_side(row.p, i.pptr, false, lane);
-            store_side(row.q, i.qptr, false, lane);
+            if (!(i.thin & 1u)) { row.p[0] = bits(HV(__builtin_elementwise_fma(lr_h, gp, P))); store_side(row.p, i.pptr, false, lane); }
+            if (!(i.thin & 2u)) { row.q[0] = bits(HV(__builtin_elementwise_fma(lr_h, gq, Q))); store_side(row.q, i.qptr, false, lane); }
             if (sampled) {
                 float g[E];
 #pragma unroll
@@ -273,12 +272,16 @@ template <int K, bool COH> struct MascotRule {
                 np_[e] = __builtin_fmaf(lrate, gp[e], pf[e]);
                 nq_[e] = __builtin_fmaf(lrate, gq[e], qf[e]);
             }
-            if (up) { for (int e = 0; e < E; ++e) row.p[e] = bits(np_[e]); }
-            else row.p[0] = bits(narrow(np_));
-            if (ip) { for (int e = 0; e < E; ++e) row.q[e] = bits(nq_[e]); }
-            else row.q[0] = bits(narrow(nq_));
-            store_side(row.p, i.pptr, up, lane);
-            store_side(row.q, i.qptr, ip, lane);
+            if (!(i.thin & 1u)) {
+                if (up) { for (int e = 0; e < E; ++e) row.p[e] = bits(np_[e]); }
+                else row.p[0] = bits(narrow(np_));
+                store_side(row.p, i.pptr, up, lane);
+            }
+            if (!(i.thin & 2u)) {
+                if (ip) { for (int e = 0; e < E; ++e) row.q[e] = bits(nq_[e]); }
+                else row.q[0] = bits(narrow(nq_));
+                store_side(row.q, i.qptr, ip, lane);
+            }
             if (sampled) {
                 if (!up) sample(gp, ug, unorm_s, grad_sum_p, ugrad_s);
                 if (!ip) sample(gq, ig, inorm_s, grad_sum_q, igrad_s);

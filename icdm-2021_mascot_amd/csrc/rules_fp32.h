@@ -15,7 +15,7 @@ template <int K> struct DenseRow {
     static constexpr int E = K / 64;
     float p[E], q[E];
 };
-struct DenseInfo { float r; uint32_t u, v; };
+struct DenseInfo { float r; uint32_t u, v, thin; };
 struct NoPrep {};
 
 template <int K, bool COH> struct DenseBase {
@@ -36,6 +36,7 @@ template <int K, bool COH> struct DenseBase {
         i.r = bcast(my.r, j);
         i.u = bcast(my.u, j);
         i.v = bcast(my.v, j);
+        i.thin = bcast(my.thin, j);
         return i;
     }
     template <int CLS> __device__ __forceinline__ void load(Row& row, const Info& i) const
@@ -43,14 +44,20 @@ template <int K, bool COH> struct DenseBase {
         const float* pp = P + (size_t)i.u * K + lane;
         const float* qq = Q + (size_t)i.v * K + lane;
 #pragma unroll
-        for (int e = 0; e < E; ++e) { row.p[e] = row_load<COH>(pp + 64 * e); row.q[e] = row_load<COH>(qq + 64 * e); }
+        for (int e = 0; e < E; ++e) { row.p[e] = row_load<COH>(pp + 64 * e, !(i.thin & 1u)); row.q[e] = row_load<COH>(qq + 64 * e, !(i.thin & 2u)); }
     }
     __device__ __forceinline__ void store(const Row& row, const Info& i) const
     {
         float* pp = P + (size_t)i.u * K + lane;
         float* qq = Q + (size_t)i.v * K + lane;
+        if (!(i.thin & 1u)) {
 #pragma unroll
-        for (int e = 0; e < E; ++e) { row_store<COH>(pp + 64 * e, row.p[e]); row_store<COH>(qq + 64 * e, row.q[e]); }
+            for (int e = 0; e < E; ++e) row_store<COH>(pp + 64 * e, row.p[e]);
+        }
+        if (!(i.thin & 2u)) {
+#pragma unroll
+            for (int e = 0; e < E; ++e) row_store<COH>(qq + 64 * e, row.q[e]);
+        }
     }
     __device__ __forceinline__ void forward(Row& nxt, const Info& in, const Row& cur, const Info& ic) const
     {
@@ -103,8 +110,10 @@ template <int K, bool COH> struct SgdRule : DenseBase<K, COH> {
 #pragma unroll
         for (int e = 0; e < E; ++e) {
             const float pe = row.p[e], qe = row.q[e];
-            row.p[e] = pe + lrate * (ruv * qe - lambda * pe);
-            row.q[e] = qe + lrate * (ruv * pe - lambda * qe);
+            const float pn = pe + lrate * (ruv * qe - lambda * pe);
+            const float qn = qe + lrate * (ruv * pe - lambda * qe);
+            row.p[e] = (i.thin & 1u) ? pe : pn;
+            row.q[e] = (i.thin & 2u) ? qe : qn;
         }
         this->store(row, i);
     }
@@ -142,8 +151,10 @@ template <int K, bool COH> struct MptRule : DenseBase<K, COH> {
         for (int e = 0; e < E; ++e) {
             const half_t gp = ruv * qh[e] - lambda_h * ph[e];
             const half_t gq = ruv * ph[e] - lambda_h * qh[e];
-            row.p[e] = row.p[e] + (lrate * (scaling_factor_rev * (float)gp));
-            row.q[e] = row.q[e] + (lrate * (scaling_factor_rev * (float)gq));
+            const float pn = row.p[e] + (lrate * (scaling_factor_rev * (float)gp));
+            const float qn = row.q[e] + (lrate * (scaling_factor_rev * (float)gq));
+            row.p[e] = (i.thin & 1u) ? row.p[e] : pn;
+            row.q[e] = (i.thin & 2u) ? row.q[e] : qn;
         }
         this->store(row, i);
     }

@@ -116,6 +116,38 @@ int dense_rmse(Common& c, const float* d_p, const float* d_q, double* out)
     return finish_rmse(c, out);
 }
 
+// Hot-row thinning table from rating counts: a row with count c has about F*c/n updates in flight
+// (F = resident workers x ratings a worker keeps in flight); keep = min(1, inflight_cap / that).
+std::vector<uint8_t> keep_table(const uint32_t* cnt, uint32_t rows, uint32_t n, uint32_t num_workers, float inflight_cap)
+{
+    const double resident = num_workers < 8192u ? num_workers : 8192u;      // 256 CUs x 32 wavefronts
+    const double F = resident * 4.0;                                         // three ratings of look-ahead
+    std::vector<uint8_t> t(rows);
+    for (uint32_t r = 0; r < rows; ++r) {
+        const double inflight = F * (double)cnt[r] / (double)n;
+        double keep = inflight > inflight_cap ? inflight_cap / inflight : 1.0;
+        int v = (int)std::floor(keep * 256.0) - 1;
+        t[r] = (uint8_t)(v < 0 ? 0 : (v > 255 ? 255 : v));
+    }
+    return t;
+}
+
+struct ThinningGuard {
+    DevBuf u, v;
+    bool active = false;
+    ~ThinningGuard() { if (active) (void)mf_set_hot_row_thinning(nullptr, nullptr); }
+    int install(const std::vector<uint8_t>& ku, const std::vector<uint8_t>& kv)
+    {
+        MF_TRY(u.alloc(ku.size(), "hipMalloc(user keep table)"));
+        MF_TRY(v.alloc(kv.size(), "hipMalloc(item keep table)"));
+        HIP_TRY(hipMemcpy(u.p, ku.data(), ku.size(), hipMemcpyHostToDevice), "H2D user keep table");
+        HIP_TRY(hipMemcpy(v.p, kv.data(), kv.size(), hipMemcpyHostToDevice), "H2D item keep table");
+        MF_TRY(mf_set_hot_row_thinning(u.as<uint8_t>(), v.as<uint8_t>()));
+        active = true;
+        return 0;
+    }
+};
+
 // ---- variants over dense fp32 P/Q (versions 2..5) ----------------------------------------------
 int train_dense(Common& c, float* p, float* q)
 {
@@ -155,6 +187,20 @@ int train_dense(Common& c, float* p, float* q)
         muppet_first_sample = c.update_count * c.update_vector_size - (uint32_t)sample_ratings_num;
     }
 
+    ThinningGuard thinning;
+    if (prm.hot_row_inflight > 0 && (version == 5 || version == 4)) {
+        DevBuf d_ucnt, d_icnt;
+        MF_TRY(d_ucnt.alloc((size_t)c.n_users * 4, "hipMalloc(user counts)"));
+        MF_TRY(d_icnt.alloc((size_t)c.n_items * 4, "hipMalloc(item counts)"));
+        HIP_TRY(hipMemset(d_ucnt.p, 0, (size_t)c.n_users * 4), "memset");
+        HIP_TRY(hipMemset(d_icnt.p, 0, (size_t)c.n_items * 4), "memset");
+        MF_TRY(mf_user_item_histogram(c.d_R.as<mf_node>(), c.n, d_ucnt.as<uint32_t>(), d_icnt.as<uint32_t>(), nullptr));
+        std::vector<uint32_t> ucnt(c.n_users), icnt(c.n_items);
+        HIP_TRY(hipMemcpy(ucnt.data(), d_ucnt.p, (size_t)c.n_users * 4, hipMemcpyDeviceToHost), "D2H user counts");
+        HIP_TRY(hipMemcpy(icnt.data(), d_icnt.p, (size_t)c.n_items * 4, hipMemcpyDeviceToHost), "D2H item counts");
+        MF_TRY(thinning.install(keep_table(ucnt.data(), c.n_users, c.n, prm.num_workers, prm.hot_row_inflight),
+                                keep_table(icnt.data(), c.n_items, c.n, prm.num_workers, prm.hot_row_inflight)));
+    }
     Timer t;
     const mf_node* R = c.d_R.as<mf_node>();
     for (uint32_t e = 0; e < prm.epoch; ++e) {
@@ -370,6 +416,11 @@ int train_mascot(Common& c, float* p, float* q)
                                            d_i2s.as<uint32_t>(), (int)c.k, c.n_items, I.groups, nullptr));
         HIP_TRY(hipDeviceSynchronize(), "synchronize");
     }
+    ThinningGuard thinning;
+    if (prm.hot_row_inflight > 0) {      // rows are in popularity-sorted order: the sorted counts index them directly
+        MF_TRY(thinning.install(keep_table(U.sorted_cnt.data(), c.n_users, c.n, prm.num_workers, prm.hot_row_inflight),
+                                keep_table(I.sorted_cnt.data(), c.n_items, c.n, prm.num_workers, prm.hot_row_inflight)));
+    }
     if (c.rep) c.rep->preprocess_ms = now_ms() - pre0;
 
     const uint32_t start_idx = 5;                                   // mf_methods.cu:110
@@ -457,6 +508,7 @@ void mf_default_params(mf_params* out)       // main.cu:19-32
     out->lambda = 0.015f; out->learning_rate = 0.01f; out->decay = 0.1f; out->sample_ratio = 0.01f; out->error_threshold = 0.001f;
     out->k = 128; out->epoch = 50; out->num_workers = 2048; out->thread_block_size = 128;
     out->user_group_num = 10; out->item_group_num = 10; out->version = 7; out->interval = 1; out->seed = 1;
+    out->hot_row_inflight = 16.0f;      // no reference counterpart: see mf_set_hot_row_thinning
 }
 
 uint32_t mf_group_end_indices(const uint32_t* sorted_cnt, uint32_t n, uint32_t requested_groups, uint32_t* end_idx_out)

@@ -221,3 +221,72 @@ def test_argument_errors_launch_nothing():
         h.mf_single_sgd_hogwild(1, 1, 1, 1, 32, 1, 1, 1, LR, LAM, 0, 0, None, None)
     with pytest.raises(MfError, match="empty rating array"):
         h.mf_single_sgd_hogwild(None, 0, 1, 1, 64, 1, 1, 1, LR, LAM, 0, 0, None, None)
+
+
+@pytest.mark.parametrize("k", [64, 128])
+@pytest.mark.parametrize("variant", ["single", "mascot"])
+def test_hot_row_thinning_drops_whole_row_updates(orc, k, variant):
+    """mf_set_hot_row_thinning: keep = 255 changes nothing; keep = 63 carries out a quarter of a row's updates,
+    a skipped row is left untouched while the other side of the rating is updated exactly as without thinning."""
+    import torch
+    h = mfutil.hip()
+    n = 4096
+    rng = np.random.default_rng(123 + k)
+    R = np.zeros(n, mfutil.NODE)
+    R["u"], R["i"], R["r"] = np.arange(n), rng.permutation(n), rng.integers(1, 6, n)      # every row is touched exactly once
+    P0 = (rng.standard_normal((n, k)) * 0.1).astype(np.float32)
+    Q0 = (rng.standard_normal((n, k)) * 0.1).astype(np.float32)
+    starts = np.arange(0, n, 128, dtype=np.uint32).reshape(-1, 1)          # one worker, consecutive windows
+    uc = starts.shape[0]
+    if variant == "mascot":
+        P0, Q0 = orc.h2f(orc.f2h(P0)), orc.h2f(orc.f2h(Q0))
+        end = np.array([n - 1], np.uint32)
+
+    def run(keep_u, keep_v):
+        dR, dS = to_dev(R), to_dev(starts)
+        ku = torch.full((n,), keep_u, dtype=torch.uint8, device="cuda")
+        kv = torch.full((n,), keep_v, dtype=torch.uint8, device="cuda")
+        h.mf_set_hot_row_thinning(ku.data_ptr(), kv.data_ptr())
+        try:
+            if variant == "single":
+                dP, dQ = to_dev(P0), to_dev(Q0)
+                h.mf_single_sgd_hogwild(dR.data_ptr(), n, dP.data_ptr(), dQ.data_ptr(), k, 1, uc, 128, LR, LAM, 5, 0, dS.data_ptr(), mfutil.stream_ptr())
+                torch.cuda.synchronize()
+                return from_dev(dP, np.float32, P0.shape), from_dev(dQ, np.float32, Q0.shape)
+            gp = mfutil.host_grouped(orc, k, P0, end, np.zeros(1, np.uint8))
+            gq = mfutil.host_grouped(orc, k, Q0, end, np.zeros(1, np.uint8))
+            dp, dq = mfutil.DeviceGrouped(gp), mfutil.DeviceGrouped(gq)
+            z = torch.zeros(4 * k + 16, dtype=torch.float32, device="cuda")
+            h.mf_mascot_sgd_hogwild(dR.data_ptr(), n, dp.ptrs.data_ptr(), dq.ptrs.data_ptr(), k, 1, uc, 128, LR, LAM,
+                                    dp.end.data_ptr(), dq.end.data_ptr(), dp.prec.data_ptr(), dq.prec.data_ptr(),
+                                    z.data_ptr(), z[k:].data_ptr(), z[2 * k:].data_ptr(), z[3 * k:].data_ptr(),
+                                    uc * 128, 1, 1, 5, 0, dS.data_ptr(), mfutil.stream_ptr())
+            torch.cuda.synchronize()
+            return orc.h2f(dp.download()[0]).reshape(n, k), orc.h2f(dq.download()[0]).reshape(n, k)
+        finally:
+            torch.cuda.synchronize()
+            h.mf_set_hot_row_thinning(None, None)
+
+    # the checker's result with every update carried out
+    if variant == "single":
+        Pw, Qw = P0.copy(), Q0.copy()
+        orc.lib.orc_sgd_epoch(k, R.ctypes.data, n, Pw.ctypes.data, Qw.ctypes.data, 1, uc, 128, LR, LAM, 5, 0, starts.ctypes.data, 1)
+    else:
+        gp = mfutil.host_grouped(orc, k, P0, end, np.zeros(1, np.uint8))
+        gq = mfutil.host_grouped(orc, k, Q0, end, np.zeros(1, np.uint8))
+        z = [np.zeros(k, np.float32) for _ in range(4)]
+        orc.lib.orc_mascot_epoch(k, R.ctypes.data, n, gp.ptrs, gq.ptrs, gp.end_idx.ctypes.data, gq.end_idx.ctypes.data,
+                                 gp.prec.ctypes.data, gq.prec.ctypes.data, 1, 1, 1, uc, 128, LR, LAM, uc * 128,
+                                 z[0].ctypes.data, z[1].ctypes.data, z[2].ctypes.data, z[3].ctypes.data, 5, 0, starts.ctypes.data, 1)
+        Pw, Qw = orc.h2f(gp.arrays[0]).reshape(n, k), orc.h2f(gq.arrays[0]).reshape(n, k)
+    P1, Q1 = run(255, 255)
+    assert np.array_equal(P1, Pw) and np.array_equal(Q1, Qw)
+    P2, Q2 = run(63, 255)
+    assert np.array_equal(Q2, Qw)                                   # item side: every update, computed from the old user row
+    changed = np.any(P2 != P0, axis=1)
+    assert np.array_equal(P2[changed], Pw[changed])                 # a user row is either untouched or fully updated
+    assert np.array_equal(P2[~changed], P0[~changed])
+    assert 0.20 < changed.mean() < 0.30                             # (63+1)/256 of the updates
+    P3, Q3 = run(255, 0)
+    assert np.array_equal(P3, Pw)
+    assert np.any(Q3 != Q0, axis=1).mean() < 0.02                   # (0+1)/256
