@@ -215,6 +215,23 @@ def cpu_baseline(prob, cfg, seed, threads, target_updates):
     return done / dt, done, dt
 
 
+def measured_traffic(a, leg):
+    """HBM bytes per launch of a plain epoch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch, scaled by
+    2.0 / 1.0, the factors a 1 GiB device copy gives; summaries under profiles/).  Counters cannot be read from inside
+    this process, so the figures are the profiled ones and only reported for the exact workload they were taken on."""
+    if a.ratings != 100_000_000 or a.seed != 2021:
+        return None
+    if a.skip_coherent:
+        return (13_986_844 * 2.0 + 24_179_238) * 1024 if leg["workers"] == 16384 else None
+    if leg["workers"] != 2048:
+        return None
+    if a.hot_row_inflight == 16.0:
+        return (19_663_594 * 2.0 + 37_531_052) * 1024
+    if a.hot_row_inflight == 0.0:
+        return (23_408_594 * 2.0 + 50_072_631) * 1024
+    return None
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -249,7 +266,9 @@ def main():
     del R
     torch.cuda.synchronize()
     setup_s = time.perf_counter() - t0
-    bytes_per_update = 12 + 2 * k * (2 + 2)          # all groups still binary16 in the measured epochs: 1036 B
+    # All groups are still binary16 in the measured epochs: a rating reads 12 B and two 256 B rows, and writes the
+    # two rows back (1036 B) unless hot-row thinning skips a write (then that row is read only).
+    read_bytes, row_bytes = 12 + 2 * k * 2, 2 * k * 2
 
     def leg(coherent, W, inflight_cap=0.0):
         h.mf_set_row_coherence(1 if coherent else 0)
@@ -259,9 +278,10 @@ def main():
         prob.set_thinning(W, 0.0)
         updates = W * uc * 128
         ms = float(per.mean())
+        bytes_per_update = read_bytes + row_bytes * kept
         return dict(ms_per_step=ms, ms_steps=[round(float(x), 3) for x in per], wall_s=wall, updates_per_step=updates,
                     ratings_per_s=a.ratings / (ms / 1e3), gbs=updates * bytes_per_update / (ms / 1e3) / 1e9, workers=W,
-                    rmse=rmse, row_updates_kept=kept)
+                    rmse=rmse, row_updates_kept=kept, bytes_per_update=bytes_per_update)
 
     if a.pmc_copy:
         src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
@@ -287,8 +307,9 @@ def main():
                    "user_groups": int(prob.sides[0]["groups"]), "item_groups": int(prob.sides[1]["groups"]), "setup_s": round(setup_s, 1)},
         "roofline": {"bound": "hbm", "achieved": main_leg["gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
                      "frac": main_leg["gbs"] / PEAK_HBM_GBS,
-                     "traffic": None,
-                     "kernel": "hogwild_kernel<MascotRule<128,true>>", "bytes_per_update": bytes_per_update,
+                     "traffic": measured_traffic(a, main_leg),
+                     "kernel": "hogwild_kernel<MascotRule<128,%s>>" % ("false" if a.skip_coherent else "true"),
+                     "bytes_per_update": round(main_leg["bytes_per_update"], 1),
                      "updates_per_launch": main_leg["updates_per_step"]},
         "ms_steps": main_leg["ms_steps"],
         "test_rmse_after_timed_epochs": {"value": main_leg["rmse"], "epochs": a.warmup + a.steps, "test_ratings": n_test},
