@@ -116,7 +116,9 @@ class MascotProblem:
             s["arena"].copy_(s["initial"])
 
     def set_thinning(self, W, inflight_cap):
-        """Hot-row thinning tables from the rating counts (rows are in popularity-sorted order), as mf_train builds them."""
+        """Hot-row tables from the rating counts (rows are in popularity-sorted order), as mf_train builds them:
+        255 = ordinary row; rows with more than one update in flight are hot rows (updates added in memory), thinned to
+        at most `inflight_cap` updates in flight."""
         torch, h = self.torch, self.h
         if not inflight_cap:
             h.mf_set_hot_row_thinning(None, None)
@@ -127,8 +129,8 @@ class MascotProblem:
         for s in self.sides:
             inflight = F * s["sorted_cnt"].astype(np.float64) / self.n
             keep = np.where(inflight > inflight_cap, inflight_cap / np.maximum(inflight, 1e-30), 1.0)
-            t = np.clip(np.floor(keep * 256.0) - 1, 0, 255).astype(np.uint8)
-            kept += float((s["sorted_cnt"].astype(np.float64) * (t.astype(np.float64) + 1) / 256.0).sum()) / self.n
+            t = np.where(inflight > 1.0, np.clip(np.floor(keep * 255.0) - 1, 0, 254), 255).astype(np.uint8)
+            kept += float((s["sorted_cnt"].astype(np.float64) * np.where(t == 255, 1.0, (t.astype(np.float64) + 1) / 255.0)).sum()) / self.n
             tabs.append(torch.from_numpy(t).to(self.R.device))
         self.keep = tabs
         h.mf_set_hot_row_thinning(tabs[0].data_ptr(), tabs[1].data_ptr())

@@ -99,8 +99,10 @@ __global__ __launch_bounds__(kMaxBlock) void hogwild_kernel(Schedule s, typename
                 x = load_rating(s.R, idx);
                 if (s.keep_u) {
                     const uint32_t rnd = (uint32_t)(mix64(s.epoch_key ^ (((uint64_t)idx << 20) ^ (uint64_t)wid ^ 0x7468696eull)) >> 40);
-                    if ((rnd & 255u) > (uint32_t)s.keep_u[x.u]) x.thin |= 1u;
-                    if (((rnd >> 8) & 255u) > (uint32_t)s.keep_v[x.v]) x.thin |= 2u;
+                    const uint32_t ku = s.keep_u[x.u], kv = s.keep_v[x.v];
+                    // two independent draws, uniform over 0..254
+                    if (ku != 255u) x.thin |= (((rnd & 0xfffu) * 255u) >> 12) > ku ? 5u : 4u;
+                    if (kv != 255u) x.thin |= (((rnd >> 12) * 255u) >> 12) > kv ? 10u : 8u;
                 }
             }
             return x;

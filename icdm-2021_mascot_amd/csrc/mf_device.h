@@ -92,29 +92,34 @@ __device__ __forceinline__ uint64_t bcast(uint64_t v, int lane)
 }
 
 // ---- device-coherent row accesses -----------------------------------------------------------
-// MI355X has one L2 per XCD and the L2s do not snoop each other for ordinary loads and stores: a row
-// cached in one XCD's L2 would not see the updates other XCDs make to it during the same kernel, and
-// each XCD would train its own private copy of every hot row.  Hogwild needs the opposite (the latest
-// value any worker wrote), so P and Q rows are read and written with agent-scope relaxed atomics: plain
-// global_load/global_store instructions with the sc1 cache policy, no fences and no read-modify-write.
+// MI355X has one L2 per XCD, and a row written with an ordinary store stays in the writing XCD's L2:
+// the other XCDs keep reading (and training) their own copies of every hot row for as long as those stay
+// cached.  Hogwild needs the opposite (the latest value any worker wrote), so with COH = true P and Q
+// rows are written with agent-scope relaxed atomic stores: plain global_store instructions with the sc1
+// cache policy, which write through to the memory side and drop the copies other L2s hold.  Loads stay
+// ordinary cached loads (measured: agent-scope loads add a third to the epoch and change nothing in the
+// convergence once the stores are coherent).
 //
-// The price: every access to a row goes to the memory side, and all accesses to one row serialise
-// there.  With a row that takes a large share of all ratings (Zipf-like synthetic data) that single row
-// bounds the epoch.  COH = false keeps ordinary cached accesses instead: each XCD then works on its own
+// The price: every store goes to the memory side, and all stores to one row serialise there.  With a row
+// that takes a large share of all ratings that single row bounds the epoch; see Schedule::keep_u for what
+// is done about it.  COH = false keeps ordinary write-back stores: each XCD then works on its own
 // L2-resident copy of a hot row between evictions (a row that is not re-used while cached behaves the
 // same either way).  The host picks per run (mf_set_row_coherence).
-// `coherent == false` (a thinned access, see Schedule::keep_u) falls back to the cached path.
-template <bool COH, class T> __device__ __forceinline__ T row_load(const T* p, bool coherent = true)
-{
-    if constexpr (COH) {
-        if (coherent) return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        return *p;
-    } else return *p;
-}
+template <class T> __device__ __forceinline__ T row_load(const T* p) { return *p; }
 template <bool COH, class T> __device__ __forceinline__ void row_store(T* p, T v)
 {
     if constexpr (COH) __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     else *p = v;
+}
+// Aggregated update of a hot row (Schedule::keep_u): the change is added in memory, so concurrent updates
+// of the row add up instead of overwriting each other.
+__device__ __forceinline__ void row_add(float* p, float d)
+{
+    (void)__hip_atomic_fetch_add(p, d, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void row_add(half2_t* p, half2_t d)
+{
+    (void)__builtin_amdgcn_global_atomic_fadd_v2f16((__attribute__((address_space(1))) half2_t*)p, d);
 }
 
 // ---- counter-based generator -----------------------------------------------------------
@@ -152,17 +157,19 @@ struct Schedule {
     uint32_t range_begin, range_end;   // processed-index range [begin, end) every worker handles in this launch
     uint64_t epoch_key;
     const uint32_t* window_start;   // optional [update_count][num_workers]
-    // Hot-row thinning (optional, both null = off).  keep_u[row] / keep_v[row] in 0..255: the update of
-    // that row is carried out with probability (keep+1)/256; otherwise the row is only read (through the
-    // caches) for the other side's update and is not written.  Under Hogwild a row with C updates in
-    // flight keeps one of them anyway; thinning such rows to about one update in flight removes the
-    // wasted traffic, which with device-coherent rows is what serialises at the memory side.
+    // Hot rows (optional, both null = off).  keep_u[row] / keep_v[row] in 0..255; 255 = an ordinary row.
+    // A row with a smaller value is a hot row: its update is carried out with probability (keep+1)/255,
+    // otherwise the row is only read for the other side's update; and an update that is carried out adds
+    // its change to the row in memory (row_add) instead of storing the new row.  Under last-writer-wins a
+    // row with C updates in flight keeps one of them; adding keeps them all, and thinning bounds C (the
+    // sum of C stale gradients is a mini-batch step C times as long) and the stores that serialise at
+    // the memory side.
     const uint8_t* keep_u;
     const uint8_t* keep_v;
 };
 
 // One lane's rating of a 64-rating chunk; the stream is read once per epoch, so bypass-style loads.
-struct Rating { float r; uint32_t u; uint32_t v; uint32_t thin; };   // thin: bit0 skip the P update, bit1 skip the Q update
+struct Rating { float r; uint32_t u; uint32_t v; uint32_t thin; };   // thin: bit0/bit1 skip the P/Q update, bit2/bit3 the P/Q row is a hot row (updates are added)
 __device__ __forceinline__ Rating load_rating(const mf_node* R, uint32_t idx)
 {
     const uint32_t* w = reinterpret_cast<const uint32_t*>(R + idx);

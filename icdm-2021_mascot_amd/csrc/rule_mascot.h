@@ -131,19 +131,36 @@ template <int K, bool COH> struct MascotRule {
         return i;
     }
 
-    static __device__ __forceinline__ void load_side(uint32_t* r, uint64_t ptr, bool fp32, int lane, bool coh)
+    static __device__ __forceinline__ void load_side(uint32_t* r, uint64_t ptr, bool fp32, int lane)
     {
         if (fp32) {
             if constexpr (E == 2) {
-                const uint64_t v = row_load<COH>(reinterpret_cast<const uint64_t*>(ptr + (uint64_t)lane * 8), coh);
+                const uint64_t v = row_load(reinterpret_cast<const uint64_t*>(ptr + (uint64_t)lane * 8));
                 r[0] = (uint32_t)v; r[1] = (uint32_t)(v >> 32);
             } else {
-                r[0] = row_load<COH>(reinterpret_cast<const uint32_t*>(ptr + (uint64_t)lane * 4), coh);
+                r[0] = row_load(reinterpret_cast<const uint32_t*>(ptr + (uint64_t)lane * 4));
             }
         } else {
-            if constexpr (E == 2) r[0] = row_load<COH>(reinterpret_cast<const uint32_t*>(ptr + (uint64_t)lane * 4), coh);
-            else r[0] = row_load<COH>(reinterpret_cast<const uint16_t*>(ptr + (uint64_t)lane * 2), coh);
+            if constexpr (E == 2) r[0] = row_load(reinterpret_cast<const uint32_t*>(ptr + (uint64_t)lane * 4));
+            else r[0] = row_load(reinterpret_cast<const uint16_t*>(ptr + (uint64_t)lane * 2));
         }
+    }
+    // hot row (Schedule::keep_u): add the change of this lane's elements to the row in memory
+    static __device__ __forceinline__ void add_side_half(uint64_t ptr, HV d, int lane)
+    {
+        if constexpr (E == 2) {
+            row_add(reinterpret_cast<half2_t*>(ptr + (uint64_t)lane * 4), d);
+        } else {
+            // one element per lane: even lanes add the pair (own, right neighbour)
+            const uint32_t mine = (uint32_t)bits(d);
+            const uint32_t other = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)mine, 0xB1 /* quad_perm 1,0,3,2 */, 0xf, 0xf, false);
+            if (!(lane & 1)) row_add(reinterpret_cast<half2_t*>(ptr + (uint64_t)lane * 2), from_bits<half2_t>(mine | (other << 16)));
+        }
+    }
+    static __device__ __forceinline__ void add_side_float(uint64_t ptr, const float* d, int lane)
+    {
+#pragma unroll
+        for (int e = 0; e < E; ++e) row_add(reinterpret_cast<float*>(ptr + (uint64_t)lane * (4 * E)) + e, d[e]);
     }
     static __device__ __forceinline__ void store_side(const uint32_t* r, uint64_t ptr, bool fp32, int lane)
     {
@@ -158,14 +175,14 @@ template <int K, bool COH> struct MascotRule {
     template <int CLS> __device__ __forceinline__ void load(Row& row, const Info& i) const
     {
         if constexpr (CLS == 1) {
-            load_side(row.p, i.pptr, false, lane, !(i.thin & 1u));
-            load_side(row.q, i.qptr, false, lane, !(i.thin & 2u));
+            load_side(row.p, i.pptr, false, lane);
+            load_side(row.q, i.qptr, false, lane);
         } else {
 #pragma unroll
             for (int e = 0; e < E; ++e) { row.p[e] = 0; row.q[e] = 0; }
             if (i.flags & kSkip) return;
-            load_side(row.p, i.pptr, i.flags & 1u, lane, !(i.thin & 1u));
-            load_side(row.q, i.qptr, i.flags & 2u, lane, !(i.thin & 2u));
+            load_side(row.p, i.pptr, i.flags & 1u, lane);
+            load_side(row.q, i.qptr, i.flags & 2u, lane);
         }
     }
     __device__ __forceinline__ void forward(Row& nxt, const Info& in, const Row& cur, const Info& ic) const
@@ -244,8 +261,14 @@ template <int K, bool COH> struct MascotRule {
             const HV ruv = splat(r_h - dot);
             const HV gp = ruv * Q - lam_h * P;
             const HV gq = ruv * P - lam_h * Q;
-            if (!(i.thin & 1u)) { row.p[0] = bits(HV(__builtin_elementwise_fma(lr_h, gp, P))); store_side(row.p, i.pptr, false, lane); }
-            if (!(i.thin & 2u)) { row.q[0] = bits(HV(__builtin_elementwise_fma(lr_h, gq, Q))); store_side(row.q, i.qptr, false, lane); }
+            if (!(i.thin & 1u)) {
+                row.p[0] = bits(HV(__builtin_elementwise_fma(lr_h, gp, P)));
+                if (i.thin & 4u) add_side_half(i.pptr, lr_h * gp, lane); else store_side(row.p, i.pptr, false, lane);
+            }
+            if (!(i.thin & 2u)) {
+                row.q[0] = bits(HV(__builtin_elementwise_fma(lr_h, gq, Q)));
+                if (i.thin & 8u) add_side_half(i.qptr, lr_h * gq, lane); else store_side(row.q, i.qptr, false, lane);
+            }
             if (sampled) {
                 float g[E];
 #pragma unroll
@@ -275,12 +298,20 @@ template <int K, bool COH> struct MascotRule {
             if (!(i.thin & 1u)) {
                 if (up) { for (int e = 0; e < E; ++e) row.p[e] = bits(np_[e]); }
                 else row.p[0] = bits(narrow(np_));
-                store_side(row.p, i.pptr, up, lane);
+                if (i.thin & 4u) {
+                    float d[E];
+                    for (int e = 0; e < E; ++e) d[e] = lrate * gp[e];
+                    if (up) add_side_float(i.pptr, d, lane); else add_side_half(i.pptr, narrow(d), lane);
+                } else store_side(row.p, i.pptr, up, lane);
             }
             if (!(i.thin & 2u)) {
                 if (ip) { for (int e = 0; e < E; ++e) row.q[e] = bits(nq_[e]); }
                 else row.q[0] = bits(narrow(nq_));
-                store_side(row.q, i.qptr, ip, lane);
+                if (i.thin & 8u) {
+                    float d[E];
+                    for (int e = 0; e < E; ++e) d[e] = lrate * gq[e];
+                    if (ip) add_side_float(i.qptr, d, lane); else add_side_half(i.qptr, narrow(d), lane);
+                } else store_side(row.q, i.qptr, ip, lane);
             }
             if (sampled) {
                 if (!up) sample(gp, ug, unorm_s, grad_sum_p, ugrad_s);

@@ -44,8 +44,23 @@ template <int K, bool COH> struct DenseBase {
         const float* pp = P + (size_t)i.u * K + lane;
         const float* qq = Q + (size_t)i.v * K + lane;
 #pragma unroll
-        for (int e = 0; e < E; ++e) { row.p[e] = row_load<COH>(pp + 64 * e, !(i.thin & 1u)); row.q[e] = row_load<COH>(qq + 64 * e, !(i.thin & 2u)); }
+        for (int e = 0; e < E; ++e) { row.p[e] = row_load(pp + 64 * e); row.q[e] = row_load(qq + 64 * e); }
     }
+    // dp, dq: the change of each element (new - old as the rule computes it), added to a hot row
+    __device__ __forceinline__ void store(const Row& row, const Info& i, const float* dp, const float* dq) const
+    {
+        float* pp = P + (size_t)i.u * K + lane;
+        float* qq = Q + (size_t)i.v * K + lane;
+        if (!(i.thin & 1u)) {
+#pragma unroll
+            for (int e = 0; e < E; ++e) { if (i.thin & 4u) row_add(pp + 64 * e, dp[e]); else row_store<COH>(pp + 64 * e, row.p[e]); }
+        }
+        if (!(i.thin & 2u)) {
+#pragma unroll
+            for (int e = 0; e < E; ++e) { if (i.thin & 8u) row_add(qq + 64 * e, dq[e]); else row_store<COH>(qq + 64 * e, row.q[e]); }
+        }
+    }
+    // rules that keep last-writer-wins on every row
     __device__ __forceinline__ void store(const Row& row, const Info& i) const
     {
         float* pp = P + (size_t)i.u * K + lane;
@@ -107,15 +122,16 @@ template <int K, bool COH> struct SgdRule : DenseBase<K, COH> {
         for (int e = 0; e < E; ++e) m[e] = row.p[e] * row.q[e];
         const float dot = dot_reference_order<E, float>(m);
         const float ruv = i.r - dot;
+        float dp[E], dq[E];
 #pragma unroll
         for (int e = 0; e < E; ++e) {
             const float pe = row.p[e], qe = row.q[e];
-            const float pn = pe + lrate * (ruv * qe - lambda * pe);
-            const float qn = qe + lrate * (ruv * pe - lambda * qe);
-            row.p[e] = (i.thin & 1u) ? pe : pn;
-            row.q[e] = (i.thin & 2u) ? qe : qn;
+            dp[e] = lrate * (ruv * qe - lambda * pe);
+            dq[e] = lrate * (ruv * pe - lambda * qe);
+            row.p[e] = (i.thin & 1u) ? pe : pe + dp[e];
+            row.q[e] = (i.thin & 2u) ? qe : qe + dq[e];
         }
-        this->store(row, i);
+        this->store(row, i, dp, dq);
     }
     __device__ __forceinline__ void finish(const Params&, uint32_t) const {}
 };
@@ -147,16 +163,17 @@ template <int K, bool COH> struct MptRule : DenseBase<K, COH> {
         for (int e = 0; e < E; ++e) { ph[e] = (half_t)row.p[e]; qh[e] = (half_t)row.q[e]; m[e] = ph[e] * qh[e]; }
         const half_t dot = dot_reference_order<E, half_t>(m);
         const half_t ruv = scaling_factor_h * (r_h - dot);
+        float dp[E], dq[E];
 #pragma unroll
         for (int e = 0; e < E; ++e) {
             const half_t gp = ruv * qh[e] - lambda_h * ph[e];
             const half_t gq = ruv * ph[e] - lambda_h * qh[e];
-            const float pn = row.p[e] + (lrate * (scaling_factor_rev * (float)gp));
-            const float qn = row.q[e] + (lrate * (scaling_factor_rev * (float)gq));
-            row.p[e] = (i.thin & 1u) ? row.p[e] : pn;
-            row.q[e] = (i.thin & 2u) ? row.q[e] : qn;
+            dp[e] = lrate * (scaling_factor_rev * (float)gp);
+            dq[e] = lrate * (scaling_factor_rev * (float)gq);
+            row.p[e] = (i.thin & 1u) ? row.p[e] : row.p[e] + dp[e];
+            row.q[e] = (i.thin & 2u) ? row.q[e] : row.q[e] + dq[e];
         }
-        this->store(row, i);
+        this->store(row, i, dp, dq);
     }
     __device__ __forceinline__ void finish(const Params&, uint32_t) const {}
 };

@@ -116,8 +116,9 @@ int dense_rmse(Common& c, const float* d_p, const float* d_q, double* out)
     return finish_rmse(c, out);
 }
 
-// Hot-row thinning table from rating counts: a row with count c has about F*c/n updates in flight
-// (F = resident workers x ratings a worker keeps in flight); keep = min(1, inflight_cap / that).
+// Hot-row table from rating counts (see mf_set_hot_row_thinning): a row with count c has about F*c/n updates in
+// flight (F = resident workers x ratings a worker keeps in flight).  Rows with more than one are hot rows (their
+// updates are added); of those, rows above inflight_cap are thinned to inflight_cap updates in flight.
 std::vector<uint8_t> keep_table(const uint32_t* cnt, uint32_t rows, uint32_t n, uint32_t num_workers, float inflight_cap)
 {
     const double resident = num_workers < 8192u ? num_workers : 8192u;      // 256 CUs x 32 wavefronts
@@ -125,9 +126,10 @@ std::vector<uint8_t> keep_table(const uint32_t* cnt, uint32_t rows, uint32_t n, 
     std::vector<uint8_t> t(rows);
     for (uint32_t r = 0; r < rows; ++r) {
         const double inflight = F * (double)cnt[r] / (double)n;
-        double keep = inflight > inflight_cap ? inflight_cap / inflight : 1.0;
-        int v = (int)std::floor(keep * 256.0) - 1;
-        t[r] = (uint8_t)(v < 0 ? 0 : (v > 255 ? 255 : v));
+        if (inflight <= 1.0) { t[r] = 255; continue; }
+        const double keep = inflight > inflight_cap ? inflight_cap / inflight : 1.0;
+        const int v = (int)std::floor(keep * 255.0) - 1;
+        t[r] = (uint8_t)(v < 0 ? 0 : (v > 254 ? 254 : v));
     }
     return t;
 }

@@ -55,14 +55,16 @@ int mf_get_row_coherence(void);
  * Default 1.  No counterpart in the reference. */
 int mf_set_epoch_splits(uint32_t splits);
 uint32_t mf_get_epoch_splits(void);
-/* Hot-row thinning for the fp32-SGD / MPT / MASCOT update calls (process-wide, both NULL = off, the default).
+/* Hot rows for the fp32-SGD / MPT / MASCOT update calls (process-wide, both NULL = off, the default).
  * user_keep[row], item_keep[row] are device arrays of bytes indexed like P and Q rows (for MASCOT: sorted row
- * order): a rating updates that row with probability (keep+1)/256; otherwise it only reads the row (through
- * the caches) for the other side's update and does not write it.  Meant for rows that take percents of all
- * ratings: under Hogwild a row with C updates in flight keeps one of them anyway, and with device-coherent
- * rows those C accesses serialise at the memory side.  mf_train builds the tables from the rating counts when
- * mf_params.hot_row_inflight > 0.  No counterpart in the reference.  The tables must stay valid while
- * launches that use them are in flight. */
+ * order).  255 marks an ordinary row.  A row with a smaller value is a hot row, meant for rows that have several
+ * updates in flight at any time: (1) a rating updates the row with probability (keep+1)/255 and otherwise only
+ * reads it for the other side's update; (2) an update that is carried out adds its change to the row in memory
+ * (an atomic add per element) instead of storing the new row, so concurrent updates add up where
+ * last-writer-wins would keep one of them.  The sum of C stale gradients is a step C times as long, which is why
+ * rows with many updates in flight are thinned.  mf_train builds the tables from the rating counts when
+ * mf_params.hot_row_inflight > 0 (MuPPET and AFP ignore them).  No counterpart in the reference.  The tables must
+ * stay valid while launches that use them are in flight. */
 int mf_set_hot_row_thinning(const uint8_t* user_keep, const uint8_t* item_keep);
 /* Number of per-block columns mf_mascot_sgd_hogwild writes into norm_sum_p / norm_sum_q
  * (the reference's `block_num`, mf_methods.cu:109). */
@@ -205,8 +207,8 @@ typedef struct {
     uint32_t verbose;         /* 1: print the reference's stdout lines (mf_methods.cu:396 etc.) */
     uint32_t cached_rows;     /* 0: device-coherent row accesses (default), 1: cached, see mf_set_row_coherence */
     uint32_t epoch_splits;    /* kernel launches per epoch, 0 or 1 = one, see mf_set_epoch_splits */
-    float hot_row_inflight;   /* > 0: thin the updates of rows expected to have more than this many updates in
-                                 flight (see mf_set_hot_row_thinning); 0 = off */
+    float hot_row_inflight;   /* > 0: rows expected to have more than one update in flight become hot rows, thinned
+                                 to at most this many updates in flight (see mf_set_hot_row_thinning); 0 = off */
 } mf_params;
 
 /* What a run reports back; every pointer is optional host memory owned by the caller. */

@@ -226,8 +226,10 @@ def test_argument_errors_launch_nothing():
 @pytest.mark.parametrize("k", [64, 128])
 @pytest.mark.parametrize("variant", ["single", "mascot"])
 def test_hot_row_thinning_drops_whole_row_updates(orc, k, variant):
-    """mf_set_hot_row_thinning: keep = 255 changes nothing; keep = 63 carries out a quarter of a row's updates,
-    a skipped row is left untouched while the other side of the rating is updated exactly as without thinning."""
+    """mf_set_hot_row_thinning: 255 = ordinary row, nothing changes; 254 = hot row, every update carried out (added
+    in memory: with one update per row the sum equals the stored row, up to the extra rounding of the binary16
+    change); 63 carries out a quarter of a row's updates, a skipped row is left untouched while the other side of
+    the rating is updated exactly as without thinning."""
     import torch
     h = mfutil.hip()
     n = 4096
@@ -279,14 +281,73 @@ def test_hot_row_thinning_drops_whole_row_updates(orc, k, variant):
                                  gp.prec.ctypes.data, gq.prec.ctypes.data, 1, 1, 1, uc, 128, LR, LAM, uc * 128,
                                  z[0].ctypes.data, z[1].ctypes.data, z[2].ctypes.data, z[3].ctypes.data, 5, 0, starts.ctypes.data, 1)
         Pw, Qw = orc.h2f(gp.arrays[0]).reshape(n, k), orc.h2f(gq.arrays[0]).reshape(n, k)
+    def same(got, want, old):
+        if variant == "single":                                     # fp32: old + change is the stored value
+            return np.array_equal(got, want)
+        # binary16: memory adds round(lr*g) to the row, the rule stores fma(lr, g, row); the extra rounding is the
+        # one of the change, so the two are within one ulp of the larger of the change and the result
+        scale = np.maximum(np.abs(want), np.abs(want - old)).astype(np.float16)
+        return np.all(np.abs(got.astype(np.float64) - want) <= np.spacing(scale).astype(np.float64))
+
     P1, Q1 = run(255, 255)
     assert np.array_equal(P1, Pw) and np.array_equal(Q1, Qw)
+    P4, Q4 = run(254, 254)
+    assert same(P4, Pw, P0) and same(Q4, Qw, Q0)
+    assert np.all(np.any(P4 != P0, axis=1)) and np.all(np.any(Q4 != Q0, axis=1))
     P2, Q2 = run(63, 255)
     assert np.array_equal(Q2, Qw)                                   # item side: every update, computed from the old user row
     changed = np.any(P2 != P0, axis=1)
-    assert np.array_equal(P2[changed], Pw[changed])                 # a user row is either untouched or fully updated
+    assert same(P2[changed], Pw[changed], P0[changed])                           # a user row is either untouched or fully updated
     assert np.array_equal(P2[~changed], P0[~changed])
-    assert 0.20 < changed.mean() < 0.30                             # (63+1)/256 of the updates
+    assert 0.20 < changed.mean() < 0.30                             # (63+1)/255 of the updates
     P3, Q3 = run(255, 0)
     assert np.array_equal(P3, Pw)
-    assert np.any(Q3 != Q0, axis=1).mean() < 0.02                   # (0+1)/256
+    assert np.any(Q3 != Q0, axis=1).mean() < 0.02                   # (0+1)/255
+
+
+@pytest.mark.parametrize("k", [64, 128])
+@pytest.mark.parametrize("variant", ["single", "mpt", "mascot"])
+def test_hot_row_updates_add_up(orc, k, variant):
+    """k wavefronts in k/4 workgroups update one hot item row at the same time.  User u's row is 0.5 * e_u, the item
+    row starts at zero and lambda is zero, so every update sees a zero dot product whatever the others have done
+    and adds lr * r_u * 0.5 to element u only: all k updates must land, exactly, in any order."""
+    import torch
+    h = mfutil.hip()
+    n, lr = k, 2.0 ** -6
+    rng = np.random.default_rng(7 + k)
+    R = np.zeros(n, mfutil.NODE)
+    R["u"], R["i"], R["r"] = rng.permutation(n), 0, rng.integers(1, 6, n)
+    P0 = (0.5 * np.eye(n, k)).astype(np.float32)
+    Q0 = np.zeros((1, k), np.float32)
+    starts = np.arange(n, dtype=np.uint32).reshape(1, n)            # n workers, one rating each
+    want = np.zeros(k, np.float32)
+    want[R["u"]] = lr * R["r"] * 0.5
+    dR, dS = to_dev(R), to_dev(starts)
+    ku = torch.full((n,), 255, dtype=torch.uint8, device="cuda")
+    kv = torch.full((1,), 254, dtype=torch.uint8, device="cuda")
+    h.mf_set_hot_row_thinning(ku.data_ptr(), kv.data_ptr())
+    try:
+        if variant == "mascot":
+            end_u, end_i = np.array([n - 1], np.uint32), np.array([0], np.uint32)
+            gp = mfutil.host_grouped(orc, k, P0, end_u, np.zeros(1, np.uint8))
+            gq = mfutil.host_grouped(orc, k, Q0, end_i, np.zeros(1, np.uint8))
+            dp, dq = mfutil.DeviceGrouped(gp), mfutil.DeviceGrouped(gq)
+            z = torch.zeros(4 * k + 4 * n, dtype=torch.float32, device="cuda")
+            h.mf_mascot_sgd_hogwild(dR.data_ptr(), n, dp.ptrs.data_ptr(), dq.ptrs.data_ptr(), k, n, 1, 1, lr, 0.0,
+                                    dp.end.data_ptr(), dq.end.data_ptr(), dp.prec.data_ptr(), dq.prec.data_ptr(),
+                                    z.data_ptr(), z[k:].data_ptr(), z[2 * k:].data_ptr(), z[2 * k + n:].data_ptr(),
+                                    1, 1, 1, 5, 0, dS.data_ptr(), mfutil.stream_ptr())
+            torch.cuda.synchronize()
+            got = orc.h2f(dq.download()[0]).reshape(k)
+        else:
+            dP, dQ = to_dev(P0), to_dev(Q0)
+            if variant == "single":
+                h.mf_single_sgd_hogwild(dR.data_ptr(), n, dP.data_ptr(), dQ.data_ptr(), k, n, 1, 1, lr, 0.0, 5, 0, dS.data_ptr(), mfutil.stream_ptr())
+            else:
+                h.mf_mpt_sgd_hogwild(dR.data_ptr(), n, dP.data_ptr(), dQ.data_ptr(), k, n, 1, 1, lr, 0, 1024.0, 5, 0, dS.data_ptr(), mfutil.stream_ptr())
+            torch.cuda.synchronize()
+            got = from_dev(dQ, np.float32, Q0.shape).reshape(k)
+    finally:
+        torch.cuda.synchronize()
+        h.mf_set_hot_row_thinning(None, None)
+    assert np.array_equal(got, want)
