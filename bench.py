@@ -217,6 +217,56 @@ def cpu_baseline(prob, cfg, seed, threads, target_updates):
     return done / dt, done, dt
 
 
+def time_fp32_sgd(torch, h, prob, W, warmup, steps, cfg, seed):
+    """The fp32-SGD update (-v 5) on the same ratings, schedule and hot-row tables: dense fp32 P and Q."""
+    dev, k, st = prob.R.device, prob.k, torch.cuda.current_stream().cuda_stream
+    P = torch.empty(prob.n_users * k, dtype=torch.float32, device=dev)
+    Q = torch.empty(prob.n_items * k, dtype=torch.float32, device=dev)
+    h.mf_init_rand_feature(P.data_ptr(), P.numel(), seed, 0, st)
+    h.mf_init_rand_feature(Q.data_ptr(), Q.numel(), seed, 1, st)
+    uc = h.mf_update_count(prob.n, W, 128)
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    for e in range(warmup + steps):
+        if e >= warmup:
+            ev[e - warmup][0].record()
+        h.mf_single_sgd_hogwild(prob.R.data_ptr(), prob.n, P.data_ptr(), Q.data_ptr(), k, W, uc, 128,
+                                h.mf_lr_schedule(cfg["lr"], cfg["decay"], e), cfg["lam"], seed, e, None, st)
+        if e >= warmup:
+            ev[e - warmup][1].record()
+    torch.cuda.synchronize()
+    acc = torch.zeros(1, dtype=torch.float64, device=dev)
+    h.mf_test_rmse(prob.test.data_ptr(), prob.test.shape[0], P.data_ptr(), Q.data_ptr(), k, acc.data_ptr(), st)
+    rmse = float(np.sqrt(acc.item() / prob.test.shape[0]))
+    return np.array([a.elapsed_time(b) for a, b in ev]), uc, rmse
+
+
+def reference_rule_rmse(prob, h, cfg, seed, threads, epochs, workers):
+    """Test RMSE of the reference update rule (the checker's MASCOT epoch as an OpenMP Hogwild loop, `threads` updates
+    in flight) after `epochs` epochs on the same shuffled ratings, initial model, schedule and learning rates."""
+    from oracle import oracle as om
+    orc = om.get()
+    prob.reset()
+    R = prob.R.cpu().numpy().view(np.uint8).reshape(-1).view(om.NODE)
+    gu, gi = prob.host_grouped()
+    uc = h.mf_update_count(prob.n, workers, 128)
+    z = [np.zeros(n, np.float32) for n in (gu.groups * prob.k, gi.groups * prob.k, gu.groups, gi.groups)]
+    for e in range(epochs):
+        t0 = time.perf_counter()
+        orc.lib.orc_mascot_epoch(prob.k, R.ctypes.data, R.size, gu.ptrs, gi.ptrs, gu.end_idx.ctypes.data, gi.end_idx.ctypes.data,
+                                 gu.prec.ctypes.data, gi.prec.ctypes.data, gu.groups, gi.groups, workers, uc, 128,
+                                 h.mf_lr_schedule(cfg["lr"], cfg["decay"], e), cfg["lam"], uc * 128,
+                                 z[0].ctypes.data, z[1].ctypes.data, z[2].ctypes.data, z[3].ctypes.data, seed, e, None, threads)
+        print("bench.py: reference rule on the CPU, epoch %d of %d, %.1f s" % (e + 1, epochs, time.perf_counter() - t0), file=sys.stderr, flush=True)
+    for s, g in zip(prob.sides, (gu, gi)):                      # score it with the same device RMSE kernel
+        host = s["arena"].cpu().numpy()
+        for o, sz, arr in zip(s["offs"], s["sizes"], g.arrays):
+            host[int(o):int(o) + int(sz) * prob.k * 2] = arr.view(np.uint8)
+        s["arena"].copy_(prob.torch.from_numpy(host))
+    rmse = prob.rmse()
+    prob.reset()
+    return rmse
+
+
 def measured_traffic(a, leg):
     """HBM bytes per launch of a plain epoch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch, scaled by
     2.0 / 1.0, the factors a 1 GiB device copy gives; summaries under profiles/).  Counters cannot be read from inside
@@ -240,16 +290,19 @@ def main():
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--ratings", type=int, default=100_000_000)
-    ap.add_argument("--workers", type=int, default=2048, help="-wg of the measured run (reference default for k=128)")
+    ap.add_argument("--workers", type=int, default=6144, help="-wg of the measured run (24 wavefronts on each of the 256 CUs)")
     ap.add_argument("--cached-workers", type=int, default=16384)
     ap.add_argument("--cpu-updates", type=int, default=6_000_000, help="size of the CPU baseline sample")
     ap.add_argument("--skip-cpu", action="store_true")
     ap.add_argument("--skip-cached", action="store_true")
     ap.add_argument("--skip-coherent", action="store_true", help="profiling aid: time only the cached-rows leg")
     ap.add_argument("--skip-exact", action="store_true", help="skip the leg with every row update carried out (no thinning)")
-    ap.add_argument("--hot-row-inflight", type=float, default=16.0, help="hot-row thinning cap of the measured run (0 = off)")
+    ap.add_argument("--hot-row-inflight", type=float, default=8.0, help="hot rows of the measured run are thinned to this many updates in flight (0 = no hot rows)")
     ap.add_argument("--pmc-copy", action="store_true",
                     help="profiling aid: also run three 1 GiB device copies, the known-size kernel that FETCH_SIZE / WRITE_SIZE are scaled by")
+    ap.add_argument("--skip-fp32", action="store_true", help="skip the fp32-SGD leg")
+    ap.add_argument("--reference-rmse", action="store_true",
+                    help="also train with the reference rule on the CPU for warmup+steps epochs (minutes) and report the test RMSE delta")
     ap.add_argument("--seed", type=int, default=2021)
     a = ap.parse_args()
     if a.gpus != 1:
@@ -331,6 +384,22 @@ def main():
                                            "kernel": "hogwild_kernel<MascotRule<128,false>>"},
                               "ms_steps": c["ms_steps"], "test_rmse_after_timed_epochs": c["rmse"]}
         h.mf_set_row_coherence(1)
+    if not a.skip_fp32 and not a.skip_coherent:
+        h.mf_set_row_coherence(1)
+        kept = prob.set_thinning(a.workers, a.hot_row_inflight)
+        per, uc, rmse = time_fp32_sgd(torch, h, prob, a.workers, a.warmup, a.steps, cfg, a.seed)
+        prob.set_thinning(a.workers, 0.0)
+        ms = float(per.mean())
+        bpu = 12 + 2 * k * 4 + 2 * k * 4 * kept
+        out["fp32_sgd"] = {"note": "fp32 SGD (-v 5) on the same ratings, workers, row access and hot-row tables",
+                           "value": a.ratings / (ms / 1e3), "unit": "ratings/s", "ms_per_step": ms, "workers": a.workers,
+                           "roofline_frac": a.workers * uc * 128 * bpu / (ms / 1e3) / 1e9 / PEAK_HBM_GBS,
+                           "test_rmse_after_timed_epochs": rmse, "mascot_speedup": ms / main_leg["ms_per_step"]}
+    if a.reference_rmse:
+        threads = min(os.cpu_count() or 1, 16)
+        ref = reference_rule_rmse(prob, h, cfg, a.seed, threads, a.warmup + a.steps, 2048)
+        out["reference_rule"] = {"test_rmse": ref, "epochs": a.warmup + a.steps, "threads": threads,
+                                 "rmse_delta": main_leg["rmse"] - ref}
     if not a.skip_cpu:
         threads = min(os.cpu_count() or 1, 16)
         prob.reset()

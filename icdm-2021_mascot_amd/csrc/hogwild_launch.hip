@@ -49,48 +49,47 @@ static int g_row_coherence = 1;
 // different XCDs are reconciled during an epoch
 static uint32_t g_epoch_splits = 1;
 
-struct Segment { uint32_t begin, end; bool tail; };
-template <class P> static auto set_tail(P& p, bool v) -> decltype(p.lds_stats, void()) { p.lds_stats = v; }
-static void set_tail(...) {}
+// What part of an epoch one call to launch() covers, in each worker's processed-rating index space.
+struct Range {
+    uint32_t begin = 0, end = 0;
+    bool accumulate = false;      // an earlier launch of the same epoch has already run
+    size_t stats_lds = 0;         // > 0: one launch of <= 256 workgroups of 16 wavefronts with this much LDS, the
+                                  // rule keeping its sampled gradient sums there (MASCOT check epochs)
+};
+template <class P> static auto set_lds_stats(P& p, bool v) -> decltype(p.lds_stats, void()) { p.lds_stats = v; }
+static void set_lds_stats(...) {}
 
 template <class Rule>
-static int launch(const char* who, const Schedule& s0, const typename Rule::Params& prm0, size_t lds, void* stream,
-                  uint32_t tail_begin = 0xffffffffu, size_t tail_lds = 0)
+static int launch(const char* who, const Schedule& s0, const typename Rule::Params& prm0, size_t lds, void* stream, Range r)
 {
-    if (s0.update_count == 0 || s0.update_vector_size == 0) return MF_OK;
-    const uint32_t total = s0.range_end;
-    // [0, body_end) runs as ordinary launches (cut into g_epoch_splits pieces on window boundaries);
-    // [body_end, total) -- the sampled tail of a MASCOT check epoch -- runs as one launch of large workgroups
-    // that keep their gradient sums in LDS
-    const bool has_tail = tail_begin < total;
-    const uint32_t body_end = has_tail ? tail_begin : total;
-    std::vector<Segment> seg;
-    uint32_t splits = Rule::kSplittable ? g_epoch_splits : 1;
-    const uint32_t body_windows = body_end / s0.update_vector_size;
-    if (splits > body_windows) splits = body_windows ? body_windows : 1;
-    for (uint32_t i = 0; i < splits; ++i) {
-        const uint32_t b = (uint32_t)((uint64_t)body_windows * i / splits) * s0.update_vector_size;
-        const uint32_t e = i + 1 == splits ? body_end : (uint32_t)((uint64_t)body_windows * (i + 1) / splits) * s0.update_vector_size;
-        if (b < e || !has_tail) seg.push_back({b, e, false});
+    if (s0.update_count == 0 || s0.update_vector_size == 0 || r.begin >= r.end) return MF_OK;
+    Schedule s = s0;
+    typename Rule::Params prm = prm0;
+    if (r.stats_lds) {
+        s.range_begin = r.begin; s.range_end = r.end;
+        prm.accumulate = r.accumulate;
+        uint32_t blocks = (s.num_workers + 15) / 16;
+        if (blocks > 256) blocks = 256;
+        if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&hogwild_kernel<Rule>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)r.stats_lds),
+                               "hipFuncSetAttribute(MaxDynamicSharedMemorySize)")) return rc;
+        set_lds_stats(prm, true);
+        hipLaunchKernelGGL((hogwild_kernel<Rule>), dim3(blocks), dim3(kMaxBlock), r.stats_lds, as_stream(stream), s, prm);
+        return launch_status(who);
     }
-    if (has_tail) seg.push_back({body_end, total, true});
+    // ordinary launches, cut into g_epoch_splits pieces on window boundaries
+    uint32_t splits = Rule::kSplittable ? g_epoch_splits : 1;
+    const uint32_t first_window = (r.begin + s0.update_vector_size - 1) / s0.update_vector_size, end_window = r.end / s0.update_vector_size;
+    const uint32_t windows = end_window > first_window ? end_window - first_window : 0;
+    if (splits > windows) splits = windows ? windows : 1;
     bool first = true;
-    for (const Segment& sg : seg) {
-        Schedule s = s0;
-        typename Rule::Params prm = prm0;
-        s.range_begin = sg.begin; s.range_end = sg.end;
-        prm.accumulate = !first;
+    for (uint32_t i = 0; i < splits; ++i) {
+        const uint32_t b = i == 0 ? r.begin : (first_window + (uint32_t)((uint64_t)windows * i / splits)) * s0.update_vector_size;
+        const uint32_t e = i + 1 == splits ? r.end : (first_window + (uint32_t)((uint64_t)windows * (i + 1) / splits)) * s0.update_vector_size;
+        if (b >= e) continue;
+        s.range_begin = b; s.range_end = e;
+        prm.accumulate = r.accumulate || !first;
         first = false;
-        if (sg.tail) {
-            uint32_t blocks = (s.num_workers + 15) / 16;
-            if (blocks > 256) blocks = 256;
-            if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&hogwild_kernel<Rule>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)tail_lds),
-                                   "hipFuncSetAttribute(MaxDynamicSharedMemorySize)")) return rc;
-            set_tail(prm, true);
-            hipLaunchKernelGGL((hogwild_kernel<Rule>), dim3(blocks), dim3(kMaxBlock), tail_lds, as_stream(stream), s, prm);
-        } else {
-            hipLaunchKernelGGL((hogwild_kernel<Rule>), dim3(grid_for(s.num_workers)), dim3(kBlock), lds, as_stream(stream), s, prm);
-        }
+        hipLaunchKernelGGL((hogwild_kernel<Rule>), dim3(grid_for(s.num_workers)), dim3(kBlock), lds, as_stream(stream), s, prm);
         if (int rc = launch_status(who)) return rc;
     }
     return MF_OK;
@@ -99,17 +98,17 @@ static int launch(const char* who, const Schedule& s0, const typename Rule::Para
 // Instantiates Rule<K, COH> for the four (k, coherence) combinations; P is the parameter pack type,
 // identical across instantiations apart from the template arguments.
 template <template <int, bool> class Rule, class MakeParams>
-static int launch_k_coh(const char* who, int k, const Schedule& s, MakeParams make, size_t lds, void* stream,
-                        uint32_t tail_begin = 0xffffffffu, size_t tail_lds = 0)
+static int launch_k_coh(const char* who, int k, const Schedule& s, MakeParams make, size_t lds, void* stream, Range r)
 {
     const bool coh = g_row_coherence != 0;
     if (k == 128) {
-        if (coh) { auto a = make(typename Rule<128, true>::Params{}); return launch<Rule<128, true>>(who, s, a, lds, stream, tail_begin, tail_lds); }
-        auto a = make(typename Rule<128, false>::Params{}); return launch<Rule<128, false>>(who, s, a, lds, stream, tail_begin, tail_lds);
+        if (coh) { auto a = make(typename Rule<128, true>::Params{}); return launch<Rule<128, true>>(who, s, a, lds, stream, r); }
+        auto a = make(typename Rule<128, false>::Params{}); return launch<Rule<128, false>>(who, s, a, lds, stream, r);
     }
-    if (coh) { auto a = make(typename Rule<64, true>::Params{}); return launch<Rule<64, true>>(who, s, a, lds, stream, tail_begin, tail_lds); }
-    auto a = make(typename Rule<64, false>::Params{}); return launch<Rule<64, false>>(who, s, a, lds, stream, tail_begin, tail_lds);
+    if (coh) { auto a = make(typename Rule<64, true>::Params{}); return launch<Rule<64, true>>(who, s, a, lds, stream, r); }
+    auto a = make(typename Rule<64, false>::Params{}); return launch<Rule<64, false>>(who, s, a, lds, stream, r);
 }
+static Range whole_epoch(const Schedule& s) { Range r; r.begin = 0; r.end = s.range_end; return r; }
 
 }  // namespace mf
 
@@ -175,7 +174,7 @@ int mf_single_sgd_hogwild(const mf_node* R, uint32_t nnz, float* p, float* q, in
     if (int rc = check_schedule("mf_single_sgd_hogwild", R, nnz, k, num_workers, update_count, update_vector_size)) return rc;
     if (!p || !q) return invalid("mf_single_sgd_hogwild: null model pointer");
     Schedule s = make_schedule(R, nnz, num_workers, update_count, update_vector_size, seed, epoch, window_start);
-    return launch_k_coh<SgdRule>("mf_single_sgd_hogwild", k, s, [&](auto a) { a.p = p; a.q = q; a.lrate = lrate; a.lambda = lambda; return a; }, 0, stream);
+    return launch_k_coh<SgdRule>("mf_single_sgd_hogwild", k, s, [&](auto a) { a.p = p; a.q = q; a.lrate = lrate; a.lambda = lambda; return a; }, 0, stream, whole_epoch(s));
 }
 
 int mf_mpt_sgd_hogwild(const mf_node* R, uint32_t nnz, float* p, float* q, int k,
@@ -188,7 +187,7 @@ int mf_mpt_sgd_hogwild(const mf_node* R, uint32_t nnz, float* p, float* q, int k
     if (!(scaling_factor > 0)) return invalid("mf_mpt_sgd_hogwild: scaling_factor must be positive");
     Schedule s = make_schedule(R, nnz, num_workers, update_count, update_vector_size, seed, epoch, window_start);
     return launch_k_coh<MptRule>("mf_mpt_sgd_hogwild", k, s, [&](auto a) {
-        a.p = p; a.q = q; a.lrate = lrate; a.scaled_lambda_half = scaled_lambda_half; a.scaling_factor = scaling_factor; return a; }, 0, stream);
+        a.p = p; a.q = q; a.lrate = lrate; a.scaled_lambda_half = scaled_lambda_half; a.scaling_factor = scaling_factor; return a; }, 0, stream, whole_epoch(s));
 }
 
 static bool muppet_precision_ok(uint8_t b) { return b == 8 || b == 12 || b == 14 || b == 16 || b == 32; }
@@ -210,7 +209,7 @@ int mf_muppet_sgd_hogwild(const mf_node* R, uint32_t nnz, float* p, float* q, in
     return launch_k_coh<MuppetRule>("mf_muppet_sgd_hogwild", k, s, [&](auto a) {
         a.p = p; a.q = q; a.lrate = lrate; a.lambda = lambda; a.first_sample = first_sample_rating_idx;
         a.sum_updated_val = sum_updated_val; a.sum_norms = sum_norms; a.num_workers = num_workers;
-        a.fwd = forward_prop_precision; a.bwd = backward_prop_precision; return a; }, 0, stream);
+        a.fwd = forward_prop_precision; a.bwd = backward_prop_precision; return a; }, 0, stream, whole_epoch(s));
 }
 
 int mf_afp_sgd_hogwild(const mf_node* R, uint32_t nnz, float* p, float* q, int k,
@@ -224,7 +223,7 @@ int mf_afp_sgd_hogwild(const mf_node* R, uint32_t nnz, float* p, float* q, int k
     // afp_sgd_kernel.h:145: int initialization_threshold = (float)(update_count*update_vector_size)/10.0f
     const int init_threshold = (int)((float)(update_count * update_vector_size) / 10.0f);
     return launch_k_coh<AfpRule>("mf_afp_sgd_hogwild", k, s, [&](auto a) {
-        a.p = p; a.q = q; a.lrate = lrate; a.lambda = lambda; a.afp_epoch = afp_epoch; a.init_threshold = init_threshold; return a; }, 0, stream);
+        a.p = p; a.q = q; a.lrate = lrate; a.lambda = lambda; a.afp_epoch = afp_epoch; a.init_threshold = init_threshold; return a; }, 0, stream, whole_epoch(s));
 }
 
 int mf_mascot_sgd_hogwild(const mf_node* R, uint32_t nnz, void* const* p, void* const* q, int k,
@@ -246,19 +245,26 @@ int mf_mascot_sgd_hogwild(const mf_node* R, uint32_t nnz, void* const* p, void* 
     const size_t lds = MascotRule<128, true>::lds_bytes(user_group_num, item_group_num);
     if (lds > 64 * 1024) return invalid("%s: group tables need %zu bytes of LDS (limit 65536)", who, lds);
     Schedule s = make_schedule(R, nnz, num_workers, update_count, update_vector_size, seed, epoch, window_start);
-    // sampled tail: its own launch with the gradient sums in LDS when they fit (160 KB per workgroup)
-    uint32_t tail_begin = 0xffffffffu;
-    size_t tail_lds = 0;
-    if (first_sample_rating_idx < update_count * update_vector_size) {
-        const size_t need = lds + (size_t)(user_group_num + item_group_num) * (size_t)k * sizeof(float);
-        if (need <= 160 * 1024) { tail_begin = first_sample_rating_idx; tail_lds = need; }
-    }
-    return launch_k_coh<MascotRule>(who, k, s, [&](auto a) {
+    auto fill = [&](auto a) {
         a.p = p; a.q = q; a.user_end = user_group_end_idx; a.item_end = item_group_end_idx;
         a.user_prec = user_group_prec_info; a.item_prec = item_group_prec_info;
         a.grad_sum_p = grad_sum_norm_p; a.grad_sum_q = grad_sum_norm_q; a.norm_sum_p = norm_sum_p; a.norm_sum_q = norm_sum_q;
         a.first_sample = first_sample_rating_idx; a.user_groups = user_group_num; a.item_groups = item_group_num;
-        a.lrate = lrate; a.lambda = lambda; a.norm_stride = grid_for(num_workers); a.lds_stats = false; return a; }, lds, stream, tail_begin, tail_lds);
+        a.lrate = lrate; a.lambda = lambda; a.norm_stride = grid_for(num_workers); a.lds_stats = false; return a; };
+    const uint32_t total = s.range_end;
+    Range body = whole_epoch(s);
+    if (first_sample_rating_idx >= total)                     // nothing is sampled: the kernel without the statistics code
+        return launch_k_coh<MascotPlainRule>(who, k, s, fill, lds, stream, body);
+    // A check epoch.  The sampled ratings [first_sample, total) run as their own launch with the gradient sums in
+    // LDS when those fit (160 KB per workgroup); otherwise the whole epoch runs with the sums in global memory.
+    const size_t need = lds + (size_t)(user_group_num + item_group_num) * (size_t)k * sizeof(float);
+    if (need > 160 * 1024) return launch_k_coh<MascotRule>(who, k, s, fill, lds, stream, body);
+    body.end = first_sample_rating_idx;
+    // the body still writes the (zero) norm sums of its workgroups, which the sampled launch then adds to
+    if (int rc = launch_k_coh<MascotPlainRule>(who, k, s, fill, lds, stream, body)) return rc;
+    Range tail;
+    tail.begin = first_sample_rating_idx; tail.end = total; tail.accumulate = body.begin < body.end; tail.stats_lds = need;
+    return launch_k_coh<MascotRule>(who, k, s, fill, lds, stream, tail);
 }
 
 }  // extern "C"

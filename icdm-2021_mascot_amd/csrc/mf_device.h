@@ -105,21 +105,28 @@ __device__ __forceinline__ uint64_t bcast(uint64_t v, int lane)
 // is done about it.  COH = false keeps ordinary write-back stores: each XCD then works on its own
 // L2-resident copy of a hot row between evictions (a row that is not re-used while cached behaves the
 // same either way).  The host picks per run (mf_set_row_coherence).
-template <class T> __device__ __forceinline__ T row_load(const T* p) { return *p; }
+//
+// Rows are addressed through pointers in the global address space: a pointer rebuilt from an integer (the
+// per-group pointer tables) would otherwise be a generic one, and generic accesses are flat instructions
+// that also count as LDS traffic, so every wait for an LDS or scalar load would wait for all row loads in flight.
+#define MF_GLOBAL __attribute__((address_space(1)))
+template <class T> __device__ __forceinline__ MF_GLOBAL T* global_ptr(T* p) { return (MF_GLOBAL T*)p; }
+template <class T> __device__ __forceinline__ MF_GLOBAL T* global_ptr(uint64_t addr) { return (MF_GLOBAL T*)addr; }
+template <class T> __device__ __forceinline__ T row_load(const T* p) { return *global_ptr(p); }
 template <bool COH, class T> __device__ __forceinline__ void row_store(T* p, T v)
 {
-    if constexpr (COH) __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    else *p = v;
+    if constexpr (COH) __hip_atomic_store(global_ptr(p), v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    else *global_ptr(p) = v;
 }
 // Aggregated update of a hot row (Schedule::keep_u): the change is added in memory, so concurrent updates
 // of the row add up instead of overwriting each other.
 __device__ __forceinline__ void row_add(float* p, float d)
 {
-    (void)__hip_atomic_fetch_add(p, d, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    (void)__hip_atomic_fetch_add(global_ptr(p), d, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 __device__ __forceinline__ void row_add(half2_t* p, half2_t d)
 {
-    (void)__builtin_amdgcn_global_atomic_fadd_v2f16((__attribute__((address_space(1))) half2_t*)p, d);
+    (void)__builtin_amdgcn_global_atomic_fadd_v2f16(global_ptr(p), d);
 }
 
 // ---- counter-based generator -----------------------------------------------------------

@@ -19,7 +19,8 @@
 
 namespace mf {
 
-template <int K, bool COH> struct MascotRule {
+// SAMPLED = false compiles the sampled-statistics code out: the kernel for launches in which no rating is sampled.
+template <int K, bool COH, bool SAMPLED> struct MascotRuleT {
     static constexpr int E = K / 64;                        // elements per lane
     static constexpr int kAhead = 3, kRing = 8;
     // chunk classes: 0 = any mix of precisions (flag-driven), 1 = every rating of the chunk touches two
@@ -55,6 +56,10 @@ template <int K, bool COH> struct MascotRule {
     uint32_t first_sample, user_groups, item_groups;
     float lrate, lambda;
     int lane;
+    // Sampled sums of the most popular group of each side (the last one; with Zipf-like data it takes half of all
+    // ratings) stay in registers and reach the shared sums once per wavefront: LDS float atomics are the bound of
+    // the sampled launch otherwise.
+    mutable float top_gp[E], top_gq[E], top_np, top_nq;
 
     static __host__ __device__ size_t lds_bytes(uint32_t ug, uint32_t ig) { return ((size_t)(ug + ig) * (8 + 4 + 4 + 1) + 31) / 16 * 16; }
     static size_t lds_stats_bytes(uint32_t ug, uint32_t ig) { return (size_t)(ug + ig) * K * sizeof(float); }
@@ -81,6 +86,8 @@ template <int K, bool COH> struct MascotRule {
         }
         grad_sum_p = a.grad_sum_p; grad_sum_q = a.grad_sum_q;
         first_sample = a.first_sample; lrate = a.lrate; lambda = a.lambda;
+        for (int e = 0; e < E; ++e) { top_gp[e] = 0.f; top_gq[e] = 0.f; }
+        top_np = 0.f; top_nq = 0.f;
         ugrad_s = nullptr; igrad_s = nullptr;
         if (a.lds_stats) {
             ugrad_s = reinterpret_cast<float*>(smem + lds_bytes(user_groups, item_groups));
@@ -234,23 +241,44 @@ template <int K, bool COH> struct MascotRule {
     {
         if constexpr (E == 2) { HV h; h.x = v; h.y = v; return h; } else return v;
     }
-    // sampled statistics of one binary16 side: ||g||^2 into the block's LDS slot, g into the global sums
-    __device__ __forceinline__ void sample(const float* g, uint32_t group, float* norm_s, float* grad_sum, float* grad_s) const
+    // sampled statistics of one binary16 side: ||g||^2 into the block's LDS slot, g into the workgroup's LDS
+    // sums or, without them, into the global sums.  The LDS accesses are spelled in the LDS address space: a
+    // pointer that may be either would make them flat instructions, which wait for every outstanding row load.
+    typedef __attribute__((address_space(3))) float lds_float;
+    static __device__ __forceinline__ void lds_add(float* p, float v)
+    {
+        (void)__hip_atomic_fetch_add((lds_float*)p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
+    __device__ __forceinline__ void add_sums(const float* g, float n, uint32_t group, float* norm_s, float* grad_sum, float* grad_s) const
+    {
+        if (lane == 0) lds_add(&norm_s[group], n);
+        if (grad_s) {      // LDS layout [group][e][lane]: consecutive lanes on consecutive banks
+#pragma unroll
+            for (int e = 0; e < E; ++e) lds_add(grad_s + (size_t)group * K + e * kWave + lane, g[e]);
+        } else {
+#pragma unroll
+            for (int e = 0; e < E; ++e) atomicAdd(grad_sum + (size_t)group * K + (size_t)lane * E + e, g[e]);
+        }
+    }
+    __device__ __forceinline__ void sample(const float* g, uint32_t group, bool user_side) const
     {
         float n = g[0] * g[0];
         if constexpr (E == 2) n = n + g[1] * g[1];
         n = reduce_wave(n, OpAdd());
-        if (lane == 0) atomicAdd(&norm_s[group], n);
-        float* dst = (grad_s ? grad_s : grad_sum) + (size_t)group * K + (size_t)lane * E;
-#pragma unroll
-        for (int e = 0; e < E; ++e) atomicAdd(dst + e, g[e]);
+        if (user_side) {
+            if (group == user_groups - 1) { for (int e = 0; e < E; ++e) top_gp[e] += g[e]; top_np += n; }
+            else add_sums(g, n, group, unorm_s, grad_sum_p, ugrad_s);
+        } else {
+            if (group == item_groups - 1) { for (int e = 0; e < E; ++e) top_gq[e] += g[e]; top_nq += n; }
+            else add_sums(g, n, group, inorm_s, grad_sum_q, igrad_s);
+        }
     }
 
     template <int CLS> __device__ __forceinline__ void update(Row& row, const Info& i, uint32_t processed) const
     {
         if (CLS == 0 && (i.flags & kSkip)) return;
         const bool up = CLS == 0 && (i.flags & 1u), ip = CLS == 0 && (i.flags & 2u);
-        const bool sampled = processed >= first_sample;
+        const bool sampled = SAMPLED && processed >= first_sample;
         const uint32_t ug = (i.flags >> 3) & 0x3fffu, ig = (i.flags >> 17) & 0x3fffu;
         if (!up && !ip) {
             // mascot_sgd_kernel.h:188-278: everything in binary16, one rounding per operation
@@ -273,10 +301,10 @@ template <int K, bool COH> struct MascotRule {
                 float g[E];
 #pragma unroll
                 for (int e = 0; e < E; ++e) g[e] = widen(gp, e);
-                sample(g, ug, unorm_s, grad_sum_p, ugrad_s);
+                sample(g, ug, true);
 #pragma unroll
                 for (int e = 0; e < E; ++e) g[e] = widen(gq, e);
-                sample(g, ig, inorm_s, grad_sum_q, igrad_s);
+                sample(g, ig, false);
             }
         } else {
             float pf[E], qf[E], m[E];
@@ -314,8 +342,8 @@ template <int K, bool COH> struct MascotRule {
                 } else store_side(row.q, i.qptr, ip, lane);
             }
             if (sampled) {
-                if (!up) sample(gp, ug, unorm_s, grad_sum_p, ugrad_s);
-                if (!ip) sample(gq, ig, inorm_s, grad_sum_q, igrad_s);
+                if (!up) sample(gp, ug, true);
+                if (!ip) sample(gq, ig, false);
             }
         }
     }
@@ -323,6 +351,11 @@ template <int K, bool COH> struct MascotRule {
     // mascot_sgd_kernel.h:448-456: per-block norm sums, layout [group][norm_stride]
     __device__ __forceinline__ void finish(const Params& a, uint32_t) const
     {
+        if constexpr (SAMPLED) {
+            const float np0 = bcast(top_np, 0), nq0 = bcast(top_nq, 0);
+            if (np0 != 0.f) add_sums(top_gp, np0, user_groups - 1, unorm_s, grad_sum_p, ugrad_s);
+            if (nq0 != 0.f) add_sums(top_gq, nq0, item_groups - 1, inorm_s, grad_sum_q, igrad_s);
+        }
         __syncthreads();
         // a launch that continues an epoch (accumulate) adds to what the earlier launches of the epoch left
         for (uint32_t g = threadIdx.x; g < user_groups; g += blockDim.x) {
@@ -340,10 +373,14 @@ template <int K, bool COH> struct MascotRule {
             }
         }
         if (ugrad_s) {     // single flush of the workgroup's gradient sums
-            for (uint32_t i = threadIdx.x; i < user_groups * K; i += blockDim.x) { const float v = ugrad_s[i]; if (v != 0.f) atomicAdd(grad_sum_p + i, v); }
-            for (uint32_t i = threadIdx.x; i < item_groups * K; i += blockDim.x) { const float v = igrad_s[i]; if (v != 0.f) atomicAdd(grad_sum_q + i, v); }
+            // LDS slot [g][e][l] holds element l*E + e of group g
+            auto element = [](uint32_t i) { const uint32_t g = i / K, r = i % K; return g * K + (r % kWave) * E + r / kWave; };
+            for (uint32_t i = threadIdx.x; i < user_groups * K; i += blockDim.x) { const float v = ugrad_s[i]; if (v != 0.f) atomicAdd(grad_sum_p + element(i), v); }
+            for (uint32_t i = threadIdx.x; i < item_groups * K; i += blockDim.x) { const float v = igrad_s[i]; if (v != 0.f) atomicAdd(grad_sum_q + element(i), v); }
         }
     }
 };
+template <int K, bool COH> using MascotRule = MascotRuleT<K, COH, true>;
+template <int K, bool COH> using MascotPlainRule = MascotRuleT<K, COH, false>;
 
 }  // namespace mf

@@ -510,7 +510,7 @@ void mf_default_params(mf_params* out)       // main.cu:19-32
     out->lambda = 0.015f; out->learning_rate = 0.01f; out->decay = 0.1f; out->sample_ratio = 0.01f; out->error_threshold = 0.001f;
     out->k = 128; out->epoch = 50; out->num_workers = 2048; out->thread_block_size = 128;
     out->user_group_num = 10; out->item_group_num = 10; out->version = 7; out->interval = 1; out->seed = 1;
-    out->hot_row_inflight = 16.0f;      // no reference counterpart: see mf_set_hot_row_thinning
+    out->hot_row_inflight = 8.0f;       // no reference counterpart: see mf_set_hot_row_thinning
 }
 
 uint32_t mf_group_end_indices(const uint32_t* sorted_cnt, uint32_t n, uint32_t requested_groups, uint32_t* end_idx_out)
