@@ -274,13 +274,9 @@ def measured_traffic(a, leg):
     if a.ratings != 100_000_000 or a.seed != 2021:
         return None
     if a.skip_coherent:
-        return (13_986_844 * 2.0 + 24_179_238) * 1024 if leg["workers"] == 16384 else None
-    if leg["workers"] != 2048:
-        return None
-    if a.hot_row_inflight == 16.0:
-        return (19_663_594 * 2.0 + 37_531_052) * 1024
-    if a.hot_row_inflight == 0.0:
-        return (23_408_594 * 2.0 + 50_072_631) * 1024
+        return (14_053_967 * 2.0 + 24_189_917) * 1024 if leg["workers"] == 16384 else None
+    if leg["workers"] == 6144 and a.hot_row_inflight == 8.0:
+        return (17_636_147 * 2.0 + 32_167_634) * 1024
     return None
 
 
@@ -292,7 +288,7 @@ def main():
     ap.add_argument("--ratings", type=int, default=100_000_000)
     ap.add_argument("--workers", type=int, default=6144, help="-wg of the measured run (24 wavefronts on each of the 256 CUs)")
     ap.add_argument("--cached-workers", type=int, default=16384)
-    ap.add_argument("--cpu-updates", type=int, default=6_000_000, help="size of the CPU baseline sample")
+    ap.add_argument("--cpu-updates", type=int, default=32_000_000, help="size of the CPU baseline sample (about 10 s on 16 threads)")
     ap.add_argument("--skip-cpu", action="store_true")
     ap.add_argument("--skip-cached", action="store_true")
     ap.add_argument("--skip-coherent", action="store_true", help="profiling aid: time only the cached-rows leg")
