@@ -393,7 +393,7 @@ def main():
                            "test_rmse_after_timed_epochs": rmse, "mascot_speedup": ms / main_leg["ms_per_step"]}
     if a.reference_rmse:
         threads = min(os.cpu_count() or 1, 16)
-        ref = reference_rule_rmse(prob, h, cfg, a.seed, threads, a.warmup + a.steps, 2048)
+        ref = reference_rule_rmse(prob, h, cfg, a.seed, threads, a.warmup + a.steps, a.workers)
         out["reference_rule"] = {"test_rmse": ref, "epochs": a.warmup + a.steps, "threads": threads,
                                  "rmse_delta": main_leg["rmse"] - ref}
     if not a.skip_cpu:

@@ -60,7 +60,7 @@ int main(int argc, const char* argv[])
     std::cout << "Decay                       : " << prm.decay << std::endl;
     std::cout << "Lambda                      : " << prm.lambda << std::endl;
     std::cout << "Iteration                   : " << prm.epoch << std::endl;
-    std::cout << "Num of workers              : " << prm.num_workers << std::endl;
+    std::cout << "Num of workers              : " << prm.num_workers << (prm.num_workers ? "" : " (chosen from the number of ratings)") << std::endl;
     std::cout << "Thread block size           : " << prm.thread_block_size << std::endl;
     std::cout << "Sample ratio                : " << prm.sample_ratio << std::endl;
     std::cout << "Error threshold             : " << prm.error_threshold << std::endl;

@@ -551,6 +551,14 @@ int mf_init_model(float* p, float* q, uint32_t n_users, uint32_t n_items, uint32
     return 0;
 }
 
+uint32_t mf_auto_workers(uint32_t n)
+{
+    // about 128 windows of 128 ratings per worker: the ratio at which the runs on 8M and on 100M ratings stay
+    // within 0.005 test RMSE of the reference rule run on the CPU; at most 24 wavefronts on each of the 256 CUs
+    uint32_t w = (n / 16384u + 3u) / 4u * 4u;
+    return w < 16u ? 16u : (w > 6144u ? 6144u : w);
+}
+
 int mf_train(const mf_params* params, const mf_node* R, uint32_t n, uint32_t n_users, uint32_t n_items,
              const mf_node* test, uint32_t test_n, float* p, float* q, mf_report* report)
 {
@@ -558,7 +566,9 @@ int mf_train(const mf_params* params, const mf_node* R, uint32_t n, uint32_t n_u
     if (test_n && !test) return invalid("mf_train: null test set");
     if (params->k != 64 && params->k != 128) return invalid("mf_train: k must be 64 or 128 (got %u)", params->k);
     if (n == 0 || n_users == 0 || n_items == 0) return invalid("mf_train: empty problem");
-    if (params->num_workers == 0) return invalid("mf_train: num_workers must be positive");
+    mf_params with_workers = *params;
+    if (with_workers.num_workers == 0) with_workers.num_workers = mf_auto_workers(n);
+    params = &with_workers;
     const uint32_t version = params->version == 0 ? 5 : params->version;
     if (version < 1 || version > 5) return invalid("mf_train: version %u is not built (1 MASCOT, 2 AFP, 3 MuPPET, 4 MPT, 5 fp32 SGD)", params->version);
     Common c;

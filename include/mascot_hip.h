@@ -71,6 +71,10 @@ int mf_set_hot_row_thinning(const uint8_t* user_keep, const uint8_t* item_keep);
 uint32_t mf_mascot_norm_blocks(uint32_t num_workers);
 /* Host-side closed forms of the schedule (mf_methods.cu:94-111,170-175). */
 uint32_t mf_update_count(uint32_t n, uint32_t num_workers, uint32_t update_vector_size);
+/* Worker count mf_train uses for mf_params.num_workers == 0: n / 16384 (about 128 windows per worker), a multiple
+ * of 4, between 16 and 6144.  The updates in flight grow with the workers and so does the distance to a sequential
+ * run; the reference's fixed default (2048, main.cu:28) suits neither 400k nor 100M ratings on this GPU. */
+uint32_t mf_auto_workers(uint32_t n);
 uint32_t mf_first_sample_rating_idx(uint32_t e, uint32_t interval, uint32_t epochs, uint32_t update_count,
                                     uint32_t update_vector_size, float sample_ratio);
 float mf_lr_schedule(float lr, float decay, uint32_t e);
@@ -198,7 +202,7 @@ typedef struct {
     uint32_t user_group_num;  /* -ug (requested; the grouping may return fewer, preprocess_utils.h:189-190) */
     uint32_t item_group_num;  /* -ig */
     uint32_t k;               /* -k  */
-    uint32_t num_workers;     /* -wg */
+    uint32_t num_workers;     /* -wg; 0 = mf_auto_workers(n) */
     uint32_t epoch;           /* -l  */
     uint32_t thread_block_size; /* -bl: accepted for compatibility; workgroups are always 4 wavefronts here */
     uint32_t version;         /* -v: 1 MASCOT, 2 AFP, 3 MuPPET, 4 MPT, 5 fp32 SGD (0 = alias of 5) */

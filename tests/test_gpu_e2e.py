@@ -105,6 +105,31 @@ def test_mascot_reduced_config2(orc):
         assert got_prec.sum() >= 1 and ref_gm.prec.sum() >= 1
 
 
+def test_mascot_half_config2_with_chosen_workers(orc):
+    """BASELINE config 2 at half size (35k x 5.35k, 4M/1M ratings, Zipf 0.9, MASCOT k=128, 100+100 groups) with the
+    worker count mf_train chooses (num_workers = 0) and hot rows on, against the reference rule as a 16-thread
+    Hogwild loop of the checker on the same shuffle and initial model: test RMSE after 12 epochs within 0.005.
+    (The full-size run, 139 s mostly in the checker, gives 0.87869 against 0.87544.)"""
+    h = mfutil.hip()
+    n_users, n_items = 35000, 5350
+    R = mfutil.make_ratings(2, n_users, n_items, 5_000_000, rank=16, alpha=0.9, step=0.5, lo=0.5, hi=5.0, mean=3.5, noise=0.8)
+    train, test = _split(R, 4_000_000)
+    k, E = 128, 12
+    assert h.mf_auto_workers(train.size) == 244
+    prm = h.default_params(k=k, num_workers=0, epoch=E, learning_rate=0.01, lam=0.015, decay=0.1, version=1, seed=3,
+                           user_group_num=100, item_group_num=100, sample_ratio=0.05, interval=2, error_threshold=20.0)
+    assert prm.hot_row_inflight > 0
+    p, q = h.init_model(n_users, n_items, k, 3)
+    p0, q0 = p.copy(), q.copy()
+    out = h.train(prm, train, n_users, n_items, test, p, q)
+    # the checker plays the same 244 workers (same windows per epoch), 16 of them at a time
+    ref, info = mfutil.oracle_train_mascot(orc, train, test, p0, q0, k, 244, E, 0.01, 0.015, 0.1, 3, 100, 100, 0.05, 2, 20.0, threads=16)
+    print("gpu", out["rmse"], "\ncpu", ref)
+    assert np.array_equal(out["user_end"], info["uend"]) and np.array_equal(out["item_end"], info["iend"])
+    assert np.all(np.diff(out["rmse"]) < 0)
+    assert abs(out["rmse"][-1] - ref[-1]) < 0.005
+
+
 def _write_tsv(path, R, offset=0):
     with open(path, "w") as f:
         for r, u, i in zip(R["r"].tolist(), R["u"].tolist(), R["i"].tolist()):

@@ -20,6 +20,12 @@ def lib():
 
 
 # ---- schedules ---------------------------------------------------------------------------------
+def test_auto_workers(lib):
+    for n, want in ((1, 16), (400_000, 24), (8_000_000, 488), (100_000_000, 6104), (250_000_000, 6144)):
+        assert lib.mf_auto_workers(n) == want
+        assert lib.mf_auto_workers(n) % 4 == 0
+
+
 def test_update_count_is_smallest_cover_and_matches_survey_table(orc, lib):
     # configs of the benchmark definition with the default 2048 workers: 2, 31, 77, 382, 954 windows
     for n, want in ((400_000, 2), (8_000_000, 31), (20_000_000, 77), (100_000_000, 382), (250_000_000, 954)):
