@@ -292,12 +292,41 @@ __global__ __launch_bounds__(kStreamBlock) void iota_kernel(uint32_t* __restrict
     const uint32_t stride = gridDim.x * blockDim.x;
     for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) a[i] = i;
 }
-__global__ __launch_bounds__(kStreamBlock) void histogram_kernel(const mf_node* __restrict__ R, uint32_t n, uint32_t* user_bin, uint32_t* item_bin)
+// user_item_histogram (preprocess_utils.h:13-19).  With Zipf-like popularity a few counters take percents of all
+// increments, and global atomics on one address serialise at the memory side.  Each workgroup therefore counts in
+// an LDS table first: kHistSlots (id, count) slots per side, a slot claimed by the first id that hashes to it (two
+// probes); ids that find both probes taken go to the global counter directly.  Popular ids claim their slots within
+// the first few ratings, so nearly all of their increments are LDS atomics, flushed once per workgroup.
+constexpr int kHistBlock = 1024;
+constexpr uint32_t kHistLog = 12, kHistSlots = 1u << kHistLog;
+__device__ __forceinline__ void histogram_count(uint32_t* tag, uint32_t* cnt, uint32_t id, uint32_t* global_bin)
 {
-    const uint32_t stride = gridDim.x * blockDim.x;
-    for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
-        atomicAdd(&user_bin[R[i].u], 1u);
-        atomicAdd(&item_bin[R[i].i], 1u);
+    uint32_t s = (id * 2654435761u) >> (32 - kHistLog);
+#pragma unroll
+    for (int probe = 0; probe < 2; ++probe, s ^= 1u) {
+        uint32_t t = tag[s];
+        if (t == 0u) t = atomicCAS(&tag[s], 0u, id + 1u);
+        if (t == 0u || t == id + 1u) { atomicAdd(&cnt[s], 1u); return; }
+    }
+    atomicAdd(&global_bin[id], 1u);
+}
+__global__ __launch_bounds__(kHistBlock) void histogram_kernel(const mf_node* __restrict__ R, uint32_t n, uint32_t per_block, uint32_t* user_bin, uint32_t* item_bin)
+{
+    __shared__ uint32_t tab[4 * kHistSlots];          // user tags, user counts, item tags, item counts: 64 KB
+    for (uint32_t i = threadIdx.x; i < 4 * kHistSlots; i += blockDim.x) tab[i] = 0u;
+    __syncthreads();
+    uint32_t* utag = tab, *ucnt = tab + kHistSlots, *itag = tab + 2 * kHistSlots, *icnt = tab + 3 * kHistSlots;
+    const uint64_t begin = (uint64_t)blockIdx.x * per_block;
+    const uint64_t end = begin + per_block < n ? begin + per_block : n;
+    for (uint64_t i = begin + threadIdx.x; i < end; i += blockDim.x) {
+        const uint32_t* w = reinterpret_cast<const uint32_t*>(R + i);
+        histogram_count(utag, ucnt, __builtin_nontemporal_load(w + 1), user_bin);
+        histogram_count(itag, icnt, __builtin_nontemporal_load(w + 2), item_bin);
+    }
+    __syncthreads();
+    for (uint32_t s = threadIdx.x; s < kHistSlots; s += blockDim.x) {
+        if (utag[s]) atomicAdd(&user_bin[utag[s] - 1u], ucnt[s]);
+        if (itag[s]) atomicAdd(&item_bin[itag[s] - 1u], icnt[s]);
     }
 }
 __global__ __launch_bounds__(kStreamBlock) void reindex_kernel(mf_node* R, const uint32_t* __restrict__ user2sorted, const uint32_t* __restrict__ item2sorted, uint32_t n)
@@ -421,7 +450,11 @@ int mf_user_item_histogram(const mf_node* R, uint32_t n, uint32_t* user_bin, uin
 {
     if (n == 0) return MF_OK;
     if (!R || !user_bin || !item_bin) return invalid("mf_user_item_histogram: null pointer");
-    hipLaunchKernelGGL(histogram_kernel, dim3(stream_grid(n)), dim3(kStreamBlock), 0, as_stream(stream), R, n, user_bin, item_bin);
+    // one workgroup per 256k ratings (a flush costs up to 8192 global atomics), at least one per CU when n allows
+    uint32_t per_block = 1u << 18;
+    while (per_block > 16384u && (uint64_t)per_block * 256u > n) per_block >>= 1;
+    const uint32_t blocks = (uint32_t)(((uint64_t)n + per_block - 1) / per_block);
+    hipLaunchKernelGGL(histogram_kernel, dim3(blocks), dim3(kHistBlock), 0, as_stream(stream), R, n, per_block, user_bin, item_bin);
     return launch_status("mf_user_item_histogram");
 }
 
