@@ -1,5 +1,5 @@
 """Builds libmascot_hip.so (the gfx950 kernels behind the C ABI of include/mascot_hip.h)
-and the quantized_mf command line in-tree with hipcc.  No GPU is needed to build."""
+and the quantized_mf / test_mf command lines in-tree with hipcc.  No GPU is needed to build."""
 import os
 import subprocess
 import sys
@@ -10,6 +10,7 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "_build")
 LIB = os.path.join(HERE, "libmascot_hip.so")
 CLI = os.path.join(HERE, "quantized_mf")
+EVAL = os.path.join(HERE, "test_mf")
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 ARCH = "gfx950"
@@ -25,6 +26,7 @@ DEVICE_FLAGS = ["--offload-arch=" + ARCH, "-O3", "-std=c++17", "-fPIC", "-ffp-co
 KERNEL_SOURCES = ["hogwild_launch.hip", "aux_kernels.hip", "sort_shuffle.hip"]
 HOST_SOURCES = ["train.cpp"]
 CLI_SOURCES = ["main.cpp", "io_utils.cpp"]
+EVAL_SOURCES = ["test_mf_main.cpp", "io_utils.cpp"]
 
 
 def _run(cmd):
@@ -52,6 +54,9 @@ def build(verbose=False):
         with ThreadPoolExecutor(max_workers=2) as ex:
             cobjs = list(ex.map(_compile, CLI_SOURCES))
         _run([HIPCC, "-o", CLI] + cobjs + ["-L" + HERE, "-lmascot_hip", "-Wl,-rpath,$ORIGIN"])
+    if all(os.path.exists(os.path.join(CSRC, s)) for s in EVAL_SOURCES):
+        eobjs = [_compile(s) for s in EVAL_SOURCES]
+        _run([HIPCC, "-o", EVAL] + eobjs + ["-L" + HERE, "-lmascot_hip", "-Wl,-rpath,$ORIGIN"])
     if verbose:
         print("built", LIB)
     return LIB

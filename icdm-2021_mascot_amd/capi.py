@@ -24,6 +24,7 @@ SIGNATURES = {
     "mf_mascot_norm_blocks": (u32, [u32]),
     "mf_update_count": (u32, [u32, u32, u32]),
     "mf_auto_workers": (u32, [u32]),
+    "mf_gpu_test_rmse": (C.c_int, [vp, u32, vp, vp, u32, u32, C.c_int, vp]),
     "mf_first_sample_rating_idx": (u32, [u32, u32, u32, u32, u32, f32]),
     "mf_lr_schedule": (f32, [f32, f32, u32]),
     "mf_window_start": (u32, [u64, u32, u32, u32, u32]),

@@ -206,3 +206,73 @@ bool save_reconst_testset(const std::vector<mf_node>& test, const std::string& t
     }
     return true;
 }
+
+bool read_trained_model(TrainedModel& m, const std::string& path)
+{
+    std::ifstream f(path);
+    if (!f) return false;
+    std::string line;
+    if (!std::getline(f, line)) return false;
+    const std::vector<std::string> tok = split(line, ' ');
+    if (tok.size() < 3) return false;
+    m.n_users = (uint32_t)std::stoul(tok[0]);
+    m.n_items = (uint32_t)std::stoul(tok[1]);
+    m.k = (uint32_t)std::atoi(tok[2].c_str());
+    m.p.assign((size_t)m.n_users * m.k, 0.f);
+    m.q.assign((size_t)m.n_items * m.k, 0.f);
+    for (float& v : m.p) if (!(f >> v)) return false;
+    for (float& v : m.q) if (!(f >> v)) return false;
+    return true;
+}
+
+std::vector<mf_node> read_testset_pretrained_model(const std::string& path)
+{
+    std::vector<mf_node> test;
+    std::ifstream f(path);
+    if (!f) return test;
+    int user_idx, item_idx;
+    column_order(path, user_idx, item_idx);
+    std::string line;
+    if (path.find("Yahoo") != std::string::npos && path.find("reconst") == std::string::npos) {
+        while (std::getline(f, line)) {
+            const std::vector<std::string> head = split(line, '|');
+            if (head.size() < 2) continue;
+            const uint32_t u = (uint32_t)std::stoi(head[0]);
+            const uint32_t cnt = (uint32_t)std::stoi(head[1]);
+            for (uint32_t j = 0; j < cnt; ++j) {
+                if (!std::getline(f, line)) break;
+                const std::vector<std::string> tok = split(line, '\t');
+                if (tok.size() < 2) continue;
+                test.push_back({((float)std::atof(tok[1].c_str()) / 25.f) + 1.0f, u, (uint32_t)std::stoi(tok[0])});
+            }
+        }
+    } else {
+        while (std::getline(f, line)) {
+            const std::vector<std::string> tok = split(line, '\t');
+            if (tok.size() != 3) continue;
+            test.push_back({parse_rating(tok[2]), (uint32_t)std::stoi(tok[user_idx]), (uint32_t)std::stoi(tok[item_idx])});
+        }
+    }
+    return test;
+}
+
+bool remove_elements(std::vector<mf_node>& test, unsigned version, const std::string& test_path)
+{
+    if (version == 1) return true;
+    std::vector<uint32_t> gone[2];
+    const std::string dir = parent_dir(test_path);
+    for (int which = 0; which < 2; ++which) {
+        const std::string path = dir + (which ? "/remove_item.txt" : "/remove_user.txt");
+        std::ifstream f(path);
+        if (f.fail()) { std::cout << "fail to write file named " << path << std::endl; return false; }   // the reference's wording
+        std::string line;
+        while (std::getline(f, line)) {
+            line.erase(line.find_last_not_of(" \n\r\t") + 1);
+            if (!line.empty()) gone[which].push_back((uint32_t)std::stoi(line));
+        }
+        std::sort(gone[which].begin(), gone[which].end());
+    }
+    auto listed = [](const std::vector<uint32_t>& v, uint32_t id) { return std::binary_search(v.begin(), v.end(), id); };
+    test.erase(std::remove_if(test.begin(), test.end(), [&](const mf_node& t) { return listed(gone[0], t.u) || listed(gone[1], t.i); }), test.end());
+    return true;
+}

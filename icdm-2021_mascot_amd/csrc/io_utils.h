@@ -27,3 +27,13 @@ bool save_trained_model(const Dataset& d, const float* p, const float* q, uint32
 bool save_trained_model_reconst(uint32_t n_users, uint32_t n_items, const float* p, const float* q, uint32_t k, const std::string& outfile);
 // save_reconst_testset, io_utils.h:374-405: reconst_<testfile> next to the test file
 bool save_reconst_testset(const std::vector<mf_node>& test, const std::string& testfile);
+
+// ---- the stand-alone evaluator (test_mf/test.cu) -------------------------------------------------------------
+struct TrainedModel { uint32_t n_users = 0, n_items = 0, k = 0; std::vector<float> p, q; };
+// read_trained_model, io_utils.h:334-372: header "users items k", then users*k and items*k numbers
+bool read_trained_model(TrainedModel& m, const std::string& path);
+// read_testset_pretrained_model, io_utils.h:407-457: raw ids as they stand in the file (no re-mapping)
+std::vector<mf_node> read_testset_pretrained_model(const std::string& path);
+// remove_elements, io_utils.h:459-514: for version != 1 drops the users / items listed in remove_user.txt /
+// remove_item.txt next to the test file; false when one of the two files cannot be opened
+bool remove_elements(std::vector<mf_node>& test, unsigned version, const std::string& test_path);

@@ -551,6 +551,32 @@ int mf_init_model(float* p, float* q, uint32_t n_users, uint32_t n_items, uint32
     return 0;
 }
 
+int mf_gpu_test_rmse(const mf_node* test, uint32_t test_n, const float* p, const float* q, uint32_t n_users, uint32_t n_items, int k, double* rmse)
+{
+    if (!rmse) return invalid("mf_gpu_test_rmse: null result pointer");
+    *rmse = 0;
+    if (test_n == 0) return invalid("mf_gpu_test_rmse: empty test set");
+    if (!test || !p || !q) return invalid("mf_gpu_test_rmse: null pointer");
+    if (k != 64 && k != 128) return invalid("mf_gpu_test_rmse: k must be 64 or 128 (got %d)", k);
+    for (uint32_t i = 0; i < test_n; ++i)        // the kernel indexes P and Q with these
+        if (test[i].u >= n_users || test[i].i >= n_items)
+            return invalid("mf_gpu_test_rmse: test rating %u names user %u / item %u, the model has %u users and %u items", i, test[i].u, test[i].i, n_users, n_items);
+    DevBuf d_test, d_p, d_q, d_sum;
+    MF_TRY(d_test.alloc((size_t)test_n * sizeof(mf_node), "hipMalloc(test set)"));
+    MF_TRY(d_p.alloc((size_t)n_users * k * 4, "hipMalloc(P)"));
+    MF_TRY(d_q.alloc((size_t)n_items * k * 4, "hipMalloc(Q)"));
+    MF_TRY(d_sum.alloc(8, "hipMalloc(sum)"));
+    HIP_TRY(hipMemcpy(d_test.p, test, (size_t)test_n * sizeof(mf_node), hipMemcpyHostToDevice), "H2D test set");
+    HIP_TRY(hipMemcpy(d_p.p, p, (size_t)n_users * k * 4, hipMemcpyHostToDevice), "H2D P");
+    HIP_TRY(hipMemcpy(d_q.p, q, (size_t)n_items * k * 4, hipMemcpyHostToDevice), "H2D Q");
+    HIP_TRY(hipMemset(d_sum.p, 0, 8), "memset sum");
+    MF_TRY(mf_test_rmse(d_test.as<mf_node>(), test_n, d_p.as<float>(), d_q.as<float>(), k, d_sum.as<double>(), nullptr));
+    double sum = 0;
+    HIP_TRY(hipMemcpy(&sum, d_sum.p, 8, hipMemcpyDeviceToHost), "D2H sum");
+    *rmse = std::sqrt(sum / (double)test_n);
+    return MF_OK;
+}
+
 uint32_t mf_auto_workers(uint32_t n)
 {
     // about 128 windows of 128 ratings per worker: the ratio at which the runs on 8M and on 100M ratings stay

@@ -162,7 +162,12 @@ int mf_group_error(float* grad_sum_norm, const float* norm_sum, uint32_t norm_bl
  * ratings into *sum_sq (one device double, caller zeroes); rmse = sqrt(sum_sq / test_n). */
 int mf_test_rmse(const mf_node* test, uint32_t test_n, const float* p, const float* q, int k,
                  double* sum_sq, void* stream);
-/* Same, reading grouped storage directly (no host gather, no H2D of P and Q). */
+/* gpu_test_rmse, rmse.h:168-189, as the stand-alone evaluator calls it (test_mf/test.cu:68): host pointers in,
+ * uploads P [n_users][k], Q [n_items][k] and the test ratings, returns sqrt(sum((r - p.q)^2) / test_n) in *rmse.
+ * Unlike the reference it rejects test ratings whose ids lie outside the model. */
+int mf_gpu_test_rmse(const mf_node* test, uint32_t test_n, const float* p, const float* q, uint32_t n_users, uint32_t n_items,
+                     int k, double* rmse);
+/* Same as mf_test_rmse, reading grouped storage directly (no host gather, no H2D of P and Q). */
 int mf_test_rmse_grouped(const mf_node* test, uint32_t test_n, void* const* p, void* const* q, int k,
                          const uint32_t* user_group_end_idx, const uint32_t* item_group_end_idx,
                          const uint8_t* user_group_prec_info, const uint8_t* item_group_prec_info,

@@ -16,6 +16,18 @@ pytestmark = pytest.mark.gpu
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 CLI = os.path.join(os.path.dirname(HERE), "icdm-2021_mascot_amd", "quantized_mf")
+EVAL = os.path.join(os.path.dirname(HERE), "icdm-2021_mascot_amd", "test_mf")
+
+
+def _evaluate(model, testfile, version):
+    """Runs the stand-alone evaluator (test_mf/test.cu) and returns the RMSE it prints."""
+    assert os.path.exists(EVAL), "test_mf is not built"
+    res = subprocess.run([EVAL, "-i", model, "-y", testfile, "-v", str(version)], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=120)
+    assert res.returncode == 0, res.stderr
+    assert "Input file                  : " + model in res.stdout and "Version                     : %d" % version in res.stdout
+    line = [l for l in res.stdout.splitlines() if l.startswith("RMSE : ")]
+    assert len(line) == 1, res.stdout
+    return float(line[0].split(":")[1])
 
 
 def _split(R, n_train):
@@ -176,6 +188,8 @@ def test_quantized_mf_command_line(orc, tmp_path, version):
         tn["u"], tn["i"], tn["r"] = rt[:, 0], rt[:, 1], rt[:, 2]
         # 6 significant digits in the text file (default ostream precision)
         assert abs(orc.rmse(k, tn, P, Q) - rm[-1]) < 2e-4
+        # the evaluator reloads the model and the re-indexed test file: same number up to the 6 digits of the text files
+        assert abs(_evaluate(model, str(tmp_path / "reconst_test.tsv"), 1) - rm[-1]) < 2e-4
     else:
         model = out + ".txt"
         head = open(model).readline().split()
@@ -191,3 +205,9 @@ def test_quantized_mf_command_line(orc, tmp_path, version):
         tn["u"] = tn["u"] * 3 + 1
         tn["i"] = tn["i"] * 2 + 5
         assert abs(orc.rmse(k, tn, P, Q) - rm[-1]) < 2e-4
+        # the evaluator reads every line of the test file (duplicates included), minus the users / items listed in
+        # remove_user.txt / remove_item.txt, and indexes the model by original id
+        every = np.ascontiguousarray(test[keep])
+        every["u"] = every["u"] * 3 + 1
+        every["i"] = every["i"] * 2 + 5
+        assert abs(_evaluate(model, te, version) - orc.rmse(k, every, P, Q)) < 1e-5
