@@ -7,6 +7,7 @@
 #include <fstream>
 #include <iostream>
 #include <sstream>
+#include <sys/stat.h>
 
 namespace {
 
@@ -50,6 +51,21 @@ std::string file_name(const std::string& path)
 
 }  // namespace
 
+namespace {
+// the stdout line and the two side-effect files of read_test_dataset (io_utils.h:200-238)
+void report_missing_and_write_remove_files(const Dataset& d, const std::string& test_path)
+{
+    std::cout << "Missing the number of ratings : " << d.test_missing << std::endl;
+    const std::string dir = parent_dir(test_path);
+    for (int which = 0; which < 2; ++which) {
+        const std::string out = dir + (which ? "/remove_item.txt" : "/remove_user.txt");
+        std::ofstream f(out);
+        if (f.fail()) { std::cout << "fail to write file named " << out << std::endl; return; }
+        for (uint32_t v : (which ? d.remove_item : d.remove_user)) f << v << std::endl;
+    }
+}
+}  // namespace
+
 bool read_training_dataset(Dataset& d, const std::string& path)
 {
     std::ifstream file(path);
@@ -90,8 +106,11 @@ bool read_training_dataset(Dataset& d, const std::string& path)
 
 bool read_test_dataset(Dataset& d, const std::string& path)
 {
-    std::vector<uint32_t> remove_user, remove_item;
-    uint32_t missing = 0;
+    std::vector<uint32_t>& remove_user = d.remove_user;
+    std::vector<uint32_t>& remove_item = d.remove_item;
+    uint32_t& missing = d.test_missing;
+    if (d.user_map.empty()) for (uint32_t i = 0; i < d.user_orig.size(); ++i) d.user_map.emplace(d.user_orig[i], i);
+    if (d.item_map.empty()) for (uint32_t i = 0; i < d.item_orig.size(); ++i) d.item_map.emplace(d.item_orig[i], i);
     std::ifstream file(path);
     int user_idx, item_idx;
     column_order(path, user_idx, item_idx);
@@ -137,18 +156,10 @@ bool read_test_dataset(Dataset& d, const std::string& path)
             }
         }
     }
-    std::cout << "Missing the number of ratings : " << missing << std::endl;
     // test_set_preprocess, preprocess_utils.h:38-52: users ascending (dense id), items ascending within a user
     for (uint32_t u = 0; u < d.max_user; ++u)
         for (const auto& kv : test_R[u]) d.test.push_back({kv.second, u, kv.first});
-
-    const std::string dir = parent_dir(path);
-    for (int which = 0; which < 2; ++which) {
-        const std::string out = dir + (which ? "/remove_item.txt" : "/remove_user.txt");
-        std::ofstream f(out);
-        if (f.fail()) { std::cout << "fail to write file named " << out << std::endl; return true; }
-        for (uint32_t v : (which ? remove_item : remove_user)) f << v << std::endl;
-    }
+    report_missing_and_write_remove_files(d, path);
     return true;
 }
 
@@ -158,12 +169,13 @@ bool save_trained_model(const Dataset& d, const float* p, const float* q, uint32
     const std::string outpath = outfile + ".txt";
     std::ofstream f(outpath);
     if (f.fail()) { std::cout << "fail to write file named " << outpath << std::endl; std::cerr << "Error: " << std::strerror(errno); return false; }
-    auto sorted_by_orig = [](const std::unordered_map<uint32_t, uint32_t>& m) {
-        std::vector<std::pair<uint32_t, uint32_t>> v(m.begin(), m.end());
+    auto sorted_by_orig = [](const std::vector<uint32_t>& orig) {       // (original id, dense id), ascending original id
+        std::vector<std::pair<uint32_t, uint32_t>> v(orig.size());
+        for (uint32_t i = 0; i < orig.size(); ++i) v[i] = {orig[i], i};
         std::sort(v.begin(), v.end());
         return v;
     };
-    const auto users = sorted_by_orig(d.user_map), items = sorted_by_orig(d.item_map);
+    const auto users = sorted_by_orig(d.user_orig), items = sorted_by_orig(d.item_orig);
     f << users.back().first + 1 << " " << items.back().first + 1 << " " << k << std::endl;
     auto dump = [&](const std::vector<std::pair<uint32_t, uint32_t>>& ids, const float* m) {
         int prev = 0;
@@ -274,5 +286,78 @@ bool remove_elements(std::vector<mf_node>& test, unsigned version, const std::st
     }
     auto listed = [](const std::vector<uint32_t>& v, uint32_t id) { return std::binary_search(v.begin(), v.end(), id); };
     test.erase(std::remove_if(test.begin(), test.end(), [&](const mf_node& t) { return listed(gone[0], t.u) || listed(gone[1], t.i); }), test.end());
+    return true;
+}
+
+// ---- binary cache of the parsed data set ----------------------------------------------------------------------
+namespace {
+struct FileId { uint64_t size = 0; int64_t mtime_s = 0, mtime_ns = 0; bool ok = false; };
+FileId file_id(const std::string& path)
+{
+    FileId id;
+    struct stat st;
+    if (stat(path.c_str(), &st) == 0) { id.size = (uint64_t)st.st_size; id.mtime_s = (int64_t)st.st_mtim.tv_sec; id.mtime_ns = (int64_t)st.st_mtim.tv_nsec; id.ok = true; }
+    return id;
+}
+struct CacheHeader {
+    char magic[8];                 // "MFCACHE1"
+    uint64_t train_size, test_size;
+    int64_t train_mtime_s, train_mtime_ns, test_mtime_s, test_mtime_ns;
+    uint64_t test_path_hash;
+    uint64_t n_train, n_test, n_remove_user, n_remove_item;
+    uint32_t n_users, n_items, test_lines_kept, test_missing;
+};
+uint64_t fnv1a(const std::string& s)
+{
+    uint64_t h = 1469598103934665603ull;
+    for (unsigned char c : s) { h ^= c; h *= 1099511628211ull; }
+    return h;
+}
+template <class T> bool write_vec(std::ofstream& f, const std::vector<T>& v) { if (!v.empty()) f.write(reinterpret_cast<const char*>(v.data()), (std::streamsize)(v.size() * sizeof(T))); return (bool)f; }
+template <class T> bool read_vec(std::ifstream& f, std::vector<T>& v, uint64_t n) { v.resize(n); if (n) f.read(reinterpret_cast<char*>(v.data()), (std::streamsize)(n * sizeof(T))); return (bool)f; }
+}  // namespace
+
+bool load_dataset(Dataset& d, const std::string& train_path, const std::string& test_path, bool use_cache, bool* from_cache)
+{
+    if (from_cache) *from_cache = false;
+    const std::string cache_path = train_path + ".mfcache";
+    const FileId tr = file_id(train_path), te = file_id(test_path);
+    if (use_cache && tr.ok) {
+        std::ifstream f(cache_path, std::ios::binary);
+        CacheHeader h;
+        if (f && f.read(reinterpret_cast<char*>(&h), sizeof h) && std::memcmp(h.magic, "MFCACHE1", 8) == 0 &&
+            h.train_size == tr.size && h.train_mtime_s == tr.mtime_s && h.train_mtime_ns == tr.mtime_ns &&
+            h.test_size == (te.ok ? te.size : 0) && h.test_mtime_s == te.mtime_s && h.test_mtime_ns == te.mtime_ns &&
+            h.test_path_hash == fnv1a(test_path)) {
+            Dataset c;
+            c.max_user = h.n_users; c.max_item = h.n_items; c.test_lines_kept = h.test_lines_kept; c.test_missing = h.test_missing;
+            if (read_vec(f, c.R, h.n_train) && read_vec(f, c.test, h.n_test) && read_vec(f, c.user_orig, h.n_users) &&
+                read_vec(f, c.item_orig, h.n_items) && read_vec(f, c.remove_user, h.n_remove_user) && read_vec(f, c.remove_item, h.n_remove_item)) {
+                d = std::move(c);
+                report_missing_and_write_remove_files(d, test_path);
+                if (from_cache) *from_cache = true;
+                return true;
+            }
+        }
+    }
+    if (!read_training_dataset(d, train_path)) return false;
+    read_test_dataset(d, test_path);
+    if (use_cache) {
+        const std::string tmp = cache_path + ".tmp";
+        std::ofstream f(tmp, std::ios::binary);
+        CacheHeader h = {};
+        std::memcpy(h.magic, "MFCACHE1", 8);
+        h.train_size = tr.size; h.train_mtime_s = tr.mtime_s; h.train_mtime_ns = tr.mtime_ns;
+        h.test_size = te.ok ? te.size : 0; h.test_mtime_s = te.mtime_s; h.test_mtime_ns = te.mtime_ns;
+        h.test_path_hash = fnv1a(test_path);
+        h.n_train = d.R.size(); h.n_test = d.test.size(); h.n_remove_user = d.remove_user.size(); h.n_remove_item = d.remove_item.size();
+        h.n_users = d.max_user; h.n_items = d.max_item; h.test_lines_kept = d.test_lines_kept; h.test_missing = d.test_missing;
+        bool ok = f && f.write(reinterpret_cast<const char*>(&h), sizeof h);
+        ok = ok && write_vec(f, d.R) && write_vec(f, d.test) && write_vec(f, d.user_orig) && write_vec(f, d.item_orig) &&
+             write_vec(f, d.remove_user) && write_vec(f, d.remove_item);
+        f.close();
+        if (ok && f) std::rename(tmp.c_str(), cache_path.c_str());
+        else { std::remove(tmp.c_str()); std::cout << "could not write " << cache_path << " (continuing without the cache)" << std::endl; }
+    }
     return true;
 }

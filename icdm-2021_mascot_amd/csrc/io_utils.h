@@ -15,12 +15,20 @@ struct Dataset {
     std::vector<uint32_t> user_orig, item_orig;   // dense id -> original id
     uint32_t max_user = 0, max_item = 0;          // number of distinct users / items
     uint32_t test_lines_kept = 0;                 // the reference's test_n (counts duplicates, io_utils.h:187)
+    uint32_t test_missing = 0;                    // test ratings dropped for an unseen user or item
+    std::vector<uint32_t> remove_user, remove_item;   // their original ids, as written to remove_user.txt / remove_item.txt
 };
 
 // read_training_dataset, io_utils.h:30-120
 bool read_training_dataset(Dataset& d, const std::string& path);
 // read_test_dataset, io_utils.h:122-240 (also writes remove_user.txt / remove_item.txt next to the file)
 bool read_test_dataset(Dataset& d, const std::string& path);
+// Both readers behind a binary cache of what they produce (no counterpart in the reference, whose parse of a
+// 100M-line file through getline/stoi/std::map takes minutes).  With use_cache the parsed and re-mapped ratings
+// are kept in <train path>.mfcache; a later call with the same two files (same paths, sizes and modification
+// times) loads that instead of parsing, prints the same "Missing the number of ratings" line and rewrites the two
+// remove_*.txt files.  Without use_cache this is read_training_dataset followed by read_test_dataset.
+bool load_dataset(Dataset& d, const std::string& train_path, const std::string& test_path, bool use_cache, bool* from_cache = nullptr);
 // save_trained_model, io_utils.h:242-303: <out>.txt, rows by original id, zero rows for absent ids
 bool save_trained_model(const Dataset& d, const float* p, const float* q, uint32_t k, const std::string& outfile);
 // save_trained_model_reconst, io_utils.h:305-332: <out>_reconst.txt, rows in the order given

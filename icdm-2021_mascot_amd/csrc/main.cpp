@@ -17,6 +17,7 @@ int main(int argc, const char* argv[])
     mf_params prm;
     mf_default_params(&prm);
     unsigned reconst_save = 0;
+    int use_cache = 0;                                // -cache 1: keep the parsed ratings in <input>.mfcache
     const char* usage = " [-t <threads> -p <predictions/user> -o <output-tsv>] <input-tsv>";
     if (argc < 2) { std::cout << argv[0] << usage << std::endl; return 0; }
     if (argc == 2) infile = argv[1];
@@ -46,6 +47,7 @@ int main(int argc, const char* argv[])
             if (a == "-cached" && has) prm.cached_rows = std::atoi(argv[i + 1]);
             if (a == "-split" && has) prm.epoch_splits = std::atoi(argv[i + 1]);
             if (a == "-hot" && has) prm.hot_row_inflight = std::atof(argv[i + 1]);
+            if (a == "-cache" && has) use_cache = std::atoi(argv[i + 1]);
             if (a == "-h") { std::cout << argv[0] << usage << std::endl; return 0; }
         }
     }
@@ -68,8 +70,9 @@ int main(int argc, const char* argv[])
     std::cout << "Seed                        : " << prm.seed << std::endl;
 
     Dataset d;
-    read_training_dataset(d, infile);
-    read_test_dataset(d, testfile);
+    bool from_cache = false;
+    load_dataset(d, infile, testfile, use_cache != 0, &from_cache);
+    if (from_cache) std::cout << "Ratings loaded from " << infile << ".mfcache" << std::endl;
     std::cout << "The number of nonzeros      : " << d.R.size() << std::endl;
     std::cout << "The number of users         : " << d.max_user << std::endl;
     std::cout << "The number of items         : " << d.max_item << std::endl;

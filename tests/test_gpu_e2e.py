@@ -211,3 +211,36 @@ def test_quantized_mf_command_line(orc, tmp_path, version):
         every["u"] = every["u"] * 3 + 1
         every["i"] = every["i"] * 2 + 5
         assert abs(_evaluate(model, te, version) - orc.rmse(k, every, P, Q)) < 1e-5
+
+
+def test_command_line_rating_cache(tmp_path):
+    """-cache 1: the second run loads <train>.mfcache instead of parsing, reports the same data set, prints the same
+    "Missing" line and rewrites remove_user.txt; touching the training file invalidates the cache."""
+    R = mfutil.make_ratings(33, 300, 120, 20_000)
+    train, test = R[:16_000], R[16_000:]
+    tr, te = str(tmp_path / "train.tsv"), str(tmp_path / "test.tsv")
+    _write_tsv(tr, train)
+    _write_tsv(te, test)
+    with open(te, "a") as f:
+        f.write("999999\t5\t3\n")
+    cmd = [CLI, "-i", tr, "-y", te, "-v", "5", "-k", "64", "-l", "2", "-wg", "16", "-seed", "4", "-cache", "1"]
+
+    def run():
+        res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=300)
+        assert res.returncode == 0, res.stderr
+        facts = [l for l in res.stdout.splitlines() if l.startswith(("The number of", "Missing the number"))]
+        return res.stdout, facts
+
+    out1, facts1 = run()
+    assert "Ratings loaded from" not in out1 and os.path.exists(tr + ".mfcache")
+    assert len(facts1) == 5 and "Missing the number of ratings : 1" in facts1
+    os.remove(str(tmp_path / "remove_user.txt"))
+    out2, facts2 = run()
+    assert "Ratings loaded from " + tr + ".mfcache" in out2
+    assert facts2 == facts1
+    assert open(str(tmp_path / "remove_user.txt")).read().split() == ["999999"]
+    with open(tr, "a") as f:                       # a changed training file is parsed again
+        f.write("1\t5\t4\n")
+    out3, facts3 = run()
+    assert "Ratings loaded from" not in out3
+    assert facts3 != facts1
