@@ -110,20 +110,16 @@ class MascotProblem:
             torch.cuda.synchronize()
             s["initial"] = arena.clone()
         self.stats = None
+        self.hot = None
 
     def reset(self):
         for s in self.sides:
             s["arena"].copy_(s["initial"])
 
-    def set_thinning(self, W, inflight_cap):
+    def hot_tables(self, W, inflight_cap):
         """Hot-row tables from the rating counts (rows are in popularity-sorted order), as mf_train builds them:
         255 = ordinary row; rows with more than one update in flight are hot rows (updates added in memory), thinned to
-        at most `inflight_cap` updates in flight."""
-        torch, h = self.torch, self.h
-        if not inflight_cap:
-            h.mf_set_hot_row_thinning(None, None)
-            self.keep = None
-            return 1.0
+        at most `inflight_cap` updates in flight.  Returns (user table, item table, fraction of row updates carried out)."""
         F = min(W, 8192) * 4.0
         tabs, kept = [], 0.0
         for s in self.sides:
@@ -131,10 +127,25 @@ class MascotProblem:
             keep = np.where(inflight > inflight_cap, inflight_cap / np.maximum(inflight, 1e-30), 1.0)
             t = np.where(inflight > 1.0, np.clip(np.floor(keep * 255.0) - 1, 0, 254), 255).astype(np.uint8)
             kept += float((s["sorted_cnt"].astype(np.float64) * np.where(t == 255, 1.0, (t.astype(np.float64) + 1) / 255.0)).sum()) / self.n
-            tabs.append(torch.from_numpy(t).to(self.R.device))
-        self.keep = tabs
-        h.mf_set_hot_row_thinning(tabs[0].data_ptr(), tabs[1].data_ptr())
-        return kept / 2
+            tabs.append(self.torch.from_numpy(t).to(self.R.device))
+        return tabs[0], tabs[1], kept / 2
+
+    def set_hot_rows(self, W, cap, early_cap=0.0, early_epochs=0):
+        """The hot-row schedule of a leg: `early_cap` during the first `early_epochs` epochs, `cap` afterwards (0 = off)."""
+        self.hot = None
+        self.h.mf_set_hot_row_thinning(None, None)
+        if cap:
+            steady = self.hot_tables(W, cap)
+            early = self.hot_tables(W, early_cap) if early_epochs and early_cap > cap else steady
+            self.hot = dict(steady=steady, early=early, early_epochs=early_epochs if early is not steady else 0)
+
+    def select_hot_rows(self, e):
+        """Installs the tables of epoch e; returns the fraction of row updates that epoch carries out."""
+        if self.hot is None:
+            return 1.0
+        u, v, kept = self.hot["early"] if e < self.hot["early_epochs"] else self.hot["steady"]
+        self.h.mf_set_hot_row_thinning(u.data_ptr(), v.data_ptr())
+        return kept
 
     def alloc_stats(self, W):
         torch, h, k = self.torch, self.h, self.k
@@ -183,19 +194,22 @@ def time_steps(torch, prob, W, warmup, steps, cfg, seed):
     prob.reset()
     prob.alloc_stats(W)
     for e in range(warmup):
+        prob.select_hot_rows(e)
         prob.epoch(e, W, cfg["epochs"], cfg["lr"], cfg["decay"], cfg["lam"], cfg["sample_ratio"], cfg["interval"], seed)
     torch.cuda.synchronize()
     ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
     t0 = time.perf_counter()
     uc = 0
+    kept = []
     for i in range(steps):
+        kept.append(prob.select_hot_rows(warmup + i))
         ev[i][0].record()
         uc = prob.epoch(warmup + i, W, cfg["epochs"], cfg["lr"], cfg["decay"], cfg["lam"], cfg["sample_ratio"], cfg["interval"], seed)
         ev[i][1].record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     per = np.array([a.elapsed_time(b) for a, b in ev])
-    return per, wall, uc
+    return per, wall, uc, float(np.mean(kept))
 
 
 def cpu_baseline(prob, cfg, seed, threads, target_updates):
@@ -226,8 +240,11 @@ def time_fp32_sgd(torch, h, prob, W, warmup, steps, cfg, seed):
     h.mf_init_rand_feature(Q.data_ptr(), Q.numel(), seed, 1, st)
     uc = h.mf_update_count(prob.n, W, 128)
     ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    kept = []
     for e in range(warmup + steps):
+        kept_e = prob.select_hot_rows(e)
         if e >= warmup:
+            kept.append(kept_e)
             ev[e - warmup][0].record()
         h.mf_single_sgd_hogwild(prob.R.data_ptr(), prob.n, P.data_ptr(), Q.data_ptr(), k, W, uc, 128,
                                 h.mf_lr_schedule(cfg["lr"], cfg["decay"], e), cfg["lam"], seed, e, None, st)
@@ -237,7 +254,7 @@ def time_fp32_sgd(torch, h, prob, W, warmup, steps, cfg, seed):
     acc = torch.zeros(1, dtype=torch.float64, device=dev)
     h.mf_test_rmse(prob.test.data_ptr(), prob.test.shape[0], P.data_ptr(), Q.data_ptr(), k, acc.data_ptr(), st)
     rmse = float(np.sqrt(acc.item() / prob.test.shape[0]))
-    return np.array([a.elapsed_time(b) for a, b in ev]), uc, rmse
+    return np.array([a.elapsed_time(b) for a, b in ev]), uc, rmse, float(np.mean(kept))
 
 
 def reference_rule_rmse(prob, h, cfg, seed, threads, epochs, workers):
@@ -275,7 +292,7 @@ def measured_traffic(a, leg):
         return None
     if a.skip_coherent:
         return (14_053_967 * 2.0 + 24_189_917) * 1024 if leg["workers"] == 16384 else None
-    if leg["workers"] == 6144 and a.hot_row_inflight == 8.0:
+    if leg["workers"] == 6144 and a.hot_row_inflight == 8.0 and a.warmup >= a.hot_row_early_epochs:
         return (17_636_147 * 2.0 + 32_167_634) * 1024
     return None
 
@@ -293,7 +310,9 @@ def main():
     ap.add_argument("--skip-cached", action="store_true")
     ap.add_argument("--skip-coherent", action="store_true", help="profiling aid: time only the cached-rows leg")
     ap.add_argument("--skip-exact", action="store_true", help="skip the leg with every row update carried out (no thinning)")
-    ap.add_argument("--hot-row-inflight", type=float, default=8.0, help="hot rows of the measured run are thinned to this many updates in flight (0 = no hot rows)")
+    ap.add_argument("--hot-row-inflight", type=float, default=2.0, help="hot rows of the measured run are thinned to this many updates in flight (0 = no hot rows)")
+    ap.add_argument("--hot-row-inflight-early", type=float, default=16.0, help="the same cap during the first epochs")
+    ap.add_argument("--hot-row-early-epochs", type=int, default=2, help="number of epochs that run with the early cap")
     ap.add_argument("--pmc-copy", action="store_true",
                     help="profiling aid: also run three 1 GiB device copies, the known-size kernel that FETCH_SIZE / WRITE_SIZE are scaled by")
     ap.add_argument("--skip-fp32", action="store_true", help="skip the fp32-SGD leg")
@@ -323,10 +342,10 @@ def main():
 
     def leg(coherent, W, inflight_cap=0.0):
         h.mf_set_row_coherence(1 if coherent else 0)
-        kept = prob.set_thinning(W, inflight_cap)
-        per, wall, uc = time_steps(torch, prob, W, a.warmup, a.steps, cfg, a.seed)
+        prob.set_hot_rows(W, inflight_cap, a.hot_row_inflight_early, a.hot_row_early_epochs)
+        per, wall, uc, kept = time_steps(torch, prob, W, a.warmup, a.steps, cfg, a.seed)
         rmse = prob.rmse()
-        prob.set_thinning(W, 0.0)
+        prob.set_hot_rows(W, 0.0)
         updates = W * uc * 128
         ms = float(per.mean())
         bytes_per_update = read_bytes + row_bytes * kept
@@ -354,12 +373,13 @@ def main():
                    "workers": main_leg["workers"], "row_access": "cached" if a.skip_coherent else "device-coherent", "update_vector_size": 128,
                    "epochs_timed": "%d..%d of 50" % (a.warmup, a.warmup + a.steps - 1), "seed": a.seed,
                    "hot_row_inflight": 0.0 if a.skip_coherent else a.hot_row_inflight,
+                   "hot_row_inflight_early": 0.0 if a.skip_coherent else a.hot_row_inflight_early, "hot_row_early_epochs": a.hot_row_early_epochs,
                    "row_updates_carried_out": round(main_leg["row_updates_kept"], 4),
                    "user_groups": int(prob.sides[0]["groups"]), "item_groups": int(prob.sides[1]["groups"]), "setup_s": round(setup_s, 1)},
         "roofline": {"bound": "hbm", "achieved": main_leg["gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
                      "frac": main_leg["gbs"] / PEAK_HBM_GBS,
                      "traffic": measured_traffic(a, main_leg),
-                     "kernel": "hogwild_kernel<MascotRule<128,%s>>" % ("false" if a.skip_coherent else "true"),
+                     "kernel": "hogwild_kernel<MascotRuleT<128,%s,false>>" % ("false" if a.skip_coherent else "true"),
                      "bytes_per_update": round(main_leg["bytes_per_update"], 1),
                      "updates_per_launch": main_leg["updates_per_step"]},
         "ms_steps": main_leg["ms_steps"],
@@ -377,14 +397,14 @@ def main():
                                       "rows; faster, converges worse, see DESIGN.md)",
                               "value": c["ratings_per_s"], "unit": "ratings/s", "ms_per_step": c["ms_per_step"], "workers": c["workers"],
                               "roofline": {"bound": "hbm", "achieved": c["gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": c["gbs"] / PEAK_HBM_GBS,
-                                           "kernel": "hogwild_kernel<MascotRule<128,false>>"},
+                                           "kernel": "hogwild_kernel<MascotRuleT<128,false,false>>"},
                               "ms_steps": c["ms_steps"], "test_rmse_after_timed_epochs": c["rmse"]}
         h.mf_set_row_coherence(1)
     if not a.skip_fp32 and not a.skip_coherent:
         h.mf_set_row_coherence(1)
-        kept = prob.set_thinning(a.workers, a.hot_row_inflight)
-        per, uc, rmse = time_fp32_sgd(torch, h, prob, a.workers, a.warmup, a.steps, cfg, a.seed)
-        prob.set_thinning(a.workers, 0.0)
+        prob.set_hot_rows(a.workers, a.hot_row_inflight, a.hot_row_inflight_early, a.hot_row_early_epochs)
+        per, uc, rmse, kept = time_fp32_sgd(torch, h, prob, a.workers, a.warmup, a.steps, cfg, a.seed)
+        prob.set_hot_rows(a.workers, 0.0)
         ms = float(per.mean())
         bpu = 12 + 2 * k * 4 + 2 * k * 4 * kept
         out["fp32_sgd"] = {"note": "fp32 SGD (-v 5) on the same ratings, workers, row access and hot-row tables",

@@ -62,7 +62,7 @@ class MfParams(C.Structure):
     _fields_ = [("lambda_", f32), ("learning_rate", f32), ("decay", f32), ("sample_ratio", f32), ("error_threshold", f32),
                 ("interval", u32), ("user_group_num", u32), ("item_group_num", u32), ("k", u32), ("num_workers", u32),
                 ("epoch", u32), ("thread_block_size", u32), ("version", u32), ("is_yahoo", u32), ("seed", u64),
-                ("verbose", u32), ("cached_rows", u32), ("epoch_splits", u32), ("hot_row_inflight", f32)]
+                ("verbose", u32), ("cached_rows", u32), ("epoch_splits", u32), ("hot_row_inflight", f32), ("hot_row_inflight_early", f32), ("hot_row_early_epochs", u32)]
 
 
 class MfReport(C.Structure):

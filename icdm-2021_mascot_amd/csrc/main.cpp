@@ -4,6 +4,7 @@
 // and `-split <n>` (row access policy and kernel launches per epoch, see include/mascot_hip.h).
 #include <sys/stat.h>
 #include <cstdlib>
+#include <cstdio>
 #include <iostream>
 #include <string>
 #include <vector>
@@ -46,7 +47,13 @@ int main(int argc, const char* argv[])
             if (a == "-seed" && has) prm.seed = std::strtoull(argv[i + 1], nullptr, 10);
             if (a == "-cached" && has) prm.cached_rows = std::atoi(argv[i + 1]);
             if (a == "-split" && has) prm.epoch_splits = std::atoi(argv[i + 1]);
-            if (a == "-hot" && has) prm.hot_row_inflight = std::atof(argv[i + 1]);
+            if (a == "-hot" && has) {            // <steady cap>[,<early cap>,<early epochs>]
+                float steady = 0, early = 0; unsigned ep = 0;
+                const int got = std::sscanf(argv[i + 1], "%f,%f,%u", &steady, &early, &ep);
+                if (got >= 1) prm.hot_row_inflight = steady;
+                if (got >= 2) prm.hot_row_inflight_early = early;
+                if (got >= 3) prm.hot_row_early_epochs = ep;
+            }
             if (a == "-cache" && has) use_cache = std::atoi(argv[i + 1]);
             if (a == "-h") { std::cout << argv[0] << usage << std::endl; return 0; }
         }

@@ -134,19 +134,38 @@ std::vector<uint8_t> keep_table(const uint32_t* cnt, uint32_t rows, uint32_t n, 
     return t;
 }
 
-struct ThinningGuard {
-    DevBuf u, v;
+// The two pairs of hot-row tables of a run: the early cap for the first epochs, while every row still grows from its
+// small initial value and the popular rows need many updates, and the steady cap afterwards.
+struct HotRows {
+    DevBuf early_u, early_v, steady_u, steady_v;
     bool active = false;
-    ~ThinningGuard() { if (active) (void)mf_set_hot_row_thinning(nullptr, nullptr); }
-    int install(const std::vector<uint8_t>& ku, const std::vector<uint8_t>& kv)
+    uint32_t early_epochs = 0;
+    ~HotRows() { if (active) (void)mf_set_hot_row_thinning(nullptr, nullptr); }
+    static int upload(DevBuf& d, const std::vector<uint8_t>& t)
     {
-        MF_TRY(u.alloc(ku.size(), "hipMalloc(user keep table)"));
-        MF_TRY(v.alloc(kv.size(), "hipMalloc(item keep table)"));
-        HIP_TRY(hipMemcpy(u.p, ku.data(), ku.size(), hipMemcpyHostToDevice), "H2D user keep table");
-        HIP_TRY(hipMemcpy(v.p, kv.data(), kv.size(), hipMemcpyHostToDevice), "H2D item keep table");
-        MF_TRY(mf_set_hot_row_thinning(u.as<uint8_t>(), v.as<uint8_t>()));
+        MF_TRY(d.alloc(t.size(), "hipMalloc(hot-row table)"));
+        HIP_TRY(hipMemcpy(d.p, t.data(), t.size(), hipMemcpyHostToDevice), "H2D hot-row table");
+        return 0;
+    }
+    int install(const mf_params& prm, const uint32_t* ucnt, uint32_t n_users, const uint32_t* icnt, uint32_t n_items, uint32_t n)
+    {
+        if (!(prm.hot_row_inflight > 0)) return 0;
+        early_epochs = prm.hot_row_inflight_early > prm.hot_row_inflight ? prm.hot_row_early_epochs : 0;
+        MF_TRY(upload(steady_u, keep_table(ucnt, n_users, n, prm.num_workers, prm.hot_row_inflight)));
+        MF_TRY(upload(steady_v, keep_table(icnt, n_items, n, prm.num_workers, prm.hot_row_inflight)));
+        if (early_epochs) {
+            MF_TRY(upload(early_u, keep_table(ucnt, n_users, n, prm.num_workers, prm.hot_row_inflight_early)));
+            MF_TRY(upload(early_v, keep_table(icnt, n_items, n, prm.num_workers, prm.hot_row_inflight_early)));
+        }
         active = true;
         return 0;
+    }
+    // tables for the launches of epoch e (a launch takes the pointers with it, so switching between launches is safe)
+    int select(uint32_t e)
+    {
+        if (!active) return 0;
+        const bool early = e < early_epochs;
+        return mf_set_hot_row_thinning((early ? early_u : steady_u).as<uint8_t>(), (early ? early_v : steady_v).as<uint8_t>());
     }
 };
 
@@ -189,7 +208,7 @@ int train_dense(Common& c, float* p, float* q)
         muppet_first_sample = c.update_count * c.update_vector_size - (uint32_t)sample_ratings_num;
     }
 
-    ThinningGuard thinning;
+    HotRows hot;
     if (prm.hot_row_inflight > 0 && (version == 5 || version == 4)) {
         DevBuf d_ucnt, d_icnt;
         MF_TRY(d_ucnt.alloc((size_t)c.n_users * 4, "hipMalloc(user counts)"));
@@ -200,12 +219,12 @@ int train_dense(Common& c, float* p, float* q)
         std::vector<uint32_t> ucnt(c.n_users), icnt(c.n_items);
         HIP_TRY(hipMemcpy(ucnt.data(), d_ucnt.p, (size_t)c.n_users * 4, hipMemcpyDeviceToHost), "D2H user counts");
         HIP_TRY(hipMemcpy(icnt.data(), d_icnt.p, (size_t)c.n_items * 4, hipMemcpyDeviceToHost), "D2H item counts");
-        MF_TRY(thinning.install(keep_table(ucnt.data(), c.n_users, c.n, prm.num_workers, prm.hot_row_inflight),
-                                keep_table(icnt.data(), c.n_items, c.n, prm.num_workers, prm.hot_row_inflight)));
+        MF_TRY(hot.install(prm, ucnt.data(), c.n_users, icnt.data(), c.n_items, c.n));
     }
     Timer t;
     const mf_node* R = c.d_R.as<mf_node>();
     for (uint32_t e = 0; e < prm.epoch; ++e) {
+        MF_TRY(hot.select(e));
         const double err0 = now_ms();
         if (version == 3) HIP_TRY(hipMemsetAsync(d_sum_updated.p, 0, c.k * 4, nullptr), "memset sum_updated_val");
         double err_ms = now_ms() - err0;
@@ -418,17 +437,15 @@ int train_mascot(Common& c, float* p, float* q)
                                            d_i2s.as<uint32_t>(), (int)c.k, c.n_items, I.groups, nullptr));
         HIP_TRY(hipDeviceSynchronize(), "synchronize");
     }
-    ThinningGuard thinning;
-    if (prm.hot_row_inflight > 0) {      // rows are in popularity-sorted order: the sorted counts index them directly
-        MF_TRY(thinning.install(keep_table(U.sorted_cnt.data(), c.n_users, c.n, prm.num_workers, prm.hot_row_inflight),
-                                keep_table(I.sorted_cnt.data(), c.n_items, c.n, prm.num_workers, prm.hot_row_inflight)));
-    }
+    HotRows hot;      // rows are in popularity-sorted order: the sorted counts index them directly
+    MF_TRY(hot.install(prm, U.sorted_cnt.data(), c.n_users, I.sorted_cnt.data(), c.n_items, c.n));
     if (c.rep) c.rep->preprocess_ms = now_ms() - pre0;
 
     const uint32_t start_idx = 5;                                   // mf_methods.cu:110
     const uint32_t total = c.update_count * c.update_vector_size;
     Timer t;
     for (uint32_t e = 0; e < prm.epoch; ++e) {
+        MF_TRY(hot.select(e));
         const uint32_t first_sample = mf_first_sample_rating_idx(e, prm.interval, prm.epoch, c.update_count, c.update_vector_size, prm.sample_ratio);
         const bool error_check = first_sample < total || (prm.interval && e >= start_idx && (e % prm.interval == start_idx % prm.interval) && prm.epoch - 1 != e);
         double err_ms = 0;
@@ -510,7 +527,7 @@ void mf_default_params(mf_params* out)       // main.cu:19-32
     out->lambda = 0.015f; out->learning_rate = 0.01f; out->decay = 0.1f; out->sample_ratio = 0.01f; out->error_threshold = 0.001f;
     out->k = 128; out->epoch = 50; out->num_workers = 2048; out->thread_block_size = 128;
     out->user_group_num = 10; out->item_group_num = 10; out->version = 7; out->interval = 1; out->seed = 1;
-    out->hot_row_inflight = 8.0f;       // no reference counterpart: see mf_set_hot_row_thinning
+    out->hot_row_inflight = 2.0f; out->hot_row_inflight_early = 16.0f; out->hot_row_early_epochs = 2;   // no reference counterpart: see mf_set_hot_row_thinning
 }
 
 uint32_t mf_group_end_indices(const uint32_t* sorted_cnt, uint32_t n, uint32_t requested_groups, uint32_t* end_idx_out)

@@ -218,6 +218,10 @@ typedef struct {
     uint32_t epoch_splits;    /* kernel launches per epoch, 0 or 1 = one, see mf_set_epoch_splits */
     float hot_row_inflight;   /* > 0: rows expected to have more than one update in flight become hot rows, thinned
                                  to at most this many updates in flight (see mf_set_hot_row_thinning); 0 = off */
+    float hot_row_inflight_early; /* the cap during the first hot_row_early_epochs epochs, while all rows still grow
+                                 from their small initial values and popular rows need many updates (default 16 for
+                                 2 epochs, then hot_row_inflight = 2) */
+    uint32_t hot_row_early_epochs;
 } mf_params;
 
 /* What a run reports back; every pointer is optional host memory owned by the caller. */
