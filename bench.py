@@ -292,8 +292,8 @@ def measured_traffic(a, leg):
         return None
     if a.skip_coherent:
         return (14_053_967 * 2.0 + 24_189_917) * 1024 if leg["workers"] == 16384 else None
-    if leg["workers"] == 6144 and a.hot_row_inflight == 8.0 and a.warmup >= a.hot_row_early_epochs:
-        return (17_636_147 * 2.0 + 32_167_634) * 1024
+    if leg["workers"] == 6144 and a.hot_row_inflight == 2.0 and a.warmup >= a.hot_row_early_epochs:
+        return (16_032_418 * 2.0 + 27_715_099) * 1024
     return None
 
 
