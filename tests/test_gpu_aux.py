@@ -41,6 +41,20 @@ def test_float2half_exhaustive_halves_and_midpoints(orc):
         assert np.array_equal(got, x.astype(np.float16).view(np.uint16))
 
 
+def test_float2half_golden_vectors():
+    """The device conversion against tests/golden/half_vectors.npz (numpy float16, see make_half_vectors.py)."""
+    import os
+    import torch
+    h = mfutil.hip()
+    g = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "half_vectors.npz"))
+    x = g["f2h_in"]
+    dx = to_dev(x)
+    dout = torch.zeros(x.size, dtype=torch.int16, device="cuda")
+    h.mf_transform_float2half(dx.data_ptr(), dout.data_ptr(), x.size, mfutil.stream_ptr())
+    _sync()
+    assert np.array_equal(dout.cpu().numpy().view(np.uint16), g["f2h_out"])
+
+
 def test_half2float_exhaustive(orc):
     import torch
     h = mfutil.hip()

@@ -197,3 +197,17 @@ def test_f16c_and_software_builds_agree_on_updates(orc, orc_soft):
                 outs.append((ph, qh, gp, gq, npv.value, nqv.value, pm, qm))
             for x, y in zip(*outs):
                 assert np.array_equal(np.asarray(x), np.asarray(y))
+
+
+def test_golden_half_vectors(orc, orc_soft):
+    """tests/golden/half_vectors.npz (numpy float16 + exact rational arithmetic, see make_half_vectors.py): the
+    checker's conversion and its add / sub / mul / fma, in the F16C build and in the software build."""
+    import os
+    g = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "half_vectors.npz"))
+    for o in (orc, orc_soft):
+        assert np.array_equal(o.f2h(g["f2h_in"]), g["f2h_out"])
+        for name, key in (("orc_half_mul", "mul"), ("orc_half_add", "add"), ("orc_half_sub", "sub")):
+            got = np.vectorize(getattr(o.lib, name), otypes=[np.uint16])(g["a"], g["b"])
+            assert np.array_equal(got, g[key]), name
+        got = np.vectorize(o.lib.orc_half_fma, otypes=[np.uint16])(g["a"], g["b"], g["c"])
+        assert np.array_equal(got, g["fma"])
