@@ -34,22 +34,44 @@ def zipf_ranks(torch, count, size, alpha, gen, dev):
     return out
 
 
-def make_workload(torch, n_users, n_items, n, seed, dev, user_alpha, item_alpha, rank, noise, mean):
-    """COO ratings [n][3] int32 (float bits, user, item) on the device, ids in random (unsorted) order."""
+# The synthetic configurations of BASELINE.json that fit one GPU (config 1 is the CPU-runnable plumbing case of the
+# tests).  Config 5's ratings are integers 0..100; like the reference does for its 0..100 data set (io_utils.h:75)
+# they are mapped to r / 25 + 1 so that the N(0, 0.01^2) start and lr 0.01 stay in binary16 range.
+CONFIGS = {
+    2: dict(n_users=70_000, n_items=10_700, n_train=8_000_000, n_test=2_000_000, user_alpha=0.9, item_alpha=0.9, rank=16, noise=0.8,
+            mean=3.5, step=0.5, lo=0.5, hi=5.0, text="70000 users x 10700 items, Zipf(0.9), 0.5-5.0 in half steps from rank-16 truth + N(0,0.8)"),
+    3: dict(n_users=162_000, n_items=59_000, n_train=20_000_000, n_test=5_000_000, user_alpha=1.0, item_alpha=1.0, rank=16, noise=0.8,
+            mean=3.5, step=0.5, lo=0.5, hi=5.0, text="162000 users x 59000 items, Zipf(1.0), 0.5-5.0 in half steps from rank-16 truth + N(0,0.8)"),
+    4: dict(n_users=480_000, n_items=17_800, n_train=100_000_000, n_test=1_400_000, user_alpha=0.8, item_alpha=1.1, rank=32, noise=0.9,
+            mean=3.6, step=1.0, lo=1.0, hi=5.0, text="480000 users x 17800 items, item Zipf(1.1), user Zipf(0.8), ints 1-5 from rank-32 truth + N(0,0.9)"),
+    5: dict(n_users=1_000_000, n_items=625_000, n_train=250_000_000, n_test=4_000_000, user_alpha=1.2, item_alpha=1.2, rank=0, noise=15.0,
+            mean=0.0, step=1.0, lo=0.0, hi=100.0, text="1000000 users x 625000 items, Zipf(1.2), ints 0-100 from 0.5 N(20,15) + 0.5 N(80,15), mapped to r/25+1"),
+}
+
+
+def make_workload(torch, n_users, n_items, n, seed, dev, user_alpha, item_alpha, rank, noise, mean, step=1.0, lo=1.0, hi=5.0):
+    """COO ratings [n][3] int32 (float bits, user, item) on the device, ids in random (unsorted) order.  rank = 0: the
+    bimodal 0..100 ratings of config 5 (no low-rank truth), mapped to r / 25 + 1."""
     gen = torch.Generator(device=dev)
     gen.manual_seed(seed)
     uperm = torch.randperm(n_users, device=dev, generator=gen)
     iperm = torch.randperm(n_items, device=dev, generator=gen)
     u = uperm[zipf_ranks(torch, n_users, n, user_alpha, gen, dev)]
     i = iperm[zipf_ranks(torch, n_items, n, item_alpha, gen, dev)]
-    U = torch.randn(n_users, rank, device=dev, generator=gen) * 0.5
-    V = torch.randn(n_items, rank, device=dev, generator=gen) * 0.5
+    if rank:
+        U = torch.randn(n_users, rank, device=dev, generator=gen) * 0.5
+        V = torch.randn(n_items, rank, device=dev, generator=gen) * 0.5
     R = torch.empty((n, 3), dtype=torch.int32, device=dev)
-    step = 10_000_000
-    for s in range(0, n, step):
-        e = min(n, s + step)
-        val = (U[u[s:e]] * V[i[s:e]]).sum(1) + mean + torch.randn(e - s, device=dev, generator=gen) * noise
-        R[s:e, 0] = val.round_().clamp_(1, 5).to(torch.float32).view(torch.int32)
+    chunk = 10_000_000
+    for s in range(0, n, chunk):
+        e = min(n, s + chunk)
+        if rank:
+            val = (U[u[s:e]] * V[i[s:e]]).sum(1) + mean + torch.randn(e - s, device=dev, generator=gen) * noise
+            val = (val / step).round_().mul_(step).clamp_(lo, hi)
+        else:
+            mode = torch.where(torch.rand(e - s, device=dev, generator=gen) < 0.5, 20.0, 80.0)
+            val = (mode + torch.randn(e - s, device=dev, generator=gen) * noise).round_().clamp_(lo, hi) / 25.0 + 1.0
+        R[s:e, 0] = val.to(torch.float32).view(torch.int32)
     R[:, 1] = u.to(torch.int32)
     R[:, 2] = i.to(torch.int32)
     return R
@@ -288,11 +310,11 @@ def measured_traffic(a, leg):
     """HBM bytes per launch of a plain epoch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch, scaled by
     2.0 / 1.0, the factors a 1 GiB device copy gives; summaries under profiles/).  Counters cannot be read from inside
     this process, so the figures are the profiled ones and only reported for the exact workload they were taken on."""
-    if a.ratings != 100_000_000 or a.seed != 2021:
+    if a.config != 4 or a.k != 128 or a.ratings != 100_000_000 or a.seed != 2021:
         return None
     if a.skip_coherent:
         return (14_053_967 * 2.0 + 24_189_917) * 1024 if leg["workers"] == 16384 else None
-    if leg["workers"] == 6144 and a.hot_row_inflight == 2.0 and a.warmup >= a.hot_row_early_epochs:
+    if leg["workers"] in (6104, 6144) and a.hot_row_inflight == 2.0 and a.warmup >= a.hot_row_early_epochs:
         return (16_032_418 * 2.0 + 27_715_099) * 1024
     return None
 
@@ -302,8 +324,10 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=2)
-    ap.add_argument("--ratings", type=int, default=100_000_000)
-    ap.add_argument("--workers", type=int, default=6144, help="-wg of the measured run (24 wavefronts on each of the 256 CUs)")
+    ap.add_argument("--config", type=int, default=4, choices=sorted(CONFIGS), help="BASELINE.json configuration (4 = the one the metric is quoted on)")
+    ap.add_argument("--ratings", type=int, default=0, help="training ratings (default: the configuration's)")
+    ap.add_argument("--k", type=int, default=128, choices=(64, 128))
+    ap.add_argument("--workers", type=int, default=0, help="-wg of the measured run (default: mf_auto_workers(ratings); 6104 at config 4)")
     ap.add_argument("--cached-workers", type=int, default=16384)
     ap.add_argument("--cpu-updates", type=int, default=32_000_000, help="size of the CPU baseline sample (about 10 s on 16 threads)")
     ap.add_argument("--skip-cpu", action="store_true")
@@ -327,11 +351,15 @@ def main():
     import torch
     h = importlib.import_module("icdm-2021_mascot_amd").load()
     dev = torch.device("cuda:0")
-    n_users, n_items, k = 480_000, 17_800, 128
+    wc = CONFIGS[a.config]
+    n_users, n_items, k = wc["n_users"], wc["n_items"], a.k
+    a.ratings = a.ratings or wc["n_train"]
+    a.workers = a.workers or h.mf_auto_workers(a.ratings)
     cfg = dict(epochs=50, lr=0.01, decay=0.1, lam=0.015, sample_ratio=0.05, interval=2, ug=100, ig=100)
     t0 = time.perf_counter()
-    n_test = 1_400_000
-    R = make_workload(torch, n_users, n_items, a.ratings + n_test, a.seed, dev, user_alpha=0.8, item_alpha=1.1, rank=32, noise=0.9, mean=3.6)
+    n_test = wc["n_test"]
+    R = make_workload(torch, n_users, n_items, a.ratings + n_test, a.seed, dev, **{key: wc[key] for key in
+                      ("user_alpha", "item_alpha", "rank", "noise", "mean", "step", "lo", "hi")})
     prob = MascotProblem(torch, h, R[:a.ratings].contiguous(), n_users, n_items, k, cfg["ug"], cfg["ig"], a.seed, test=R[a.ratings:].contiguous())
     del R
     torch.cuda.synchronize()
@@ -368,8 +396,8 @@ def main():
         "value": main_leg["ratings_per_s"], "unit": "ratings/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
         "ms_per_step": main_leg["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16", "data": "synthetic",
-        "config": {"workload": "config 4: 480000 users x 17800 items, %d train ratings, item Zipf(1.1), user Zipf(0.8), "
-                               "ints 1-5 from rank-32 truth + N(0,0.9); MASCOT -v 1 -k 128 -ug 100 -ig 100 -s 0.05 -it 2 -e 20" % a.ratings,
+        "config": {"workload": "config %d: %s, %d train ratings; MASCOT -v 1 -k %d -ug 100 -ig 100 -s 0.05 -it 2 -e 20"
+                               % (a.config, wc["text"], a.ratings, k),
                    "workers": main_leg["workers"], "row_access": "cached" if a.skip_coherent else "device-coherent", "update_vector_size": 128,
                    "epochs_timed": "%d..%d of 50" % (a.warmup, a.warmup + a.steps - 1), "seed": a.seed,
                    "hot_row_inflight": 0.0 if a.skip_coherent else a.hot_row_inflight,
@@ -379,7 +407,7 @@ def main():
         "roofline": {"bound": "hbm", "achieved": main_leg["gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
                      "frac": main_leg["gbs"] / PEAK_HBM_GBS,
                      "traffic": measured_traffic(a, main_leg),
-                     "kernel": "hogwild_kernel<MascotRuleT<128,%s,false>>" % ("false" if a.skip_coherent else "true"),
+                     "kernel": "hogwild_kernel<MascotRuleT<%d,%s,false>>" % (k, "false" if a.skip_coherent else "true"),
                      "bytes_per_update": round(main_leg["bytes_per_update"], 1),
                      "updates_per_launch": main_leg["updates_per_step"]},
         "ms_steps": main_leg["ms_steps"],
@@ -397,7 +425,7 @@ def main():
                                       "rows; faster, converges worse, see DESIGN.md)",
                               "value": c["ratings_per_s"], "unit": "ratings/s", "ms_per_step": c["ms_per_step"], "workers": c["workers"],
                               "roofline": {"bound": "hbm", "achieved": c["gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": c["gbs"] / PEAK_HBM_GBS,
-                                           "kernel": "hogwild_kernel<MascotRuleT<128,false,false>>"},
+                                           "kernel": "hogwild_kernel<MascotRuleT<%d,false,false>>" % k},
                               "ms_steps": c["ms_steps"], "test_rmse_after_timed_epochs": c["rmse"]}
         h.mf_set_row_coherence(1)
     if not a.skip_fp32 and not a.skip_coherent:
