@@ -107,7 +107,7 @@ int main(int argc, const char* argv[])
         return rc > 0 ? rc : 1;
     }
     // timing summary in the reference's units (micro seconds unless stated), mf_methods.cu:401-418
-    if (prm.version == 1) {
+    if (prm.version == 1 || prm.version == 6) {
         std::cout << "\n<Preprocessing time (micro sec)>" << std::endl;
         std::cout << "Total preprocessing time         : " << rep.preprocess_ms * 1000 << std::endl;
         std::cout << "\n<User & item parameter copy exec time (micro sec)>" << std::endl;
@@ -124,9 +124,10 @@ int main(int argc, const char* argv[])
     std::cout << "Ratings per second (update kernel): " << (double)d.R.size() * prm.epoch / (rep.sgd_ms / 1000.0) << std::endl;
 
     if (!outfile.empty()) {
-        if (prm.version == 1) save_trained_model_reconst(d.max_user, d.max_item, p.data(), q.data(), prm.k, outfile);
+        // -v 6 trains in the same re-indexed row order as -v 1, so its model is written in that layout as well
+        if (prm.version == 1 || prm.version == 6) save_trained_model_reconst(d.max_user, d.max_item, p.data(), q.data(), prm.k, outfile);
         else save_trained_model(d, p.data(), q.data(), prm.k, outfile);
     }
-    if (prm.version == 1 && reconst_save == 1) save_reconst_testset(test_reconst, testfile);
+    if ((prm.version == 1 || prm.version == 6) && reconst_save == 1) save_reconst_testset(test_reconst, testfile);
     return 0;
 }

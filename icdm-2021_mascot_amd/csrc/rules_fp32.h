@@ -178,4 +178,94 @@ template <int K, bool COH> struct MptRule : DenseBase<K, COH> {
     __device__ __forceinline__ void finish(const Params&, uint32_t) const {}
 };
 
+// mem_quant_sgd_k128/k64_hogwild_kernel, sgd/sgd_kernel.h:81-164: dense binary16 P/Q, binary32 arithmetic.  Lane L holds
+// elements L and L+64 of a row (two coalesced 128-byte accesses), widened.  The reference's lane l sums its products
+// left to right, p1*q1 + p2*q2 + p3*q3 + p4*q4 over elements l, l+32, l+64, l+96: with a = m0[l], b = m0[l+32],
+// c = m1[l], d = m1[l+32] (l = L mod 32) that is ((a + b) + c) + d, formed identically in both half-waves.
+template <int K, bool COH> struct MemQuantRule {
+    static constexpr int E = K / 64;
+    using Row = DenseRow<K>;
+    using Info = DenseInfo;
+    using Prep = NoPrep;
+    static constexpr int kClasses = 1;
+    static constexpr int kAhead = 3, kRing = 8;
+    static constexpr bool kSplittable = true;
+    struct Params { uint16_t* p; uint16_t* q; float lrate; float lambda; bool accumulate; };
+    uint16_t* P; uint16_t* Q; float lrate, lambda; int lane;
+
+    __device__ __forceinline__ void init(const Params& a, uint8_t*, int lane_, uint32_t) { P = a.p; Q = a.q; lrate = a.lrate; lambda = a.lambda; lane = lane_; }
+    __device__ __forceinline__ Prep prepare(const Rating&, bool) const { return Prep(); }
+    __device__ __forceinline__ int classify(const Prep&, bool) const { return 0; }
+    __device__ __forceinline__ Info info(const Rating& my, const Prep&, int j) const
+    {
+        Info i;
+        i.r = bcast(my.r, j); i.u = bcast(my.u, j); i.v = bcast(my.v, j); i.thin = bcast(my.thin, j);
+        return i;
+    }
+    template <int CLS> __device__ __forceinline__ void load(Row& row, const Info& i) const
+    {
+        const uint16_t* pp = P + (size_t)i.u * K + lane;
+        const uint16_t* qq = Q + (size_t)i.v * K + lane;
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+            row.p[e] = (float)from_bits<half_t>((uint32_t)row_load(pp + 64 * e));
+            row.q[e] = (float)from_bits<half_t>((uint32_t)row_load(qq + 64 * e));
+        }
+    }
+    __device__ __forceinline__ void forward(Row& nxt, const Info& in, const Row& cur, const Info& ic) const
+    {
+        if (in.u == ic.u) {
+#pragma unroll
+            for (int e = 0; e < E; ++e) nxt.p[e] = cur.p[e];
+        }
+        if (in.v == ic.v) {
+#pragma unroll
+            for (int e = 0; e < E; ++e) nxt.q[e] = cur.q[e];
+        }
+    }
+    // store the rounded row, or add the rounded change to a hot row: even lanes add the pair (own, right neighbour)
+    __device__ __forceinline__ void write_side(uint16_t* base, const float* now, const float* change, bool hot) const
+    {
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+            if (hot) {
+                const uint32_t mine = bits((half_t)change[e]);
+                const uint32_t other = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)mine, 0xB1 /* quad_perm 1,0,3,2 */, 0xf, 0xf, false);
+                if (!(lane & 1)) row_add(reinterpret_cast<half2_t*>(base + 64 * e), from_bits<half2_t>(mine | (other << 16)));
+            } else {
+                row_store<COH>(base + 64 * e, (uint16_t)bits((half_t)now[e]));
+            }
+        }
+    }
+    template <int CLS> __device__ __forceinline__ void update(Row& row, const Info& i, uint32_t) const
+    {
+        float dot;
+        if constexpr (E == 1) {
+            dot = reduce_wave(row.p[0] * row.q[0], OpAdd());                // k = 64: p1*q1 + p2*q2, then the tree
+        } else {
+            const float m0 = row.p[0] * row.q[0], m1 = row.p[1] * row.q[1];
+            const float o0 = lane_xor32(m0), o1 = lane_xor32(m1);
+            const bool upper = lane >= 32;
+            float s = m0 + o0;                                              // a + b
+            s = s + (upper ? o1 : m1);                                      // + c
+            s = s + (upper ? m1 : o1);                                      // + d
+            dot = reduce_half_wave(s, OpAdd());
+        }
+        const float ruv = i.r - dot;
+        float dp[E], dq[E];
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+            const float pe = row.p[e], qe = row.q[e];
+            dp[e] = lrate * (ruv * qe - lambda * pe);
+            dq[e] = lrate * (ruv * pe - lambda * qe);
+            // the register copy is what the row holds afterwards: the sum rounded to binary16
+            row.p[e] = (i.thin & 1u) ? pe : (float)(half_t)(pe + dp[e]);
+            row.q[e] = (i.thin & 2u) ? qe : (float)(half_t)(qe + dq[e]);
+        }
+        if (!(i.thin & 1u)) write_side(P + (size_t)i.u * K + lane, row.p, dp, i.thin & 4u);
+        if (!(i.thin & 2u)) write_side(Q + (size_t)i.v * K + lane, row.q, dq, i.thin & 8u);
+    }
+    __device__ __forceinline__ void finish(const Params&, uint32_t) const {}
+};
+
 }  // namespace mf

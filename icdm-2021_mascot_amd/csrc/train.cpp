@@ -169,7 +169,40 @@ struct HotRows {
     }
 };
 
-// ---- variants over dense fp32 P/Q (versions 2..5) ----------------------------------------------
+// Whole-model precision switching (-v 8, training_switching_only, mf_methods.cu:1396-1562): the MASCOT kernel with
+// one group per side that holds every row in its original order (the arithmetic of switching_only_sgd_k128/k64 is
+// the binary16 / binary32 case of the MASCOT kernel, sgd/sgd_kernel.h:166-344), the sampled statistics of both sides
+// added together, and both sides promoted at once.
+struct WholeModel {
+    DevBuf hp, hq, ptr_p, ptr_q, end_u, end_i, prec, gsp, gsq, nsp, nsq;
+    uint32_t norm_blocks = 0;
+    bool is_float = false;
+    float initial_error = 1.f;
+    int init(Common& c, const float* d_p, const float* d_q, uint32_t num_workers)
+    {
+        const size_t pn = (size_t)c.n_users * c.k, qn = (size_t)c.n_items * c.k;
+        MF_TRY(hp.alloc(pn * 2, "hipMalloc(binary16 P)"));
+        MF_TRY(hq.alloc(qn * 2, "hipMalloc(binary16 Q)"));
+        MF_TRY(mf_transform_float2half(d_p, hp.as<uint16_t>(), pn, nullptr));
+        MF_TRY(mf_transform_float2half(d_q, hq.as<uint16_t>(), qn, nullptr));
+        norm_blocks = mf_mascot_norm_blocks(num_workers);
+        MF_TRY(ptr_p.alloc(8, "hipMalloc")); MF_TRY(ptr_q.alloc(8, "hipMalloc")); MF_TRY(end_u.alloc(4, "hipMalloc")); MF_TRY(end_i.alloc(4, "hipMalloc"));
+        MF_TRY(prec.alloc(1, "hipMalloc")); MF_TRY(gsp.alloc(c.k * 4, "hipMalloc")); MF_TRY(gsq.alloc(c.k * 4, "hipMalloc"));
+        MF_TRY(nsp.alloc((size_t)norm_blocks * 4, "hipMalloc")); MF_TRY(nsq.alloc((size_t)norm_blocks * 4, "hipMalloc"));
+        const uint32_t eu = c.n_users - 1, ei = c.n_items - 1;
+        HIP_TRY(hipMemcpy(end_u.p, &eu, 4, hipMemcpyHostToDevice), "H2D"); HIP_TRY(hipMemcpy(end_i.p, &ei, 4, hipMemcpyHostToDevice), "H2D");
+        return point_at(hp.p, hq.p, 0);
+    }
+    int point_at(void* p, void* q, uint8_t precision)
+    {
+        HIP_TRY(hipMemcpy(ptr_p.p, &p, 8, hipMemcpyHostToDevice), "H2D"); HIP_TRY(hipMemcpy(ptr_q.p, &q, 8, hipMemcpyHostToDevice), "H2D");
+        HIP_TRY(hipMemcpy(prec.p, &precision, 1, hipMemcpyHostToDevice), "H2D");
+        is_float = precision != 0;
+        return 0;
+    }
+};
+
+// ---- variants over dense P/Q (versions 2..5, 7, 8) ----------------------------------------------
 int train_dense(Common& c, float* p, float* q)
 {
     const mf_params& prm = *c.prm;
@@ -208,8 +241,21 @@ int train_dense(Common& c, float* p, float* q)
         muppet_first_sample = c.update_count * c.update_vector_size - (uint32_t)sample_ratings_num;
     }
 
+    // -v 7: dense binary16 storage next to the fp32 buffers, which then only serve the RMSE and the result
+    DevBuf d_hp, d_hq;
+    if (version == 7) {
+        MF_TRY(d_hp.alloc(pn * 2, "hipMalloc(binary16 P)"));
+        MF_TRY(d_hq.alloc(qn * 2, "hipMalloc(binary16 Q)"));
+        MF_TRY(mf_transform_float2half(d_p.as<float>(), d_hp.as<uint16_t>(), pn, nullptr));
+        MF_TRY(mf_transform_float2half(d_q.as<float>(), d_hq.as<uint16_t>(), qn, nullptr));
+    }
+    WholeModel whole;
+    const uint32_t total = c.update_count * c.update_vector_size;
+    const uint32_t whole_sample_num = (uint32_t)(int)((float)total * prm.sample_ratio);       // mf_methods.cu:1425
+    if (version == 8) MF_TRY(whole.init(c, d_p.as<float>(), d_q.as<float>(), prm.num_workers));
+
     HotRows hot;
-    if (prm.hot_row_inflight > 0 && (version == 5 || version == 4)) {
+    if (prm.hot_row_inflight > 0 && (version == 5 || version == 4 || version == 7 || version == 8)) {
         DevBuf d_ucnt, d_icnt;
         MF_TRY(d_ucnt.alloc((size_t)c.n_users * 4, "hipMalloc(user counts)"));
         MF_TRY(d_icnt.alloc((size_t)c.n_items * 4, "hipMalloc(item counts)"));
@@ -225,6 +271,7 @@ int train_dense(Common& c, float* p, float* q)
     const mf_node* R = c.d_R.as<mf_node>();
     for (uint32_t e = 0; e < prm.epoch; ++e) {
         MF_TRY(hot.select(e));
+        bool whole_check = false;
         const double err0 = now_ms();
         if (version == 3) HIP_TRY(hipMemsetAsync(d_sum_updated.p, 0, c.k * 4, nullptr), "memset sum_updated_val");
         double err_ms = now_ms() - err0;
@@ -243,9 +290,51 @@ int train_dense(Common& c, float* p, float* q)
         }
         case 2: MF_TRY(mf_afp_sgd_hogwild(R, c.n, d_p.as<float>(), d_q.as<float>(), (int)c.k, prm.num_workers, c.update_count, c.update_vector_size,
                                           c.lr[e], prm.lambda, (int)e, prm.seed, e, nullptr, nullptr)); break;
+        case 7: MF_TRY(mf_mem_quant_sgd_hogwild(R, c.n, d_hp.as<uint16_t>(), d_hq.as<uint16_t>(), (int)c.k, prm.num_workers, c.update_count,
+                                                c.update_vector_size, c.lr[e], prm.lambda, prm.seed, e, nullptr, nullptr)); break;
+        case 8: {
+            // mf_methods.cu:1460-1466: sampled only while the model is binary16
+            whole_check = !whole.is_float && prm.interval && e >= 5 && (e % prm.interval == 5 % prm.interval) && prm.epoch - 1 != e;
+            if (whole_check) {
+                t.stop();
+                const double e0 = now_ms();
+                HIP_TRY(hipMemsetAsync(whole.gsp.p, 0, c.k * 4, nullptr), "memset"); HIP_TRY(hipMemsetAsync(whole.gsq.p, 0, c.k * 4, nullptr), "memset");
+                err_ms += now_ms() - e0;
+                t.start();
+            }
+            MF_TRY(mf_mascot_sgd_hogwild(R, c.n, whole.ptr_p.as<void*>(), whole.ptr_q.as<void*>(), (int)c.k, prm.num_workers, c.update_count,
+                                         c.update_vector_size, c.lr[e], prm.lambda, whole.end_u.as<uint32_t>(), whole.end_i.as<uint32_t>(),
+                                         whole.prec.as<uint8_t>(), whole.prec.as<uint8_t>(), whole.gsp.as<float>(), whole.gsq.as<float>(),
+                                         whole.nsp.as<float>(), whole.nsq.as<float>(), whole_check ? total - whole_sample_num : total, 1, 1,
+                                         prm.seed, e, nullptr, nullptr));
+            break;
+        }
         default: return invalid("mf_train: version %u is not a dense variant", version);
         }
         const float sgd_ms = t.stop();
+        if (version == 7 || (version == 8 && !whole.is_float)) {      // the fp32 copy the RMSE kernel and the caller read
+            MF_TRY(mf_transform_half2float((version == 7 ? d_hp : whole.hp).as<uint16_t>(), d_p.as<float>(), pn, nullptr));
+            MF_TRY(mf_transform_half2float((version == 7 ? d_hq : whole.hq).as<uint16_t>(), d_q.as<float>(), qn, nullptr));
+        }
+        if (version == 8 && whole_check) {      // mf_methods.cu:1506-1536
+            const double e0 = now_ms();
+            std::vector<float> gs(2 * c.k), ns(2 * (size_t)whole.norm_blocks);
+            HIP_TRY(hipMemcpy(gs.data(), whole.gsp.p, c.k * 4, hipMemcpyDeviceToHost), "D2H"); HIP_TRY(hipMemcpy(gs.data() + c.k, whole.gsq.p, c.k * 4, hipMemcpyDeviceToHost), "D2H");
+            HIP_TRY(hipMemcpy(ns.data(), whole.nsp.p, (size_t)whole.norm_blocks * 4, hipMemcpyDeviceToHost), "D2H");
+            HIP_TRY(hipMemcpy(ns.data() + whole.norm_blocks, whole.nsq.p, (size_t)whole.norm_blocks * 4, hipMemcpyDeviceToHost), "D2H");
+            float norm_acc = 0, sum_norms_acc = 0;
+            for (float v : ns) norm_acc += v;
+            for (uint32_t i = 0; i < c.k; ++i) sum_norms_acc += std::pow(gs[i] + gs[c.k + i], 2.0f);
+            float quantization_error = sum_norms_acc / norm_acc;
+            quantization_error = quantization_error / whole.initial_error;
+            if (prm.verbose) { std::printf("Quantization error : %g\n", (double)quantization_error); std::fflush(stdout); }
+            if (e == 5) whole.initial_error = quantization_error;
+            if (e > 5 && quantization_error > prm.error_threshold) {      // both sides to binary32 (d_p, d_q were just widened)
+                MF_TRY(whole.point_at(d_p.p, d_q.p, 1));
+                if (c.rep) c.rep->switching_ms += now_ms() - e0;
+            }
+            err_ms += now_ms() - e0;
+        }
         double rmse = 0;
         MF_TRY(dense_rmse(c, d_p.as<float>(), d_q.as<float>(), &rmse));
         report_epoch(c, e, rmse, sgd_ms);
@@ -613,7 +702,7 @@ int mf_train(const mf_params* params, const mf_node* R, uint32_t n, uint32_t n_u
     if (with_workers.num_workers == 0) with_workers.num_workers = mf_auto_workers(n);
     params = &with_workers;
     const uint32_t version = params->version == 0 ? 5 : params->version;
-    if (version < 1 || version > 5) return invalid("mf_train: version %u is not built (1 MASCOT, 2 AFP, 3 MuPPET, 4 MPT, 5 fp32 SGD)", params->version);
+    if (version < 1 || version > 8) return invalid("mf_train: version %u does not exist (1 MASCOT, 2 AFP, 3 MuPPET, 4 MPT, 5 fp32 SGD, 6 MASCOT, 7 binary16 storage, 8 whole-model switching)", params->version);
     Common c;
     c.prm = params; c.n = n; c.n_users = n_users; c.n_items = n_items; c.test_n = test_n; c.k = params->k; c.rep = report;
     if (report) { report->preprocess_ms = report->switching_ms = report->error_ms = report->sgd_ms = report->total_ms = 0; report->muppet_final_bits = 0; }
@@ -625,7 +714,9 @@ int mf_train(const mf_params* params, const mf_node* R, uint32_t n, uint32_t n_u
     struct Restore { int c; uint32_t s; ~Restore() { (void)mf_set_row_coherence(c); (void)mf_set_epoch_splits(s); } } restore{saved_coherence, saved_splits};
     fill_schedule(c);
     MF_TRY(upload_and_shuffle(c, R, test));
-    const int rc = version == 1 ? train_mascot(c, p, q) : train_dense(c, p, q);
+    // -v 6 (mascot_training_mf_naive, mf_methods.cu:926-1301) is MASCOT with the group search done from global memory
+    // and shifted end-index tables: the same schedule, arithmetic and epoch logic, so it runs the MASCOT path
+    const int rc = (version == 1 || version == 6) ? train_mascot(c, p, q) : train_dense(c, p, q);
     if (rc == 0 && report) report->total_ms = now_ms() - t0;
     return rc;
 }

@@ -90,6 +90,12 @@ int mf_single_sgd_hogwild(const mf_node* R, uint32_t nnz, float* p, float* q, in
                           float lrate, float lambda,
                           uint64_t seed, uint32_t epoch, const uint32_t* window_start, void* stream);
 
+/* mem_quant_sgd_k128/k64_hogwild_kernel launch (-v 7, the reference's default version), mf_methods.cu:1345-1372:
+ * dense binary16 P [users][k], Q [items][k] (bit patterns), binary32 arithmetic, new values rounded to binary16. */
+int mf_mem_quant_sgd_hogwild(const mf_node* R, uint32_t nnz, uint16_t* p, uint16_t* q, int k,
+                             uint32_t num_workers, uint32_t update_count, uint32_t update_vector_size,
+                             float lrate, float lambda,
+                             uint64_t seed, uint32_t epoch, const uint32_t* window_start, void* stream);
 /* mpt_sgd_k128/k64_hogwild_kernel, mpt/mpt_sgd_kernel.h:1-93, mpt/mpt_sgd_kernel_k64.h;
  * launch site mf_methods.cu:772-799.  scaled_lambda_half = binary16 bits of lambda*scaling_factor
  * (mf_methods.cu:764-765). */
@@ -210,7 +216,9 @@ typedef struct {
     uint32_t num_workers;     /* -wg; 0 = mf_auto_workers(n) */
     uint32_t epoch;           /* -l  */
     uint32_t thread_block_size; /* -bl: accepted for compatibility; workgroups are always 4 wavefronts here */
-    uint32_t version;         /* -v: 1 MASCOT, 2 AFP, 3 MuPPET, 4 MPT, 5 fp32 SGD (0 = alias of 5) */
+    uint32_t version;         /* -v: 1 MASCOT, 2 AFP, 3 MuPPET, 4 MPT, 5 fp32 SGD (0 = alias of 5), 6 MASCOT (the reference's
+                                 naive kernel: same arithmetic, runs the MASCOT path), 7 binary16 storage with
+                                 binary32 arithmetic, 8 whole-model precision switching */
     uint32_t is_yahoo;        /* MuPPET starts at 12 bit (mf_methods.cu:600) */
     uint64_t seed;            /* replaces time(0) / clock() seeding */
     uint32_t verbose;         /* 1: print the reference's stdout lines (mf_methods.cu:396 etc.) */

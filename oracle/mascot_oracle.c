@@ -411,6 +411,35 @@ void orc_sgd_update(int k, float* p, float* q, float r, float lr, float lambda)
     }
 }
 
+/* mem_quant_sgd_k128/k64_hogwild_kernel body, sgd/sgd_kernel.h:126-163 (k = 64: sgd_kernel_k64.h): binary16 storage,
+ * binary32 arithmetic.  Per lane the products are summed left to right (p1*q1 + p2*q2 + p3*q3 + p4*q4), then the
+ * 16,8,4,2,1 tree; the new values are rounded to binary16 once.  No contraction (nvcc's choice there is unpinned). */
+void orc_mem_quant_update(int k, uint16_t* p, uint16_t* q, float r, float lr, float lambda)
+{
+    float pf[128], qf[128], x[LANES];
+    for (int e = 0; e < k; e++) { pf[e] = orc_h2f(p[e]); qf[e] = orc_h2f(q[e]); }
+    for (int l = 0; l < LANES; l++) {
+        float m0 = pf[l] * qf[l];
+        float m1 = pf[l + 32] * qf[l + 32];
+        float a = m0 + m1;
+        if (k == 128) {
+            float m2 = pf[l + 64] * qf[l + 64];
+            a = a + m2;
+            float m3 = pf[l + 96] * qf[l + 96];
+            a = a + m3;
+        }
+        x[l] = a;
+    }
+    float ruv = r - tree_f(x);
+    for (int e = 0; e < k; e++) {
+        float pe = pf[e], qe = qf[e];
+        float a = ruv * qe; float b = lambda * pe; float c = a - b; float d = lr * c; float n = pe + d;
+        p[e] = orc_f2h(n);
+        a = ruv * pe; b = lambda * qe; c = a - b; d = lr * c; n = qe + d;
+        q[e] = orc_f2h(n);
+    }
+}
+
 /* mpt_sgd_k128/k64_hogwild_kernel body, mpt/mpt_sgd_kernel.h:15-16,38-91.
  * scaled_lambda_h = __float2half_rn(lambda * 1000) is formed by the host (mf_methods.cu:764-765). */
 void orc_mpt_update(int k, float* p, float* q, float r, float lr, uint16_t scaled_lambda_h, float scaling_factor)
@@ -821,6 +850,14 @@ void orc_sgd_epoch(int k, const orc_node* R, uint32_t nnz, float* P, float* Q,
 {
     if (threads <= 1) { FOR_EACH_UPDATE_SEQ(orc_sgd_update(k, P + (size_t)nd->u * k, Q + (size_t)nd->i * k, nd->r, lr, lambda);) }
     else { FOR_EACH_UPDATE_PAR(orc_sgd_update(k, P + (size_t)nd->u * k, Q + (size_t)nd->i * k, nd->r, lr, lambda);) }
+}
+
+void orc_mem_quant_epoch(int k, const orc_node* R, uint32_t nnz, uint16_t* P, uint16_t* Q,
+                         uint32_t num_workers, uint32_t update_count, uint32_t update_vector_size,
+                         float lr, float lambda, uint64_t seed, uint32_t epoch, const uint32_t* window_start, int threads)
+{
+    if (threads <= 1) { FOR_EACH_UPDATE_SEQ(orc_mem_quant_update(k, P + (size_t)nd->u * k, Q + (size_t)nd->i * k, nd->r, lr, lambda);) }
+    else { FOR_EACH_UPDATE_PAR(orc_mem_quant_update(k, P + (size_t)nd->u * k, Q + (size_t)nd->i * k, nd->r, lr, lambda);) }
 }
 
 void orc_mpt_epoch(int k, const orc_node* R, uint32_t nnz, float* P, float* Q,

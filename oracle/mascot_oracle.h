@@ -61,6 +61,8 @@ void orc_init_normal(uint64_t seed, uint64_t stream, float* out, uint64_t n);
 
 /* ---- single updates (in place on one P row and one Q row) -------------- */
 void orc_sgd_update(int k, float* p, float* q, float r, float lr, float lambda);
+/* mem_quant_sgd (-v 7), sgd/sgd_kernel.h:81-164: binary16 rows, binary32 arithmetic */
+void orc_mem_quant_update(int k, uint16_t* p, uint16_t* q, float r, float lr, float lambda);
 void orc_mpt_update(int k, float* p, float* q, float r, float lr, uint16_t scaled_lambda_h, float scaling_factor);
 /* prec: 0 = binary16 row (uint16_t*), 1 = binary32 row (float*).  grad_p/grad_q (k floats)
  * and norm_p/norm_q receive the sampled statistics of the binary16 sides; untouched for
@@ -82,6 +84,9 @@ void orc_afp_update(int k, orc_afp_state* s, float* p, float* q, float r, float 
 
 /* ---- whole-launch restatements (sequential: ite-major, then worker) ---- */
 /* window_start may be NULL (then orc_window_start(seed, epoch, wid, ite, nnz) is used). */
+void orc_mem_quant_epoch(int k, const orc_node* R, uint32_t nnz, uint16_t* P, uint16_t* Q,
+                         uint32_t num_workers, uint32_t update_count, uint32_t update_vector_size,
+                         float lr, float lambda, uint64_t seed, uint32_t epoch, const uint32_t* window_start, int threads);
 void orc_sgd_epoch(int k, const orc_node* R, uint32_t nnz, float* P, float* Q,
                    uint32_t num_workers, uint32_t update_count, uint32_t update_vector_size,
                    float lr, float lambda, uint64_t seed, uint32_t epoch, const uint32_t* window_start, int threads);

@@ -66,6 +66,8 @@ class Oracle:
             "orc_shuffle_keys": (None, [u64, u64, vp]), "orc_shuffle": (None, [u64, vp, vp, u64]),
             "orc_init_normal": (None, [u64, u64, vp, u64]),
             "orc_sgd_update": (None, [i32, vp, vp, f32, f32, f32]),
+            "orc_mem_quant_update": (None, [i32, vp, vp, f32, f32, f32]),
+            "orc_mem_quant_epoch": (None, [i32, vp, u32, vp, vp, u32, u32, u32, f32, f32, u64, u32, vp, i32]),
             "orc_mpt_update": (None, [i32, vp, vp, f32, f32, u16, f32]),
             "orc_mascot_update": (None, [i32, vp, i32, vp, i32, f32, f32, f32, vp, vp, C.POINTER(f32), C.POINTER(f32)]),
             "orc_muppet_update": (None, [i32, vp, vp, f32, f32, f32, i32, i32, vp, C.POINTER(f32)]),

@@ -176,6 +176,62 @@ def oracle_train_dense(orc, version, R, test, P, Q, k, W, epochs, lr, lam, decay
     return np.array(rmse), dict(final_bits=bits_ladder[min(pidx_c.value, 4)])
 
 
+def oracle_train_mem_quant(orc, R, test, P, Q, k, W, epochs, lr, lam, decay, seed, threads=8):
+    """training_mem_quant_mf (-v 7, mf_methods.cu:1303-1394) on the CPU: dense binary16 rows, binary32 arithmetic.
+    P, Q: binary16-representable fp32 in, the widened result out; returns per-epoch test RMSE."""
+    Rs = orc.shuffle(seed, R)
+    uc = orc.lib.orc_update_count(Rs.size, W, 128)
+    Ph, Qh = orc.f2h(P), orc.f2h(Q)
+    rmse = []
+    for e in range(epochs):
+        orc.lib.orc_mem_quant_epoch(k, Rs.ctypes.data, Rs.size, Ph.ctypes.data, Qh.ctypes.data, W, uc, 128,
+                                    orc.lib.orc_lr_schedule(lr, decay, e), lam, seed, e, None, threads)
+        P[...] = orc.h2f(Ph).reshape(P.shape)
+        Q[...] = orc.h2f(Qh).reshape(Q.shape)
+        rmse.append(orc.rmse(k, test, P, Q))
+    return np.array(rmse)
+
+
+def oracle_train_switching_only(orc, R, test, P, Q, k, W, epochs, lr, lam, decay, seed, sample_ratio, interval, threshold, threads=8):
+    """training_switching_only (-v 8, mf_methods.cu:1396-1562) on the CPU: the whole model in binary16 until the sampled
+    error of both sides together exceeds the threshold, then in binary32.  The per-update arithmetic of
+    switching_only_sgd_k128/k64 (sgd/sgd_kernel.h:166-344) is the binary16 / binary32 case of the MASCOT update, so the
+    checker's MASCOT epoch runs it with one group per side.  Returns (per-epoch RMSE, switching epoch or -1, errors)."""
+    n_users, n_items = P.shape[0], Q.shape[0]
+    Rs = orc.shuffle(seed, R)
+    uc = orc.lib.orc_update_count(Rs.size, W, 128)
+    uend, iend = np.array([n_users - 1], np.uint32), np.array([n_items - 1], np.uint32)
+    gu = host_grouped(orc, k, P, uend, np.zeros(1, np.uint8))
+    gi = host_grouped(orc, k, Q, iend, np.zeros(1, np.uint8))
+    total = uc * 128
+    sample_num = int(np.float32(total) * np.float32(sample_ratio))
+    initial, switched, is_float, rmse, errors = np.float32(1.0), -1, False, [], []
+    for e in range(epochs):
+        check = (not is_float) and interval and e >= 5 and (e % interval == 5 % interval) and epochs - 1 != e
+        gsp, gsq, nsp, nsq = np.zeros(k, np.float32), np.zeros(k, np.float32), np.zeros(1, np.float32), np.zeros(1, np.float32)
+        orc.lib.orc_mascot_epoch(k, Rs.ctypes.data, Rs.size, gu.ptrs, gi.ptrs, gu.end_idx.ctypes.data, gi.end_idx.ctypes.data,
+                                 gu.prec.ctypes.data, gi.prec.ctypes.data, 1, 1, W, uc, 128, orc.lib.orc_lr_schedule(lr, decay, e), lam,
+                                 total - sample_num if check else total, gsp.ctypes.data, gsq.ctypes.data, nsp.ctypes.data, nsq.ctypes.data,
+                                 seed, e, None, threads)
+        if check:
+            err = np.float32(np.sum((gsp + gsq).astype(np.float32) ** 2, dtype=np.float32)) / np.float32(nsp[0] + nsq[0]) / initial
+            errors.append((e, float(err)))
+            if e == 5:
+                initial = err
+            if e > 5 and err > threshold:
+                for gm in (gu, gi):
+                    gm.arrays[0] = orc.h2f(gm.arrays[0]).astype(np.float32)
+                    gm.prec[0] = 1
+                    gm.refresh()
+                is_float, switched = True, e
+        Pn = gu.arrays[0] if gu.prec[0] else orc.h2f(gu.arrays[0])
+        Qn = gi.arrays[0] if gi.prec[0] else orc.h2f(gi.arrays[0])
+        P[...] = np.asarray(Pn, np.float32).reshape(P.shape)
+        Q[...] = np.asarray(Qn, np.float32).reshape(Q.shape)
+        rmse.append(orc.rmse(k, test, P, Q))
+    return np.array(rmse), switched, errors
+
+
 def oracle_train_mascot(orc, R, test, P, Q, k, W, epochs, lr, lam, decay, seed, ug, ig, sample_ratio, interval, threshold, threads=8):
     """mascot_training_mf, mf_methods.cu:36-434, on the CPU: shuffle, histogram, sort, grouping, re-index,
     scatter into binary16 groups, epochs with sampled error estimation and precision switching."""

@@ -79,6 +79,47 @@ def test_dense_variants_track_the_checker(orc, version, k):
         assert out["report"].muppet_final_bits in (8, 12, 14, 16, 32)
 
 
+@pytest.mark.parametrize("k", [64, 128])
+def test_binary16_storage_variant_tracks_the_checker(orc, k):
+    """-v 7 (the reference's default version): binary16 storage, binary32 arithmetic."""
+    h = mfutil.hip()
+    n_users, n_items = 3000, 1200
+    R = mfutil.make_ratings(91 + k, n_users, n_items, 250_000, rank=8, alpha=1.0)
+    train, test = _split(R, 200_000)
+    W, E = 4, 10
+    prm = h.default_params(k=k, num_workers=W, epoch=E, learning_rate=0.01, lam=0.05, decay=0.1, version=7, seed=5)
+    p, q = h.init_model(n_users, n_items, k, 5, half_rounded=True)
+    p0, q0 = p.copy(), q.copy()
+    out = h.train(prm, train, n_users, n_items, test, p, q)
+    ref = mfutil.oracle_train_mem_quant(orc, train, test, p0, q0, k, W, E, 0.01, 0.05, 0.1, 5)
+    print("gpu", out["rmse"], "\ncpu", ref)
+    assert out["rmse"][-1] < out["rmse"][0]
+    assert abs(out["rmse"][-1] - ref[-1]) < 0.005
+    assert np.array_equal(p, orc.h2f(orc.f2h(p)).reshape(p.shape))          # what comes back is binary16-representable
+    assert abs(orc.rmse(k, test, p, q) - out["rmse"][-1]) < 1e-6
+
+
+def test_whole_model_switching_variant_tracks_the_checker(orc):
+    """-v 8: the whole model in binary16 until the sampled error of both sides together exceeds the threshold."""
+    h = mfutil.hip()
+    n_users, n_items, k = 3000, 1200, 128
+    R = mfutil.make_ratings(17, n_users, n_items, 250_000, rank=8, alpha=1.0)
+    train, test = _split(R, 200_000)
+    W, E = 4, 14
+    prm = h.default_params(k=k, num_workers=W, epoch=E, learning_rate=0.01, lam=0.05, decay=0.1, version=8, seed=5,
+                           sample_ratio=0.05, interval=2, error_threshold=0.3)
+    p, q = h.init_model(n_users, n_items, k, 5, half_rounded=True)
+    p0, q0 = p.copy(), q.copy()
+    out = h.train(prm, train, n_users, n_items, test, p, q)
+    ref, switched, errors = mfutil.oracle_train_switching_only(orc, train, test, p0, q0, k, W, E, 0.01, 0.05, 0.1, 5, 0.05, 2, 0.3)
+    print("gpu", out["rmse"], "\ncpu", ref, "switched at", switched, errors)
+    assert abs(out["rmse"][-1] - ref[-1]) < 0.005
+    assert abs(orc.rmse(k, test, p, q) - out["rmse"][-1]) < 1e-6
+    # the run switched iff the model that comes back is no longer binary16-representable
+    gpu_switched = not np.array_equal(p, orc.h2f(orc.f2h(p)).reshape(p.shape))
+    assert gpu_switched == (switched >= 0)
+
+
 def test_mascot_reduced_config2(orc):
     """BASELINE config 2 at one tenth: Zipf(0.9), rank-16 truth, ratings 0.5-5.0 in half steps; MASCOT k=128,
     sample ratio 0.05, period 2; a low threshold so that groups do switch to binary32 within 12 epochs."""
@@ -148,7 +189,7 @@ def _write_tsv(path, R, offset=0):
             f.write("%d\t%d\t%g\n" % (u * 3 + 1 + offset, i * 2 + 5, r))
 
 
-@pytest.mark.parametrize("version", [1, 5])
+@pytest.mark.parametrize("version", [1, 5, 7])
 def test_quantized_mf_command_line(orc, tmp_path, version):
     """The C++ command line: reference flags in, per-epoch "<epoch> <lr> <rmse>" lines and the reference's
     model-file layout out (io_utils.h:242-332)."""

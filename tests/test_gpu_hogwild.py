@@ -39,6 +39,22 @@ def test_sgd_fp32_bit_exact(orc, k, W, uc, window):
 
 
 @pytest.mark.parametrize("k", [64, 128])
+@pytest.mark.parametrize("W,uc,window", [(1, 1, 1), (6, 3, 128), (9, 2, 70), (64, 2, 128)])
+def test_mem_quant_bit_exact(orc, k, W, uc, window):
+    """-v 7: dense binary16 rows, binary32 arithmetic, per-lane products summed left to right."""
+    import torch
+    h = mfutil.hip()
+    R, starts, P, Q = mfutil.conflict_free_problem(15 + k + W, k, W, uc, window)
+    Ph, Qh = orc.f2h(P).reshape(P.shape), orc.f2h(Q).reshape(Q.shape)
+    dR, dS, dP, dQ = to_dev(R), to_dev(starts), to_dev(Ph), to_dev(Qh)
+    h.mf_mem_quant_sgd_hogwild(dR.data_ptr(), R.size, dP.data_ptr(), dQ.data_ptr(), k, W, uc, window, LR, LAM, 1234, 0, dS.data_ptr(), mfutil.stream_ptr())
+    torch.cuda.synchronize()
+    orc.lib.orc_mem_quant_epoch(k, R.ctypes.data, R.size, Ph.ctypes.data, Qh.ctypes.data, W, uc, window, LR, LAM, 0, 0, starts.ctypes.data, 1)
+    assert np.array_equal(from_dev(dP, np.uint16, P.shape), Ph)
+    assert np.array_equal(from_dev(dQ, np.uint16, Q.shape), Qh)
+
+
+@pytest.mark.parametrize("k", [64, 128])
 @pytest.mark.parametrize("W,uc,window", [(1, 1, 1), (7, 3, 128), (64, 2, 128)])
 def test_mpt_bit_exact(orc, k, W, uc, window):
     R, starts, P, Q = mfutil.conflict_free_problem(20 + k + W, k, W, uc, window)

@@ -236,6 +236,39 @@ def test_fp32_sgd_is_a_gradient_step(orc, k):
 
 
 @pytest.mark.parametrize("k", [64, 128])
+def test_mem_quant_is_a_gradient_step_rounded_to_binary16(orc, k):
+    """-v 7: binary16 rows, binary32 arithmetic.  The new row is the fp64 gradient step from the stored values,
+    rounded to binary16: within half an ulp plus the binary32 arithmetic error; and the dot product is summed per
+    lane left to right, which a crafted row tells apart from the pairwise order of the fp32-SGD kernel."""
+    rng = np.random.default_rng(40 + k)
+    for _ in range(50):
+        p = (rng.standard_normal(k) * 0.2).astype(np.float16)
+        q = (rng.standard_normal(k) * 0.2).astype(np.float16)
+        r, lr, lam = float(rng.integers(1, 6)), 0.01, 0.05
+        gp, gq = _objective_grad(p.astype(np.float64), q.astype(np.float64), r, np.float64(np.float32(lam)))
+        p1, q1 = p.view(np.uint16).copy(), q.view(np.uint16).copy()
+        orc.lib.orc_mem_quant_update(k, p1.ctypes.data, q1.ctypes.data, r, lr, lam)
+        lr64 = np.float64(np.float32(lr))
+        for got, want in ((p1.view(np.float16), p - lr64 * gp), (q1.view(np.float16), q - lr64 * gq)):
+            ulp = np.spacing(np.abs(want).astype(np.float16)).astype(np.float64)
+            assert np.all(np.abs(got.astype(np.float64) - want) <= 0.5 * ulp + 1e-6)
+    if k == 128:
+        # lane 0 holds elements 0, 32, 64, 96 with products 2^24, 1, 1, 1.  In binary32, left to right:
+        # ((2^24 + 1) + 1) + 1 = 2^24 (every + 1 is a tie that rounds to even); pairwise: (2^24 + 1) + (1 + 1) = 2^24 + 2.
+        p = np.zeros(k, np.float16); q = np.zeros(k, np.float16)
+        p[[0, 32, 64, 96]] = [4096, 1, 1, 1]
+        q[[0, 32, 64, 96]] = [4096, 1, 1, 1]
+        f = np.float32
+        left_to_right = f(f(f(f(2 ** 24) + f(1)) + f(1)) + f(1))
+        pairwise = f(f(f(2 ** 24) + f(1)) + f(f(1) + f(1)))
+        assert left_to_right == 2 ** 24 and pairwise == 2 ** 24 + 2
+        p1, q1 = p.view(np.uint16).copy(), q.view(np.uint16).copy()
+        orc.lib.orc_mem_quant_update(k, p1.ctypes.data, q1.ctypes.data, float(2 ** 24), 0.25, 0.0)
+        assert p1.view(np.float16)[32] == 1.0            # r - dot = 0: nothing moves; the pairwise order would give 0.5
+        assert np.array_equal(p1, p.view(np.uint16)) and np.array_equal(q1, q.view(np.uint16))
+
+
+@pytest.mark.parametrize("k", [64, 128])
 def test_mascot_cases_are_gradient_steps_and_consistent(orc, k):
     """All four precision cases take the same gradient step up to their storage precision; the sampled
     statistics are that gradient (sign: ascent direction ruv*q - lambda*p) and its squared norm."""
@@ -413,6 +446,12 @@ def test_argument_checks_need_no_gpu(lib):
     prm = lib.default_params()
     assert (prm.k, prm.epoch, prm.num_workers, prm.version, prm.interval) == (128, 50, 2048, 7, 1)      # main.cu:19-32
     assert abs(prm.lambda_ - 0.015) < 1e-9 and abs(prm.sample_ratio - 0.01) < 1e-9
-    with pytest.raises(capi.MfError, match="version 7 is not built"):
+    prm.version = 9
+    with pytest.raises(capi.MfError, match="version 9 does not exist"):
         lib.call("mf_train", C.byref(prm), 1, 1, 1, 1, None, 0, 1, 1, None)
+    with pytest.raises(capi.MfError, match="ids outside the model|names user"):
+        from oracle.oracle import NODE
+        node = np.zeros(1, NODE); node["u"] = 5
+        p = np.zeros(128, np.float32); out = C.c_double(0)
+        lib.call("mf_gpu_test_rmse", node.ctypes.data, 1, p.ctypes.data, p.ctypes.data, 1, 1, 128, C.byref(out))
     assert lib.mf_set_row_coherence(1) == 0 and lib.mf_get_row_coherence() == 1
