@@ -1,13 +1,14 @@
 // MuPPET (block fixed point, muppet/muppet_sgd_kernel.h) and AFP (adaptive fixed point,
 // afp/afp_sgd_kernel.h) update rules over dense fp32 P/Q.
 //
-// Both rules derive per-rating scale factors from warp-wide statistics whose value depends on how
-// the reference groups elements per lane (lane l owns elements l, l+32, l+64, l+96 and sums them left
-// to right before the tree).  To keep those sums bit-identical, the wavefront mirrors the 32-lane
-// warp: lane L loads elements L and L+64, swaps with lane L^32, and then both half-waves hold, per
-// lane, the same 2 (k=64) or 4 (k=128) values the reference lane (L mod 32) holds.  All statistics are
-// computed redundantly in both halves with the reference's 16,8,4,2,1 tree; each lane finally
-// updates and stores only the elements it loaded.
+// Both rules derive per-rating scale factors from warp-wide statistics.  Lane L holds elements L and L+64 of a row
+// (k = 64: element L), i.e. the lower half-wave holds what the reference's lane l = L keeps as its 1st and 3rd value
+// (elements l, l+64) and the upper half-wave its 2nd and 4th (l+32, l+96).  Minima, maxima and the int8 dot product
+// are exact in any order, so they are plain 64-lane reductions.  Where the order of floating-point additions
+// matters it is reproduced: the binary16 dot keeps the reference's .x lane sums in the lower half-wave and the .y
+// sums in the upper one (two independent 16,8,4,2,1 trees, added at the end); squared norms pair the halves first,
+// (x[l]^2 + x[l+32]^2) + (x[l+64]^2 + x[l+96]^2).  Only AFP's occasional error measurement (QEM), whose per-lane
+// sums run left to right over all four values, rebuilds the 32-lane view (Mirror) in both half-waves.
 #pragma once
 #include "rules_fp32.h"
 
@@ -83,57 +84,55 @@ template <int K, bool COH> struct MuppetRule : DenseBase<K, COH> {
     float lrate, lambda; uint32_t first_sample; float* sum_updated_val; int fwd, bwd;
     float sum_norms_reg;
     float grad_acc[K / 64];
-    bool upper;
 
     __device__ __forceinline__ void init(const Params& a, uint8_t*, int lane_, uint32_t)
     {
         this->P = a.p; this->Q = a.q; this->lane = lane_; lrate = a.lrate; lambda = a.lambda;
         first_sample = a.first_sample; sum_updated_val = a.sum_updated_val; fwd = a.fwd; bwd = a.bwd;
-        sum_norms_reg = 0.f; upper = lane_ >= 32;
+        sum_norms_reg = 0.f;
 #pragma unroll
         for (int e = 0; e < E; ++e) grad_acc[e] = 0.f;
     }
+    // sum over the k values x[j]^2 in the reference's order: per lane (x0^2 + x1^2) + (x2^2 + x3^2); sq[e] = own squares
+    static __device__ __forceinline__ float lane_sum_of_squares(const float* sq)
+    {
+        float a = step_xor32(sq[0], OpAdd());
+        if constexpr (E == 2) { const float b = step_xor32(sq[1], OpAdd()); a = a + b; }
+        return a;
+    }
     template <int CLS> __device__ __forceinline__ void update(Row& row, const Info& i, uint32_t processed)
     {
-        Mirror<K> p, q;
-        p.build(row.p, upper); q.build(row.q, upper);
+        const float* p = row.p; const float* q = row.q;
         float p_min = 0, p_max = 0, q_min = 0, q_max = 0, sp = 0, sq = 0, pred;
         if (fwd != 32) {
-            p_min = p_max = p.v[0]; q_min = q_max = q.v[0];
-#pragma unroll
-            for (int j = 1; j < J; ++j) {
-                p_min = fminf(p_min, p.v[j]); p_max = fmaxf(p_max, p.v[j]);
-                q_min = fminf(q_min, q.v[j]); q_max = fmaxf(q_max, q.v[j]);
+            p_min = p_max = p[0]; q_min = q_max = q[0];
+            if constexpr (E == 2) {
+                p_min = fminf(p_min, p[1]); p_max = fmaxf(p_max, p[1]);
+                q_min = fminf(q_min, q[1]); q_max = fmaxf(q_max, q[1]);
             }
-            p_min = tree32(p_min, OpMin()); q_min = tree32(q_min, OpMin());
-            p_max = tree32(p_max, OpMax()); q_max = tree32(q_max, OpMax());
+            p_min = reduce_wave(p_min, OpMin()); q_min = reduce_wave(q_min, OpMin());
+            p_max = reduce_wave(p_max, OpMax()); q_max = reduce_wave(q_max, OpMax());
             sp = pow2u(muppet_scale_index((unsigned)fwd, p_max, p_min));
             sq = pow2u(muppet_scale_index((unsigned)fwd, q_max, q_min));
         }
         if (fwd == 8) {
             int acc = 0;
 #pragma unroll
-            for (int j = 0; j < J; ++j) acc += f2i8_sat(roundf(p.v[j] * sp)) * f2i8_sat(roundf(q.v[j] * sq));
-            acc = tree32(acc, OpAdd());
+            for (int e = 0; e < E; ++e) acc += f2i8_sat(roundf(p[e] * sp)) * f2i8_sat(roundf(q[e] * sq));
+            acc = reduce_wave(acc, OpAdd());
             pred = acc / (sp * sq);
         } else if (fwd == 32) {
-            float a = p.v[0] * q.v[0] + p.v[1] * q.v[1];
-            if constexpr (J == 4) { float b = p.v[2] * q.v[2] + p.v[3] * q.v[3]; a = a + b; }
-            pred = tree32(a, OpAdd());
+            float m[E];
+#pragma unroll
+            for (int e = 0; e < E; ++e) m[e] = p[e] * q[e];
+            pred = dot_reference_order<E, float>(m);
         } else {
             const float sp_rev = 1 / sp, sq_rev = 1 / sq;
-            // half2 lanes of the reference: .x = elements l (and l+64), .y = elements l+32 (and l+96)
-            half2_t t;
-            t.x = grid_h(p.v[0], sp, sp_rev) * grid_h(q.v[0], sq, sq_rev);
-            t.y = grid_h(p.v[1], sp, sp_rev) * grid_h(q.v[1], sq, sq_rev);
-            if constexpr (J == 4) {
-                half2_t t2;
-                t2.x = grid_h(p.v[2], sp, sp_rev) * grid_h(q.v[2], sq, sq_rev);
-                t2.y = grid_h(p.v[3], sp, sp_rev) * grid_h(q.v[3], sq, sq_rev);
-                t = t + t2;
-            }
-            t = tree32(t, OpAdd());
-            pred = (float)(half_t)(t.x + t.y);
+            // the reference's half2 lanes: .x sums elements l, l+64 (lower half-wave here), .y elements l+32, l+96 (upper)
+            half_t t = grid_h(p[0], sp, sp_rev) * grid_h(q[0], sq, sq_rev);
+            if constexpr (E == 2) t = t + grid_h(p[1], sp, sp_rev) * grid_h(q[1], sq, sq_rev);
+            t = reduce_half_wave(t, OpAdd());
+            pred = (float)(half_t)step_xor32(t, OpAdd());
         }
         const float ruv = i.r - pred;
         float sb = 0;
@@ -143,57 +142,48 @@ template <int K, bool COH> struct MuppetRule : DenseBase<K, COH> {
             const float bmax = fmaxf(fmaxf(p_max, q_max), fmaxf(neg_lambda, ruv));
             sb = pow2u(muppet_scale_index((unsigned)bwd, bmax, bmin));
         }
-        float gp[J], gq[J];
+        float gp[E], gq[E];
         if (bwd == 8) {
             const float sq_rev = 1 / (sb * sb);
             const int ruv_i = f2i8_sat(roundf(ruv * sb));
             const int lam_i = f2i8_sat(roundf(-1.0f * lambda * sb));
 #pragma unroll
-            for (int j = 0; j < J; ++j) {
-                const int pi = f2i8_sat(roundf(p.v[j] * sb)), qi = f2i8_sat(roundf(q.v[j] * sb));
-                gp[j] = (float)(qi * ruv_i + pi * lam_i) * sq_rev;
-                gq[j] = (float)(pi * ruv_i + qi * lam_i) * sq_rev;
+            for (int e = 0; e < E; ++e) {
+                const int pi = f2i8_sat(roundf(p[e] * sb)), qi = f2i8_sat(roundf(q[e] * sb));
+                gp[e] = (float)(qi * ruv_i + pi * lam_i) * sq_rev;
+                gq[e] = (float)(pi * ruv_i + qi * lam_i) * sq_rev;
             }
         } else if (bwd == 32) {
 #pragma unroll
-            for (int j = 0; j < J; ++j) {
-                gp[j] = ruv * q.v[j] - lambda * p.v[j];
-                gq[j] = ruv * p.v[j] - lambda * q.v[j];
+            for (int e = 0; e < E; ++e) {
+                gp[e] = ruv * q[e] - lambda * p[e];
+                gq[e] = ruv * p[e] - lambda * q[e];
             }
         } else {
             const float sb_rev = 1 / sb;
             const half_t t_ruv = grid_h(ruv, sb, sb_rev), t_lam = grid_h(-1 * lambda, sb, sb_rev);
 #pragma unroll
-            for (int j = 0; j < J; ++j) {
-                const half_t ph = grid_h(p.v[j], sb, sb_rev), qh = grid_h(q.v[j], sb, sb_rev);
-                gp[j] = (float)(half_t)(qh * t_ruv + ph * t_lam);
-                gq[j] = (float)(half_t)(ph * t_ruv + qh * t_lam);
+            for (int e = 0; e < E; ++e) {
+                const half_t ph = grid_h(p[e], sb, sb_rev), qh = grid_h(q[e], sb, sb_rev);
+                gp[e] = (float)(half_t)(qh * t_ruv + ph * t_lam);
+                gq[e] = (float)(half_t)(ph * t_ruv + qh * t_lam);
             }
         }
 #pragma unroll
         for (int e = 0; e < E; ++e) {
-            float g = upper ? gp[2 * e + 1] : gp[2 * e];
-            float h = upper ? gq[2 * e + 1] : gq[2 * e];
-            row.p[e] = row.p[e] + lrate * g;
-            row.q[e] = row.q[e] + lrate * h;
+            row.p[e] = row.p[e] + lrate * gp[e];
+            row.q[e] = row.q[e] + lrate * gq[e];
         }
         this->store(row, i);
         if (fwd != 32 && bwd != 32 && processed >= first_sample) {
-            float np = gp[0] * gp[0] + gp[1] * gp[1];
-            float nq = gq[0] * gq[0] + gq[1] * gq[1];
-            if constexpr (J == 4) {
-                float b = gp[2] * gp[2] + gp[3] * gp[3]; np = np + b;
-                float c = gq[2] * gq[2] + gq[3] * gq[3]; nq = nq + c;
-            }
-            float npq = np + nq;
-            npq = tree32(npq, OpAdd());
+            float sp2[E], sq2[E];
+#pragma unroll
+            for (int e = 0; e < E; ++e) { sp2[e] = gp[e] * gp[e]; sq2[e] = gq[e] * gq[e]; }
+            float npq = lane_sum_of_squares(sp2) + lane_sum_of_squares(sq2);
+            npq = reduce_half_wave(npq, OpAdd());
             sum_norms_reg += npq;
 #pragma unroll
-            for (int e = 0; e < E; ++e) {
-                float g = upper ? gp[2 * e + 1] : gp[2 * e];
-                float h = upper ? gq[2 * e + 1] : gq[2 * e];
-                grad_acc[e] += g + h;       // flushed once per worker in finish()
-            }
+            for (int e = 0; e < E; ++e) grad_acc[e] += gp[e] + gq[e];       // flushed once per worker in finish()
         }
     }
     __device__ __forceinline__ void finish(const Params& a, uint32_t wid) const
@@ -287,14 +277,15 @@ template <int K, bool COH> struct AfpRule : DenseBase<K, COH> {
     }
     template <int CLS> __device__ __forceinline__ void update(Row& row, const Info& i, uint32_t)
     {
-        Mirror<K> p, q;
-        p.build(row.p, upper); q.build(row.q, upper);
-        float p_abs = fabsf(p.v[0]), q_abs = fabsf(q.v[0]);
-#pragma unroll
-        for (int j = 1; j < J; ++j) { p_abs = fmaxf(p_abs, fabsf(p.v[j])); q_abs = fmaxf(q_abs, fabsf(q.v[j])); }
+        const float* p = row.p; const float* q = row.q;
+        float p_abs = fabsf(p[0]), q_abs = fabsf(q[0]);
+        if constexpr (E == 2) { p_abs = fmaxf(p_abs, fabsf(p[1])); q_abs = fmaxf(q_abs, fabsf(q[1])); }
+        // the three re-measurements below happen every itv-th update of the worker; they sum their error terms per
+        // lane from left to right over all four values, so they work on the 32-lane view
         if (cur_iter == upd_u) {
-            const float mx = tree32(p_abs, OpMax());
-            const float diff = qem(p.v, mx);
+            Mirror<K> pm; pm.build(row.p, upper);
+            const float mx = reduce_wave(p_abs, OpMax());
+            const float diff = qem(pm.v, mx);
             if (cur_iter == 0) uq.mov_avg_range = mx;
             uq = uniform(afp_qpa(diff, mx, uq.mov_avg_range));
             sp = pow2i(uq.r);
@@ -302,8 +293,9 @@ template <int K, bool COH> struct AfpRule : DenseBase<K, COH> {
             upd_u += uq.itv;
         }
         if (cur_iter == upd_i) {
-            const float mx = tree32(q_abs, OpMax());
-            const float diff = qem(q.v, mx);
+            Mirror<K> qm; qm.build(row.q, upper);
+            const float mx = reduce_wave(q_abs, OpMax());
+            const float diff = qem(qm.v, mx);
             if (cur_iter == 0) iq.mov_avg_range = mx;
             iq = uniform(afp_qpa(diff, mx, iq.mov_avg_range));
             sq = pow2i(iq.r);
@@ -314,62 +306,55 @@ template <int K, bool COH> struct AfpRule : DenseBase<K, COH> {
         if (uq.n == 8 && iq.n == 8) {
             int acc = 0;
 #pragma unroll
-            for (int j = 0; j < J; ++j) acc += afp_sat8(roundf(p.v[j] * sp)) * afp_sat8(roundf(q.v[j] * sq));
-            acc = tree32(acc, OpAdd());
+            for (int e = 0; e < E; ++e) acc += afp_sat8(roundf(p[e] * sp)) * afp_sat8(roundf(q[e] * sq));
+            acc = reduce_wave(acc, OpAdd());
             pred = acc / (sp * sq);
         } else {
             const float sp_rev = 1 / sp, sq_rev = 1 / sq;
-            half2_t t;
-            t.x = (half_t)afp_grid(p.v[0], sp, sp_rev) * (half_t)afp_grid(q.v[0], sq, sq_rev);
-            t.y = (half_t)afp_grid(p.v[1], sp, sp_rev) * (half_t)afp_grid(q.v[1], sq, sq_rev);
-            if constexpr (J == 4) {
-                half2_t t2;
-                t2.x = (half_t)afp_grid(p.v[2], sp, sp_rev) * (half_t)afp_grid(q.v[2], sq, sq_rev);
-                t2.y = (half_t)afp_grid(p.v[3], sp, sp_rev) * (half_t)afp_grid(q.v[3], sq, sq_rev);
-                t = t + t2;
-            }
-            t = tree32(t, OpAdd());
-            pred = (float)(half_t)(t.x + t.y);
+            // the reference's half2 lanes: .x sums elements l, l+64 (lower half-wave here), .y elements l+32, l+96 (upper)
+            half_t t = (half_t)afp_grid(p[0], sp, sp_rev) * (half_t)afp_grid(q[0], sq, sq_rev);
+            if constexpr (E == 2) t = t + (half_t)afp_grid(p[1], sp, sp_rev) * (half_t)afp_grid(q[1], sq, sq_rev);
+            t = reduce_half_wave(t, OpAdd());
+            pred = (float)(half_t)step_xor32(t, OpAdd());
         }
         const float ruv = i.r - pred;
         if (cur_iter == upd_b) {
+            Mirror<K> pm, qm; pm.build(row.p, upper); qm.build(row.q, upper);
             float mx = fmaxf(p_abs, q_abs);
             mx = fmaxf(fmaxf(mx, fabsf(lambda)), fabsf(ruv));
-            mx = tree32(mx, OpMax());
-            const float diff = qem_bp(p.v, q.v, ruv, mx);
+            mx = reduce_wave(mx, OpMax());
+            const float diff = qem_bp(pm.v, qm.v, ruv, mx);
             if (cur_iter == 0) bq.mov_avg_range = mx;
             bq = uniform(afp_qpa(diff, mx, bq.mov_avg_range));
             sb = pow2i(bq.r);
             if (afp_epoch == 0 && cur_iter < init_threshold) bq.itv = 1;
             upd_b += bq.itv;
         }
-        float gp[J], gq[J];
+        float gp[E], gq[E];
         if (bq.n == 8) {
             const int lam_i = afp_sat8(roundf(-1.0f * lambda * sb));
             const int ruv_i = afp_sat8(roundf(ruv * sb));
             const float sq_rev = 1 / (sb * sb);
 #pragma unroll
-            for (int j = 0; j < J; ++j) {
-                const int pi = afp_sat8(roundf(p.v[j] * sb)), qi = afp_sat8(roundf(q.v[j] * sb));
-                gp[j] = (float)(qi * ruv_i + pi * lam_i) * sq_rev;
-                gq[j] = (float)(pi * ruv_i + qi * lam_i) * sq_rev;
+            for (int e = 0; e < E; ++e) {
+                const int pi = afp_sat8(roundf(p[e] * sb)), qi = afp_sat8(roundf(q[e] * sb));
+                gp[e] = (float)(qi * ruv_i + pi * lam_i) * sq_rev;
+                gq[e] = (float)(pi * ruv_i + qi * lam_i) * sq_rev;
             }
         } else {
             const float sb_rev = 1 / sb;
             const half_t t_ruv = (half_t)afp_grid(ruv, sb, sb_rev), t_lam = (half_t)afp_grid(-1.0f * lambda, sb, sb_rev);
 #pragma unroll
-            for (int j = 0; j < J; ++j) {
-                const half_t ph = (half_t)afp_grid(p.v[j], sb, sb_rev), qh = (half_t)afp_grid(q.v[j], sb, sb_rev);
-                gp[j] = (float)(half_t)(qh * t_ruv + ph * t_lam);
-                gq[j] = (float)(half_t)(ph * t_ruv + qh * t_lam);
+            for (int e = 0; e < E; ++e) {
+                const half_t ph = (half_t)afp_grid(p[e], sb, sb_rev), qh = (half_t)afp_grid(q[e], sb, sb_rev);
+                gp[e] = (float)(half_t)(qh * t_ruv + ph * t_lam);
+                gq[e] = (float)(half_t)(ph * t_ruv + qh * t_lam);
             }
         }
 #pragma unroll
         for (int e = 0; e < E; ++e) {
-            const float g = upper ? gp[2 * e + 1] : gp[2 * e];
-            const float h = upper ? gq[2 * e + 1] : gq[2 * e];
-            row.p[e] = row.p[e] + lrate * g;
-            row.q[e] = row.q[e] + lrate * h;
+            row.p[e] = row.p[e] + lrate * gp[e];
+            row.q[e] = row.q[e] + lrate * gq[e];
         }
         this->store(row, i);
         cur_iter += 1;
