@@ -314,8 +314,8 @@ def measured_traffic(a, leg):
         return None
     if a.skip_coherent:
         return (14_053_967 * 2.0 + 24_189_917) * 1024 if leg["workers"] == 16384 else None
-    if leg["workers"] in (6104, 6144) and a.hot_row_inflight == 2.0 and a.warmup >= a.hot_row_early_epochs:
-        return (16_032_418 * 2.0 + 27_715_099) * 1024
+    if leg["workers"] == 6104 and a.hot_row_inflight == 2.0 and a.warmup >= a.hot_row_early_epochs:
+        return (15_939_771 * 2.0 + 27_557_326) * 1024
     return None
 
 
@@ -335,7 +335,7 @@ def main():
     ap.add_argument("--skip-coherent", action="store_true", help="profiling aid: time only the cached-rows leg")
     ap.add_argument("--skip-exact", action="store_true", help="skip the leg with every row update carried out (no thinning)")
     ap.add_argument("--hot-row-inflight", type=float, default=2.0, help="hot rows of the measured run are thinned to this many updates in flight (0 = no hot rows)")
-    ap.add_argument("--hot-row-inflight-early", type=float, default=16.0, help="the same cap during the first epochs")
+    ap.add_argument("--hot-row-inflight-early", type=float, default=8.0, help="the same cap during the first epochs")
     ap.add_argument("--hot-row-early-epochs", type=int, default=2, help="number of epochs that run with the early cap")
     ap.add_argument("--pmc-copy", action="store_true",
                     help="profiling aid: also run three 1 GiB device copies, the known-size kernel that FETCH_SIZE / WRITE_SIZE are scaled by")

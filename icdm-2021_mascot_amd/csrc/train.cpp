@@ -91,7 +91,7 @@ void fill_schedule(Common& c)
     }
 }
 
-void report_epoch(Common& c, uint32_t e, double rmse, float sgd_ms)
+int report_epoch(Common& c, uint32_t e, double rmse, float sgd_ms)
 {
     if (c.rep) {
         if (c.rep->rmse_per_epoch) c.rep->rmse_per_epoch[e] = rmse;
@@ -99,6 +99,10 @@ void report_epoch(Common& c, uint32_t e, double rmse, float sgd_ms)
         c.rep->sgd_ms += sgd_ms;
     }
     if (c.prm->verbose) { std::printf("%u %g %g\n", e + 1, (double)c.lr[e], rmse); std::fflush(stdout); }   // mf_methods.cu:396
+    if (c.test_n && !std::isfinite(rmse))
+        return invalid("mf_train: the model diverged in epoch %u (the test RMSE is not finite); lower the learning rate, or the "
+                       "hot-row caps (hot_row_inflight_early, hot_row_inflight) if hot rows are on", e + 1);
+    return 0;
 }
 
 int finish_rmse(Common& c, double* out)
@@ -337,7 +341,7 @@ int train_dense(Common& c, float* p, float* q)
         }
         double rmse = 0;
         MF_TRY(dense_rmse(c, d_p.as<float>(), d_q.as<float>(), &rmse));
-        report_epoch(c, e, rmse, sgd_ms);
+        MF_TRY(report_epoch(c, e, rmse, sgd_ms));
 
         if (version == 3) {      // mf_methods.cu:659-697
             const double e0 = now_ms();
@@ -581,7 +585,7 @@ int train_mascot(Common& c, float* p, float* q)
                                     U.groups, I.groups, c.d_sum_sq.as<double>(), nullptr));
         double rmse = 0;
         MF_TRY(finish_rmse(c, &rmse));
-        report_epoch(c, e, rmse, sgd_ms);
+        MF_TRY(report_epoch(c, e, rmse, sgd_ms));
     }
 
     {   // trained model back to the host in sorted row order (what save_trained_model_reconst writes)
@@ -616,7 +620,7 @@ void mf_default_params(mf_params* out)       // main.cu:19-32
     out->lambda = 0.015f; out->learning_rate = 0.01f; out->decay = 0.1f; out->sample_ratio = 0.01f; out->error_threshold = 0.001f;
     out->k = 128; out->epoch = 50; out->num_workers = 2048; out->thread_block_size = 128;
     out->user_group_num = 10; out->item_group_num = 10; out->version = 7; out->interval = 1; out->seed = 1;
-    out->hot_row_inflight = 2.0f; out->hot_row_inflight_early = 16.0f; out->hot_row_early_epochs = 2;   // no reference counterpart: see mf_set_hot_row_thinning
+    out->hot_row_inflight = 2.0f; out->hot_row_inflight_early = 8.0f; out->hot_row_early_epochs = 2;   // no reference counterpart: see mf_set_hot_row_thinning
 }
 
 uint32_t mf_group_end_indices(const uint32_t* sorted_cnt, uint32_t n, uint32_t requested_groups, uint32_t* end_idx_out)

@@ -227,8 +227,9 @@ typedef struct {
     float hot_row_inflight;   /* > 0: rows expected to have more than one update in flight become hot rows, thinned
                                  to at most this many updates in flight (see mf_set_hot_row_thinning); 0 = off */
     float hot_row_inflight_early; /* the cap during the first hot_row_early_epochs epochs, while all rows still grow
-                                 from their small initial values and popular rows need many updates (default 16 for
-                                 2 epochs, then hot_row_inflight = 2) */
+                                 from their small initial values and popular rows need many updates (default 8 for
+                                 2 epochs, then hot_row_inflight = 2; 16 diverges in one run of sixteen at 100M
+                                 ratings) */
     uint32_t hot_row_early_epochs;
 } mf_params;
 

@@ -240,7 +240,7 @@ def test_argument_errors_launch_nothing():
 
 
 @pytest.mark.parametrize("k", [64, 128])
-@pytest.mark.parametrize("variant", ["single", "mascot"])
+@pytest.mark.parametrize("variant", ["single", "mascot", "mascot_ff", "mascot_hf"])
 def test_hot_row_thinning_drops_whole_row_updates(orc, k, variant):
     """mf_set_hot_row_thinning: 255 = ordinary row, nothing changes; 254 = hot row, every update carried out (added
     in memory: with one update per row the sum equals the stored row, up to the extra rounding of the binary16
@@ -256,9 +256,17 @@ def test_hot_row_thinning_drops_whole_row_updates(orc, k, variant):
     Q0 = (rng.standard_normal((n, k)) * 0.1).astype(np.float32)
     starts = np.arange(0, n, 128, dtype=np.uint32).reshape(-1, 1)          # one worker, consecutive windows
     uc = starts.shape[0]
-    if variant == "mascot":
-        P0, Q0 = orc.h2f(orc.f2h(P0)), orc.h2f(orc.f2h(Q0))
+    uprec = np.array([1 if variant == "mascot_ff" else 0], np.uint8)       # binary32 user rows / item rows
+    iprec = np.array([0 if variant == "mascot" else 1], np.uint8)
+    if variant != "single":
+        if not uprec[0]:
+            P0 = orc.h2f(orc.f2h(P0)).reshape(P0.shape)
+        if not iprec[0]:
+            Q0 = orc.h2f(orc.f2h(Q0)).reshape(Q0.shape)
         end = np.array([n - 1], np.uint32)
+
+    def rows(a):
+        return (a if a.dtype == np.float32 else orc.h2f(a)).reshape(n, k).astype(np.float32)
 
     def run(keep_u, keep_v):
         dR, dS = to_dev(R), to_dev(starts)
@@ -271,8 +279,8 @@ def test_hot_row_thinning_drops_whole_row_updates(orc, k, variant):
                 h.mf_single_sgd_hogwild(dR.data_ptr(), n, dP.data_ptr(), dQ.data_ptr(), k, 1, uc, 128, LR, LAM, 5, 0, dS.data_ptr(), mfutil.stream_ptr())
                 torch.cuda.synchronize()
                 return from_dev(dP, np.float32, P0.shape), from_dev(dQ, np.float32, Q0.shape)
-            gp = mfutil.host_grouped(orc, k, P0, end, np.zeros(1, np.uint8))
-            gq = mfutil.host_grouped(orc, k, Q0, end, np.zeros(1, np.uint8))
+            gp = mfutil.host_grouped(orc, k, P0, end, uprec)
+            gq = mfutil.host_grouped(orc, k, Q0, end, iprec)
             dp, dq = mfutil.DeviceGrouped(gp), mfutil.DeviceGrouped(gq)
             z = torch.zeros(4 * k + 16, dtype=torch.float32, device="cuda")
             h.mf_mascot_sgd_hogwild(dR.data_ptr(), n, dp.ptrs.data_ptr(), dq.ptrs.data_ptr(), k, 1, uc, 128, LR, LAM,
@@ -280,7 +288,7 @@ def test_hot_row_thinning_drops_whole_row_updates(orc, k, variant):
                                     z.data_ptr(), z[k:].data_ptr(), z[2 * k:].data_ptr(), z[3 * k:].data_ptr(),
                                     uc * 128, 1, 1, 5, 0, dS.data_ptr(), mfutil.stream_ptr())
             torch.cuda.synchronize()
-            return orc.h2f(dp.download()[0]).reshape(n, k), orc.h2f(dq.download()[0]).reshape(n, k)
+            return rows(dp.download()[0]), rows(dq.download()[0])
         finally:
             torch.cuda.synchronize()
             h.mf_set_hot_row_thinning(None, None)
@@ -290,30 +298,32 @@ def test_hot_row_thinning_drops_whole_row_updates(orc, k, variant):
         Pw, Qw = P0.copy(), Q0.copy()
         orc.lib.orc_sgd_epoch(k, R.ctypes.data, n, Pw.ctypes.data, Qw.ctypes.data, 1, uc, 128, LR, LAM, 5, 0, starts.ctypes.data, 1)
     else:
-        gp = mfutil.host_grouped(orc, k, P0, end, np.zeros(1, np.uint8))
-        gq = mfutil.host_grouped(orc, k, Q0, end, np.zeros(1, np.uint8))
+        gp = mfutil.host_grouped(orc, k, P0, end, uprec)
+        gq = mfutil.host_grouped(orc, k, Q0, end, iprec)
         z = [np.zeros(k, np.float32) for _ in range(4)]
         orc.lib.orc_mascot_epoch(k, R.ctypes.data, n, gp.ptrs, gq.ptrs, gp.end_idx.ctypes.data, gq.end_idx.ctypes.data,
                                  gp.prec.ctypes.data, gq.prec.ctypes.data, 1, 1, 1, uc, 128, LR, LAM, uc * 128,
                                  z[0].ctypes.data, z[1].ctypes.data, z[2].ctypes.data, z[3].ctypes.data, 5, 0, starts.ctypes.data, 1)
-        Pw, Qw = orc.h2f(gp.arrays[0]).reshape(n, k), orc.h2f(gq.arrays[0]).reshape(n, k)
-    def same(got, want, old):
-        if variant == "single":                                     # fp32: old + change is the stored value
+        Pw, Qw = rows(gp.arrays[0]), rows(gq.arrays[0])
+
+    def same(got, want, old, binary32=False):
+        if variant == "single":                                     # fp32 SGD: old + change is the stored value
             return np.array_equal(got, want)
-        # binary16: memory adds round(lr*g) to the row, the rule stores fma(lr, g, row); the extra rounding is the
-        # one of the change, so the two are within one ulp of the larger of the change and the result
-        scale = np.maximum(np.abs(want), np.abs(want - old)).astype(np.float16)
+        # MASCOT: memory adds round(lr*g) to the row, the rule stores fma(lr, g, row); the extra rounding is the one of
+        # the change, so the two are within one ulp (of the row's format) of the larger of the change and the result
+        fmt = np.float32 if binary32 else np.float16
+        scale = np.maximum(np.abs(want), np.abs(want - old)).astype(fmt)
         return np.all(np.abs(got.astype(np.float64) - want) <= np.spacing(scale).astype(np.float64))
 
     P1, Q1 = run(255, 255)
     assert np.array_equal(P1, Pw) and np.array_equal(Q1, Qw)
     P4, Q4 = run(254, 254)
-    assert same(P4, Pw, P0) and same(Q4, Qw, Q0)
+    assert same(P4, Pw, P0, uprec[0]) and same(Q4, Qw, Q0, iprec[0])
     assert np.all(np.any(P4 != P0, axis=1)) and np.all(np.any(Q4 != Q0, axis=1))
     P2, Q2 = run(63, 255)
     assert np.array_equal(Q2, Qw)                                   # item side: every update, computed from the old user row
     changed = np.any(P2 != P0, axis=1)
-    assert same(P2[changed], Pw[changed], P0[changed])                           # a user row is either untouched or fully updated
+    assert same(P2[changed], Pw[changed], P0[changed], uprec[0])                           # a user row is either untouched or fully updated
     assert np.array_equal(P2[~changed], P0[~changed])
     assert 0.20 < changed.mean() < 0.30                             # (63+1)/255 of the updates
     P3, Q3 = run(255, 0)
