@@ -9,7 +9,7 @@
 
 namespace mf {
 
-// hot-row thinning tables (device pointers, see Schedule::keep_u); null = off
+// hot-row tables (device pointers, see Schedule::keep_u); null = off
 static const uint8_t* g_keep_u = nullptr;
 static const uint8_t* g_keep_v = nullptr;
 static thread_local char g_error[512] = "";
@@ -42,7 +42,7 @@ static Schedule make_schedule(const mf_node* R, uint32_t nnz, uint32_t num_worke
 }
 static inline uint32_t grid_for(uint32_t num_workers) { return (num_workers + kWavesPerBlock - 1) / kWavesPerBlock; }
 
-// 0: ordinary cached row accesses, 1: agent-scope coherent row accesses (see row_load in mf_device.h)
+// 0: ordinary write-back row stores, 1: agent-scope coherent row stores (see row_store in mf_device.h)
 static int g_row_coherence = 1;
 // number of consecutive kernel launches one call is cut into (each worker's windows are split evenly);
 // a kernel boundary writes back and invalidates the per-XCD L2s, which is how cached row copies of

@@ -40,11 +40,13 @@ typedef struct { float r; uint32_t u; uint32_t i; } mf_node;
 int mf_version(void);
 const char* mf_last_error(void);
 /* How the update kernels read and write P/Q rows (process-wide, takes effect at the next launch):
- *   1 (default)  device-coherent: every row access bypasses the per-XCD L2 (agent-scope relaxed atomics),
- *                so a worker always sees the latest row any other worker stored -- the semantics the
- *                reference gets from a GPU with one L2.  All accesses to one row serialise at the
- *                memory side, which bounds the epoch when a single row takes percents of all ratings.
- *   0            cached: ordinary loads and stores; each of the 8 XCDs works on its own L2-resident copy
+ *   1 (default)  device-coherent: every row store writes through the per-XCD L2 to the memory side and drops the
+ *                copies other L2s hold (agent-scope relaxed atomic stores; loads stay ordinary cached loads),
+ *                so a worker sees the latest row any other worker stored -- the semantics the reference
+ *                gets from a GPU with one L2.  All stores to one row serialise at the memory side, which
+ *                bounds the epoch when a single row takes percents of all ratings (see
+ *                mf_set_hot_row_thinning for what mf_train does about that).
+ *   0            cached: ordinary write-back stores; each of the 8 XCDs works on its own L2-resident copy
  *                of a hot row until it is evicted, copies are merged last-writer-wins.
  * No counterpart in the reference (one L2, nothing to choose).  mf_train picks per run, see there. */
 int mf_set_row_coherence(int coherent);
@@ -222,7 +224,7 @@ typedef struct {
     uint32_t is_yahoo;        /* MuPPET starts at 12 bit (mf_methods.cu:600) */
     uint64_t seed;            /* replaces time(0) / clock() seeding */
     uint32_t verbose;         /* 1: print the reference's stdout lines (mf_methods.cu:396 etc.) */
-    uint32_t cached_rows;     /* 0: device-coherent row accesses (default), 1: cached, see mf_set_row_coherence */
+    uint32_t cached_rows;     /* 0: device-coherent row stores (default), 1: cached, see mf_set_row_coherence */
     uint32_t epoch_splits;    /* kernel launches per epoch, 0 or 1 = one, see mf_set_epoch_splits */
     float hot_row_inflight;   /* > 0: rows expected to have more than one update in flight become hot rows, thinned
                                  to at most this many updates in flight (see mf_set_hot_row_thinning); 0 = off */
