@@ -65,8 +65,20 @@ struct Common {
     mf_report* rep;
 };
 
+// The kernels index P and Q with the ids in the ratings and cannot know the row counts: check them here, on the
+// host, where a bad id is an error message and not an out-of-bounds access on the device.
+int check_ids(const char* what, const mf_node* R, uint32_t n, uint32_t n_users, uint32_t n_items)
+{
+    for (uint32_t i = 0; i < n; ++i)
+        if (R[i].u >= n_users || R[i].i >= n_items)
+            return invalid("mf_train: %s rating %u names user %u / item %u, the model has %u users and %u items", what, i, R[i].u, R[i].i, n_users, n_items);
+    return 0;
+}
+
 int upload_and_shuffle(Common& c, const mf_node* R, const mf_node* test)
 {
+    MF_TRY(check_ids("training", R, c.n, c.n_users, c.n_items));
+    MF_TRY(check_ids("test", test, c.test_n, c.n_users, c.n_items));
     DevBuf staging;
     MF_TRY(staging.alloc((size_t)c.n * sizeof(mf_node), "hipMalloc(ratings staging)"));
     MF_TRY(c.d_R.alloc((size_t)c.n * sizeof(mf_node), "hipMalloc(ratings)"));

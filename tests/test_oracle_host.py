@@ -446,9 +446,15 @@ def test_argument_checks_need_no_gpu(lib):
     prm = lib.default_params()
     assert (prm.k, prm.epoch, prm.num_workers, prm.version, prm.interval) == (128, 50, 2048, 7, 1)      # main.cu:19-32
     assert abs(prm.lambda_ - 0.015) < 1e-9 and abs(prm.sample_ratio - 0.01) < 1e-9
+    from oracle.oracle import NODE
     prm.version = 9
     with pytest.raises(capi.MfError, match="version 9 does not exist"):
         lib.call("mf_train", C.byref(prm), 1, 1, 1, 1, None, 0, 1, 1, None)
+    prm.version = 5
+    bad = np.zeros(3, NODE); bad["i"][2] = 7
+    pq = np.zeros(4 * 128, np.float32)
+    with pytest.raises(capi.MfError, match="training rating 2 names user 0 / item 7"):
+        lib.call("mf_train", C.byref(prm), bad.ctypes.data, 3, 4, 4, None, 0, pq.ctypes.data, pq.ctypes.data, None)
     with pytest.raises(capi.MfError, match="ids outside the model|names user"):
         from oracle.oracle import NODE
         node = np.zeros(1, NODE); node["u"] = 5
