@@ -62,7 +62,51 @@ __device__ __forceinline__ void process_chunk(Rule& rule, const Rating& my, cons
     }
 }
 
-template <class Rule>
+// A chunk of exactly kWave ratings (the usual case: windows are multiples of 64).  Same pipeline, but every
+// memory instruction of the steady state sits on a straight line: loads that are issued under a condition make
+// the compiler's wait-count bookkeeping fall back to "wait for everything", which turns the look-ahead into one
+// full memory latency per rating.  Ring slots start out with row ids nothing can match, so the first ratings
+// need no special case either.
+template <class Rule, int CLS, bool HOT>
+__device__ __forceinline__ void process_full_chunk(Rule& rule, const Rating& my, const typename Rule::Prep& prep, uint32_t processed)
+{
+    constexpr int A = Rule::kAhead;
+    constexpr int S = Rule::kRing;
+    static_assert(S >= 2 * A + 1 && kWave % S == 0, "the ring divides a full chunk");
+    typename Rule::Row ring[S];
+    typename Rule::Info inf[S];
+    static_for<0, S>([&](auto D) { inf[decltype(D)::value] = rule.no_row(); });
+    auto fetch_rows = [&](auto SL, int j) {
+        constexpr int sl = decltype(SL)::value;
+        inf[sl] = rule.info(my, prep, j);
+        if constexpr (!HOT) inf[sl].thin = 0u;
+        rule.template load<CLS>(ring[sl], inf[sl]);
+    };
+    auto step = [&](auto D, int j) {
+        constexpr int d = decltype(D)::value;
+        static_for<0, A>([&](auto H) {
+            constexpr int h = A - decltype(H)::value;          // A, A-1, ..., 1: newest wins
+            constexpr int sh = (d - h + 2 * S) % S;
+            rule.forward(ring[d], inf[d], ring[sh], inf[sh]);
+        });
+        rule.template update<CLS>(ring[d], inf[d], processed + (uint32_t)j);
+    };
+    static_for<0, A>([&](auto D) { fetch_rows(D, decltype(D)::value); });
+    for (int j0 = 0; j0 < kWave - S; j0 += S) {
+        static_for<0, S>([&](auto D) {
+            constexpr int d = decltype(D)::value;
+            fetch_rows(std::integral_constant<int, (d + A) % S>(), j0 + d + A);
+            step(D, j0 + d);
+        });
+    }
+    static_for<0, S>([&](auto D) {
+        constexpr int d = decltype(D)::value;
+        if constexpr (d + A < S) fetch_rows(std::integral_constant<int, d + A>(), kWave - S + d + A);
+        step(D, kWave - S + d);
+    });
+}
+
+template <class Rule, bool HOT>
 __global__ __launch_bounds__(kMaxBlock) void hogwild_kernel(Schedule s, typename Rule::Params prm)
 {
     extern __shared__ __align__(16) uint8_t smem[];
@@ -97,7 +141,7 @@ __global__ __launch_bounds__(kMaxBlock) void hogwild_kernel(Schedule s, typename
                 uint32_t idx = st + off;
                 if (idx >= s.nnz || idx < st) idx -= s.nnz;
                 x = load_rating(s.R, idx);
-                if (s.keep_u) {
+                if constexpr (HOT) {
                     const uint32_t rnd = (uint32_t)(mix64(s.epoch_key ^ (((uint64_t)idx << 20) ^ (uint64_t)wid ^ 0x7468696eull)) >> 40);
                     const uint32_t ku = s.keep_u[x.u], kv = s.keep_v[x.v];
                     // two independent draws, uniform over 0..254
@@ -125,8 +169,18 @@ __global__ __launch_bounds__(kMaxBlock) void hogwild_kernel(Schedule s, typename
             const bool valid = lane < n;
             typename Rule::Prep prep = rule.prepare(my, valid);
             const int cls = rule.classify(prep, valid);
-            if (Rule::kClasses > 1 && cls == 1) process_chunk<Rule, 1>(rule, my, prep, n, processed);
-            else process_chunk<Rule, 0>(rule, my, prep, n, processed);
+            // classes (see the rules): 1 and 2 promise ratings that all take the same memory instructions; full
+            // chunks of those run the straight-line pipeline, everything else the general one
+            if (Rule::kClasses > 1 && cls == 1) {
+                if (n == kWave) process_full_chunk<Rule, 1, HOT>(rule, my, prep, processed);
+                else process_chunk<Rule, 1>(rule, my, prep, n, processed);
+            } else if (Rule::kClasses > 2 && cls == 2 && n == kWave) {
+                process_full_chunk<Rule, 2, HOT>(rule, my, prep, processed);
+            } else if (Rule::kClasses == 1 && n == kWave) {
+                process_full_chunk<Rule, 0, HOT>(rule, my, prep, processed);
+            } else {
+                process_chunk<Rule, 0>(rule, my, prep, n, processed);
+            }
             if (!more) break;
             processed = nprocessed; c = nc; ite = nite; start = nstart; n = nn; my = nmy;
         }

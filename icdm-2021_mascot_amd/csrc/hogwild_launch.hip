@@ -59,8 +59,16 @@ struct Range {
 template <class P> static auto set_lds_stats(P& p, bool v) -> decltype(p.lds_stats, void()) { p.lds_stats = v; }
 static void set_lds_stats(...) {}
 
+template <class Rule, bool HOT>
+static int launch_hot(const char* who, const Schedule& s0, const typename Rule::Params& prm0, size_t lds, void* stream, Range r);
+// the kernel comes in two builds: with and without the hot-row code (Schedule::keep_u)
 template <class Rule>
 static int launch(const char* who, const Schedule& s0, const typename Rule::Params& prm0, size_t lds, void* stream, Range r)
+{
+    return s0.keep_u ? launch_hot<Rule, true>(who, s0, prm0, lds, stream, r) : launch_hot<Rule, false>(who, s0, prm0, lds, stream, r);
+}
+template <class Rule, bool HOT>
+static int launch_hot(const char* who, const Schedule& s0, const typename Rule::Params& prm0, size_t lds, void* stream, Range r)
 {
     if (s0.update_count == 0 || s0.update_vector_size == 0 || r.begin >= r.end) return MF_OK;
     Schedule s = s0;
@@ -70,10 +78,10 @@ static int launch(const char* who, const Schedule& s0, const typename Rule::Para
         prm.accumulate = r.accumulate;
         uint32_t blocks = (s.num_workers + 15) / 16;
         if (blocks > 256) blocks = 256;
-        if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&hogwild_kernel<Rule>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)r.stats_lds),
+        if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&hogwild_kernel<Rule, HOT>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)r.stats_lds),
                                "hipFuncSetAttribute(MaxDynamicSharedMemorySize)")) return rc;
         set_lds_stats(prm, true);
-        hipLaunchKernelGGL((hogwild_kernel<Rule>), dim3(blocks), dim3(kMaxBlock), r.stats_lds, as_stream(stream), s, prm);
+        hipLaunchKernelGGL((hogwild_kernel<Rule, HOT>), dim3(blocks), dim3(kMaxBlock), r.stats_lds, as_stream(stream), s, prm);
         return launch_status(who);
     }
     // ordinary launches, cut into g_epoch_splits pieces on window boundaries
@@ -89,7 +97,7 @@ static int launch(const char* who, const Schedule& s0, const typename Rule::Para
         s.range_begin = b; s.range_end = e;
         prm.accumulate = r.accumulate || !first;
         first = false;
-        hipLaunchKernelGGL((hogwild_kernel<Rule>), dim3(grid_for(s.num_workers)), dim3(kBlock), lds, as_stream(stream), s, prm);
+        hipLaunchKernelGGL((hogwild_kernel<Rule, HOT>), dim3(grid_for(s.num_workers)), dim3(kBlock), lds, as_stream(stream), s, prm);
         if (int rc = launch_status(who)) return rc;
     }
     return MF_OK;

@@ -23,9 +23,11 @@ namespace mf {
 template <int K, bool COH, bool SAMPLED> struct MascotRuleT {
     static constexpr int E = K / 64;                        // elements per lane
     static constexpr int kAhead = 3, kRing = 8;
-    // chunk classes: 0 = any mix of precisions (flag-driven), 1 = every rating of the chunk touches two
-    // binary16 rows (the state every group starts in): loads and arithmetic without any branching
-    static constexpr int kClasses = 2;
+    // chunk classes: 1 = every rating of the chunk touches two binary16 rows (the state every group starts in): loads
+    // and arithmetic without any branching; 2 = any mix of precisions, every rating inside the group tables: every
+    // path through a rating issues the same number of memory instructions; 0 = anything, including ratings that are
+    // skipped (an index outside the tables)
+    static constexpr int kClasses = 3;
     using HV = typename std::conditional<E == 2, half2_t, half_t>::type;
 
     struct Params {
@@ -125,8 +127,10 @@ template <int K, bool COH, bool SAMPLED> struct MascotRuleT {
     }
     __device__ __forceinline__ int classify(const Prep& pr, bool valid) const
     {
-        return __builtin_amdgcn_ballot_w64(valid && (pr.flags & 7u) != 0u) == 0ull ? 1 : 0;
+        if (__builtin_amdgcn_ballot_w64(valid && (pr.flags & kSkip) != 0u) != 0ull) return 0;
+        return __builtin_amdgcn_ballot_w64(valid && (pr.flags & 3u) != 0u) == 0ull ? 1 : 2;
     }
+    static __device__ __forceinline__ Info no_row() { return Info{0.f, 0ull, 0ull, kSkip, 0u}; }      // forward() ignores skipped slots
     __device__ __forceinline__ Info info(const Rating& my, const Prep& pr, int j) const
     {
         Info i;
@@ -187,21 +191,20 @@ template <int K, bool COH, bool SAMPLED> struct MascotRuleT {
         } else {
 #pragma unroll
             for (int e = 0; e < E; ++e) { row.p[e] = 0; row.q[e] = 0; }
-            if (i.flags & kSkip) return;
+            if (CLS == 0 && (i.flags & kSkip)) return;
             load_side(row.p, i.pptr, i.flags & 1u, lane);
             load_side(row.q, i.qptr, i.flags & 2u, lane);
         }
     }
+    // selects, no branches: a branch here would sit between the row loads and their first use
     __device__ __forceinline__ void forward(Row& nxt, const Info& in, const Row& cur, const Info& ic) const
     {
-        if ((in.flags | ic.flags) & kSkip) return;
-        if (in.pptr == ic.pptr) {
+        const bool live = !((in.flags | ic.flags) & kSkip);
+        const bool same_p = live && in.pptr == ic.pptr, same_q = live && in.qptr == ic.qptr;
 #pragma unroll
-            for (int e = 0; e < E; ++e) nxt.p[e] = cur.p[e];
-        }
-        if (in.qptr == ic.qptr) {
-#pragma unroll
-            for (int e = 0; e < E; ++e) nxt.q[e] = cur.q[e];
+        for (int e = 0; e < E; ++e) {
+            nxt.p[e] = same_p ? cur.p[e] : nxt.p[e];
+            nxt.q[e] = same_q ? cur.q[e] : nxt.q[e];
         }
     }
 
@@ -277,7 +280,7 @@ template <int K, bool COH, bool SAMPLED> struct MascotRuleT {
     template <int CLS> __device__ __forceinline__ void update(Row& row, const Info& i, uint32_t processed) const
     {
         if (CLS == 0 && (i.flags & kSkip)) return;
-        const bool up = CLS == 0 && (i.flags & 1u), ip = CLS == 0 && (i.flags & 2u);
+        const bool up = CLS != 1 && (i.flags & 1u), ip = CLS != 1 && (i.flags & 2u);
         const bool sampled = SAMPLED && processed >= first_sample;
         const uint32_t ug = (i.flags >> 3) & 0x3fffu, ig = (i.flags >> 17) & 0x3fffu;
         if (!up && !ip) {

@@ -30,6 +30,7 @@ template <int K, bool COH> struct DenseBase {
 
     __device__ __forceinline__ Prep prepare(const Rating&, bool) const { return Prep(); }
     __device__ __forceinline__ int classify(const Prep&, bool) const { return 0; }
+    static __device__ __forceinline__ Info no_row() { return Info{0.f, 0xffffffffu, 0xffffffffu, 0u}; }   // matches no rating
     __device__ __forceinline__ Info info(const Rating& my, const Prep&, int j) const
     {
         Info i;
@@ -196,6 +197,7 @@ template <int K, bool COH> struct MemQuantRule {
     __device__ __forceinline__ void init(const Params& a, uint8_t*, int lane_, uint32_t) { P = a.p; Q = a.q; lrate = a.lrate; lambda = a.lambda; lane = lane_; }
     __device__ __forceinline__ Prep prepare(const Rating&, bool) const { return Prep(); }
     __device__ __forceinline__ int classify(const Prep&, bool) const { return 0; }
+    static __device__ __forceinline__ Info no_row() { return Info{0.f, 0xffffffffu, 0xffffffffu, 0u}; }
     __device__ __forceinline__ Info info(const Rating& my, const Prep&, int j) const
     {
         Info i;
