@@ -467,7 +467,7 @@ void orc_mpt_update(int k, float* p, float* q, float r, float lr, uint16_t scale
 void orc_mascot_update(int k, void* pv, int user_prec, void* qv, int item_prec, float r, float lr, float lambda,
                        float* grad_p, float* grad_q, float* norm_p, float* norm_q)
 {
-    float pf[128], qf[128], gp[128], gq[128];
+    float pf[128] = {0}, qf[128] = {0}, gp[128], gq[128];
     if (!user_prec && !item_prec) {
         uint16_t* p = (uint16_t*)pv; uint16_t* q = (uint16_t*)qv;
         float lr_h = rn16f(lr), lam_h = rn16f(lambda), r_h = rn16f(r);       /* :79-80,189 */

@@ -14,6 +14,11 @@
  *   - MuPPET / AFP: floor/ceil(log2f(x)) for x within one ulp of a power of
  *     two, and float -> int8 conversion of values outside [-128,127], depend on
  *     CUDA's libdevice / cvt behaviour.  parity unpinned for those inputs.
+ *   - orc_sgd_update / orc_mem_quant_update: binary32 arithmetic that nvcc may
+ *     contract into fma where the source writes a*b - c*d; this restatement
+ *     rounds every operation.  parity unpinned for that choice (the update is
+ *     pinned as a gradient step within binary32 rounding, the summation order
+ *     by a crafted row).
  */
 #ifndef MASCOT_ORACLE_H
 #define MASCOT_ORACLE_H
