@@ -422,7 +422,8 @@ def main():
     if not a.skip_cached:
         c = leg(False, a.cached_workers)
         out["cached_rows"] = {"note": "same workload with ordinary cached row accesses (each XCD trains its own L2-resident copy of hot "
-                                      "rows; faster, converges worse, see DESIGN.md)",
+                                      "rows; faster, converges worse, see DESIGN.md); its algorithmic bytes can exceed the HBM peak because "
+                                      "hot rows are served and overwritten in L2 without reaching memory",
                               "value": c["ratings_per_s"], "unit": "ratings/s", "ms_per_step": c["ms_per_step"], "workers": c["workers"],
                               "roofline": {"bound": "hbm", "achieved": c["gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": c["gbs"] / PEAK_HBM_GBS,
                                            "kernel": "hogwild_kernel<MascotRuleT<%d,false,false>>" % k},

@@ -117,12 +117,27 @@ __global__ __launch_bounds__(kMaxBlock) void hogwild_kernel(Schedule s, typename
     Rule rule;
     rule.init(prm, smem, lane, first_wid);              // may synchronise the workgroup
     // a launch normally has one wavefront per worker; a launch with fewer wavefronts (the sampled tail of
-    // a MASCOT epoch, which keeps per-workgroup statistics in LDS) lets each wavefront play several workers
-    for (uint32_t wid = first_wid; wid < s.num_workers && s.range_begin < s.range_end; wid += total_waves) {
-        // this worker handles ratings with processed index in [range_begin, range_end)
-        uint32_t processed = s.range_begin;
-        uint32_t ite = s.range_begin / s.update_vector_size;
-        uint32_t c = s.range_begin - ite * s.update_vector_size;
+    // a MASCOT epoch, which keeps per-workgroup statistics in LDS) lets each wavefront play several workers,
+    // and may cut every worker's range into s.pieces parts (on chunk boundaries) to even out the wavefronts' loads
+    const uint32_t pieces = s.pieces ? s.pieces : 1u;
+    for (uint32_t item = first_wid; item < s.num_workers * pieces && s.range_begin < s.range_end; item += total_waves) {
+        const uint32_t wid = item % s.num_workers, piece = item / s.num_workers;
+        // this wavefront handles the worker's ratings with processed index in [range_begin, range_end)
+        uint32_t range_begin = s.range_begin, range_end = s.range_end;
+        if (pieces > 1) {
+            auto cut = [&](uint32_t i) -> uint32_t {
+                if (i == 0) return s.range_begin;
+                if (i == pieces) return s.range_end;
+                const uint32_t at = s.range_begin + (uint32_t)((uint64_t)(s.range_end - s.range_begin) * i / pieces);
+                const uint32_t down = at - (at % s.update_vector_size) % (uint32_t)kWave;     // a chunk boundary of its window
+                return down > s.range_begin ? down : s.range_begin;
+            };
+            range_begin = cut(piece); range_end = cut(piece + 1);
+            if (range_begin >= range_end) continue;
+        }
+        uint32_t processed = range_begin;
+        uint32_t ite = range_begin / s.update_vector_size;
+        uint32_t c = range_begin - ite * s.update_vector_size;
         auto window_of = [&](uint32_t it) -> uint32_t {
             uint32_t st;
             if (s.window_start) st = s.window_start[(size_t)it * s.num_workers + wid] % s.nnz;
@@ -131,7 +146,7 @@ __global__ __launch_bounds__(kMaxBlock) void hogwild_kernel(Schedule s, typename
         };
         auto chunk_len = [&](uint32_t cc, uint32_t pp) -> int {
             uint32_t left = s.update_vector_size - cc;
-            if (left > s.range_end - pp) left = s.range_end - pp;
+            if (left > range_end - pp) left = range_end - pp;
             return left < (uint32_t)kWave ? (int)left : kWave;
         };
         auto fetch = [&](uint32_t st, uint32_t cc, int nn) -> Rating {
@@ -158,7 +173,7 @@ __global__ __launch_bounds__(kMaxBlock) void hogwild_kernel(Schedule s, typename
             // position of the chunk after this one, and its ratings, requested now
             uint32_t nprocessed = processed + (uint32_t)n;
             uint32_t nc = c + (uint32_t)n, nite = ite, nstart = start;
-            const bool more = nprocessed < s.range_end;
+            const bool more = nprocessed < range_end;
             int nn = 0;
             Rating nmy = {0.f, 0u, 0u, 0u};
             if (more) {

@@ -37,7 +37,7 @@ static Schedule make_schedule(const mf_node* R, uint32_t nnz, uint32_t num_worke
 {
     Schedule s;
     s.R = R; s.nnz = nnz; s.num_workers = num_workers; s.update_count = update_count;
-    s.update_vector_size = update_vector_size; s.range_begin = 0; s.range_end = update_count * update_vector_size; s.epoch_key = window_epoch_key(seed, epoch); s.window_start = window_start; s.keep_u = g_keep_u; s.keep_v = g_keep_v;
+    s.update_vector_size = update_vector_size; s.pieces = 1; s.range_begin = 0; s.range_end = update_count * update_vector_size; s.epoch_key = window_epoch_key(seed, epoch); s.window_start = window_start; s.keep_u = g_keep_u; s.keep_v = g_keep_v;
     return s;
 }
 static inline uint32_t grid_for(uint32_t num_workers) { return (num_workers + kWavesPerBlock - 1) / kWavesPerBlock; }
@@ -77,7 +77,16 @@ static int launch_hot(const char* who, const Schedule& s0, const typename Rule::
         s.range_begin = r.begin; s.range_end = r.end;
         prm.accumulate = r.accumulate;
         uint32_t blocks = (s.num_workers + 15) / 16;
-        if (blocks > 256) blocks = 256;
+        if (blocks > 256) {
+            // more workers than the 4096 wavefronts of this launch: cut each worker's range into the number of
+            // pieces that leaves the fewest idle wavefronts in the last pass
+            blocks = 256;
+            double best = 1e30;
+            for (uint32_t p = 1; p <= 4; ++p) {
+                const double passes = (double)(((uint64_t)s.num_workers * p + 4095) / 4096) / p;
+                if (passes < best - 1e-9) { best = passes; s.pieces = p; }
+            }
+        }
         if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&hogwild_kernel<Rule, HOT>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)r.stats_lds),
                                "hipFuncSetAttribute(MaxDynamicSharedMemorySize)")) return rc;
         set_lds_stats(prm, true);
@@ -276,7 +285,7 @@ int mf_mascot_sgd_hogwild(const mf_node* R, uint32_t nnz, void* const* p, void* 
         return launch_k_coh<MascotPlainRule>(who, k, s, fill, lds, stream, body);
     // A check epoch.  The sampled ratings [first_sample, total) run as their own launch with the gradient sums in
     // LDS when those fit (160 KB per workgroup); otherwise the whole epoch runs with the sums in global memory.
-    const size_t need = lds + (size_t)(user_group_num + item_group_num) * (size_t)k * sizeof(float);
+    const size_t need = lds + (size_t)(user_group_num + item_group_num) * ((size_t)k + 1) * sizeof(float);      // sums and one lock per group
     if (need > 160 * 1024) return launch_k_coh<MascotRule>(who, k, s, fill, lds, stream, body);
     body.end = first_sample_rating_idx;
     // the body still writes the (zero) norm sums of its workgroups, which the sampled launch then adds to

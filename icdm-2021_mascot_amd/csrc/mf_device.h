@@ -162,6 +162,8 @@ struct Schedule {
     uint32_t update_count;
     uint32_t update_vector_size;
     uint32_t range_begin, range_end;   // processed-index range [begin, end) every worker handles in this launch
+    uint32_t pieces;                   // >= 1: the range of a worker is cut into this many parts, each played by a
+                                       // wavefront of its own (only launches with fewer wavefronts than workers)
     uint64_t epoch_key;
     const uint32_t* window_start;   // optional [update_count][num_workers]
     // Hot rows (optional, both null = off).  keep_u[row] / keep_v[row] in 0..255; 255 = an ordinary row.

@@ -55,16 +55,16 @@ template <int K, bool COH, bool SAMPLED> struct MascotRuleT {
     uint8_t* uprec_s; uint8_t* iprec_s;
     float* grad_sum_p; float* grad_sum_q;
     float* ugrad_s; float* igrad_s;      // per-workgroup [groups][K] sums in LDS, or null
+    uint32_t* ulock_s; uint32_t* ilock_s; // with them: one lock per group (add_sums_locked)
     uint32_t first_sample, user_groups, item_groups;
     float lrate, lambda;
     int lane;
     // Sampled sums of the most popular group of each side (the last one; with Zipf-like data it takes half of all
-    // ratings) stay in registers and reach the shared sums once per wavefront: LDS float atomics are the bound of
-    // the sampled launch otherwise.
+    // ratings) stay in registers and reach the shared sums once per wavefront: one contended group lock less.
     mutable float top_gp[E], top_gq[E], top_np, top_nq;
 
     static __host__ __device__ size_t lds_bytes(uint32_t ug, uint32_t ig) { return ((size_t)(ug + ig) * (8 + 4 + 4 + 1) + 31) / 16 * 16; }
-    static size_t lds_stats_bytes(uint32_t ug, uint32_t ig) { return (size_t)(ug + ig) * K * sizeof(float); }
+    static size_t lds_stats_bytes(uint32_t ug, uint32_t ig) { return (size_t)(ug + ig) * (K + 1) * sizeof(float); }
 
     __device__ __forceinline__ void init(const Params& a, uint8_t* smem, int lane_, uint32_t)
     {
@@ -90,11 +90,13 @@ template <int K, bool COH, bool SAMPLED> struct MascotRuleT {
         first_sample = a.first_sample; lrate = a.lrate; lambda = a.lambda;
         for (int e = 0; e < E; ++e) { top_gp[e] = 0.f; top_gq[e] = 0.f; }
         top_np = 0.f; top_nq = 0.f;
-        ugrad_s = nullptr; igrad_s = nullptr;
+        ugrad_s = nullptr; igrad_s = nullptr; ulock_s = nullptr; ilock_s = nullptr;
         if (a.lds_stats) {
             ugrad_s = reinterpret_cast<float*>(smem + lds_bytes(user_groups, item_groups));
             igrad_s = ugrad_s + (size_t)user_groups * K;
-            for (uint32_t i = threadIdx.x; i < (user_groups + item_groups) * K; i += blockDim.x) ugrad_s[i] = 0.f;
+            ulock_s = reinterpret_cast<uint32_t*>(igrad_s + (size_t)item_groups * K);
+            ilock_s = ulock_s + user_groups;
+            for (uint32_t i = threadIdx.x; i < (user_groups + item_groups) * (K + 1); i += blockDim.x) ugrad_s[i] = 0.f;   // sums and locks
         }
         __syncthreads();
     }
@@ -248,17 +250,46 @@ template <int K, bool COH, bool SAMPLED> struct MascotRuleT {
     // sums or, without them, into the global sums.  The LDS accesses are spelled in the LDS address space: a
     // pointer that may be either would make them flat instructions, which wait for every outstanding row load.
     typedef __attribute__((address_space(3))) float lds_float;
+    typedef __attribute__((address_space(3))) uint32_t lds_u32;
     static __device__ __forceinline__ void lds_add(float* p, float v)
     {
         (void)__hip_atomic_fetch_add((lds_float*)p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     }
-    __device__ __forceinline__ void add_sums(const float* g, float n, uint32_t group, float* norm_s, float* grad_sum, float* grad_s) const
+    // Adds to a group's sums in LDS under the group's lock.  A 64-lane ds_add_f32 occupies the LDS of a gfx950 CU
+    // for about 190 clocks (a third of a lane per clock, measured), an integer exchange and ordinary reads and
+    // writes run at full rate: taking the lock, reading, adding in registers and writing back is ten times
+    // faster.  The LDS operations of one wavefront execute in program order, so the release (the last write) is
+    // seen after the sums; every access is volatile, which keeps the compiler to that order as well.  The holder
+    // releases after a fixed straight-line sequence, so every waiting wavefront gets the lock.
+    __device__ __forceinline__ void add_sums_locked(const float* g, float n, uint32_t group, float* norm_s, float* grad_s, uint32_t* lock_s) const
     {
-        if (lane == 0) lds_add(&norm_s[group], n);
-        if (grad_s) {      // LDS layout [group][e][lane]: consecutive lanes on consecutive banks
+        volatile lds_u32* lock = (volatile lds_u32*)(lock_s + group);
+        for (;;) {
+            uint32_t held = 1u;
+            if (lane == 0) held = __hip_atomic_exchange(lock, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            if (__builtin_amdgcn_readfirstlane(held) == 0u) break;
+            __builtin_amdgcn_s_sleep(1);
+        }
+        // LDS layout [group][e][lane]: consecutive lanes on consecutive banks
+        volatile lds_float* sums = (volatile lds_float*)(grad_s + (size_t)group * K + lane);
+        volatile lds_float* norm = (volatile lds_float*)(norm_s + group);
+        float have[E], have_n = 0.f;
 #pragma unroll
-            for (int e = 0; e < E; ++e) lds_add(grad_s + (size_t)group * K + e * kWave + lane, g[e]);
+        for (int e = 0; e < E; ++e) have[e] = sums[e * kWave];
+        if (lane == 0) have_n = *norm;
+#pragma unroll
+        for (int e = 0; e < E; ++e) sums[e * kWave] = have[e] + g[e];
+        if (lane == 0) {
+            *norm = have_n + n;
+            __hip_atomic_store(lock, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        }
+    }
+    __device__ __forceinline__ void add_sums(const float* g, float n, uint32_t group, float* norm_s, float* grad_sum, float* grad_s, uint32_t* lock_s) const
+    {
+        if (grad_s) {
+            add_sums_locked(g, n, group, norm_s, grad_s, lock_s);
         } else {
+            if (lane == 0) lds_add(&norm_s[group], n);
 #pragma unroll
             for (int e = 0; e < E; ++e) atomicAdd(grad_sum + (size_t)group * K + (size_t)lane * E + e, g[e]);
         }
@@ -270,10 +301,10 @@ template <int K, bool COH, bool SAMPLED> struct MascotRuleT {
         n = reduce_wave(n, OpAdd());
         if (user_side) {
             if (group == user_groups - 1) { for (int e = 0; e < E; ++e) top_gp[e] += g[e]; top_np += n; }
-            else add_sums(g, n, group, unorm_s, grad_sum_p, ugrad_s);
+            else add_sums(g, n, group, unorm_s, grad_sum_p, ugrad_s, ulock_s);
         } else {
             if (group == item_groups - 1) { for (int e = 0; e < E; ++e) top_gq[e] += g[e]; top_nq += n; }
-            else add_sums(g, n, group, inorm_s, grad_sum_q, igrad_s);
+            else add_sums(g, n, group, inorm_s, grad_sum_q, igrad_s, ilock_s);
         }
     }
 
@@ -356,8 +387,8 @@ template <int K, bool COH, bool SAMPLED> struct MascotRuleT {
     {
         if constexpr (SAMPLED) {
             const float np0 = bcast(top_np, 0), nq0 = bcast(top_nq, 0);
-            if (np0 != 0.f) add_sums(top_gp, np0, user_groups - 1, unorm_s, grad_sum_p, ugrad_s);
-            if (nq0 != 0.f) add_sums(top_gq, nq0, item_groups - 1, inorm_s, grad_sum_q, igrad_s);
+            if (np0 != 0.f) add_sums(top_gp, np0, user_groups - 1, unorm_s, grad_sum_p, ugrad_s, ulock_s);
+            if (nq0 != 0.f) add_sums(top_gq, nq0, item_groups - 1, inorm_s, grad_sum_q, igrad_s, ilock_s);
         }
         __syncthreads();
         // a launch that continues an epoch (accumulate) adds to what the earlier launches of the epoch left
