@@ -179,13 +179,15 @@ template <int K, bool COH> struct MptRule : DenseBase<K, COH> {
     __device__ __forceinline__ void finish(const Params&, uint32_t) const {}
 };
 
-// mem_quant_sgd_k128/k64_hogwild_kernel, sgd/sgd_kernel.h:81-164: dense binary16 P/Q, binary32 arithmetic.  Lane L holds
-// elements L and L+64 of a row (two coalesced 128-byte accesses), widened.  The reference's lane l sums its products
-// left to right, p1*q1 + p2*q2 + p3*q3 + p4*q4 over elements l, l+32, l+64, l+96: with a = m0[l], b = m0[l+32],
-// c = m1[l], d = m1[l+32] (l = L mod 32) that is ((a + b) + c) + d, formed identically in both half-waves.
+// mem_quant_sgd_k128/k64_hogwild_kernel, sgd/sgd_kernel.h:81-164: dense binary16 P/Q, binary32 arithmetic.
+// k = 64: lane L holds element L.  k = 128: lane L holds the pair of elements 2L, 2L+1 (one 4-byte access per lane and
+// side, as in the MASCOT kernel).  The reference's lane l sums its products left to right,
+// p1*q1 + p2*q2 + p3*q3 + p4*q4 over elements l, l+32, l+64, l+96, and then runs the 16,8,4,2,1 tree over l.  Element
+// l + 32j sits in row j of 16 lanes, position l/2, half l%2: the four rows are summed in order first, the tree's
+// steps 16,8,4,2 are rotations by 8,4,2,1 inside a row and its last step adds the two halves.
 template <int K, bool COH> struct MemQuantRule {
     static constexpr int E = K / 64;
-    using Row = DenseRow<K>;
+    struct Row { uint32_t p, q; };      // the binary16 values as loaded (a pair at k = 128): half the registers of widened rows
     using Info = DenseInfo;
     using Prep = NoPrep;
     static constexpr int kClasses = 1;
@@ -204,68 +206,82 @@ template <int K, bool COH> struct MemQuantRule {
         i.r = bcast(my.r, j); i.u = bcast(my.u, j); i.v = bcast(my.v, j); i.thin = bcast(my.thin, j);
         return i;
     }
+    __device__ __forceinline__ uint32_t load_side(const uint16_t* row) const
+    {
+        if constexpr (E == 2) return row_load(reinterpret_cast<const uint32_t*>(row) + lane);
+        else return (uint32_t)row_load(row + lane);
+    }
     template <int CLS> __device__ __forceinline__ void load(Row& row, const Info& i) const
     {
-        const uint16_t* pp = P + (size_t)i.u * K + lane;
-        const uint16_t* qq = Q + (size_t)i.v * K + lane;
-#pragma unroll
-        for (int e = 0; e < E; ++e) {
-            row.p[e] = (float)from_bits<half_t>((uint32_t)row_load(pp + 64 * e));
-            row.q[e] = (float)from_bits<half_t>((uint32_t)row_load(qq + 64 * e));
-        }
+        row.p = load_side(P + (size_t)i.u * K);
+        row.q = load_side(Q + (size_t)i.v * K);
     }
     __device__ __forceinline__ void forward(Row& nxt, const Info& in, const Row& cur, const Info& ic) const
     {
-        if (in.u == ic.u) {
-#pragma unroll
-            for (int e = 0; e < E; ++e) nxt.p[e] = cur.p[e];
-        }
-        if (in.v == ic.v) {
-#pragma unroll
-            for (int e = 0; e < E; ++e) nxt.q[e] = cur.q[e];
-        }
+        if (in.u == ic.u) nxt.p = cur.p;
+        if (in.v == ic.v) nxt.q = cur.q;
     }
-    // store the rounded row, or add the rounded change to a hot row: even lanes add the pair (own, right neighbour)
-    __device__ __forceinline__ void write_side(uint16_t* base, const float* now, const float* change, bool hot) const
+    static __device__ __forceinline__ void widen(float* f, uint32_t raw)
     {
-#pragma unroll
-        for (int e = 0; e < E; ++e) {
-            if (hot) {
-                const uint32_t mine = bits((half_t)change[e]);
+        if constexpr (E == 2) { const half2_t h = from_bits<half2_t>(raw); f[0] = (float)h.x; f[1] = (float)h.y; }
+        else f[0] = (float)from_bits<half_t>(raw);
+    }
+    static __device__ __forceinline__ uint32_t narrow(const float* f)
+    {
+        if constexpr (E == 2) { half2_t h; h.x = (half_t)f[0]; h.y = (half_t)f[1]; return bits(h); }
+        else return bits((half_t)f[0]);
+    }
+    // store the rounded row, or add the rounded change to a hot row
+    __device__ __forceinline__ void write_side(uint16_t* row, uint32_t now, const float* change, bool hot) const
+    {
+        if constexpr (E == 2) {
+            uint32_t* at = reinterpret_cast<uint32_t*>(row) + lane;
+            if (hot) row_add(reinterpret_cast<half2_t*>(at), from_bits<half2_t>(narrow(change)));
+            else row_store<COH>(at, now);
+        } else {
+            if (hot) {      // even lanes add the pair (own, right neighbour)
+                const uint32_t mine = narrow(change);
                 const uint32_t other = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)mine, 0xB1 /* quad_perm 1,0,3,2 */, 0xf, 0xf, false);
-                if (!(lane & 1)) row_add(reinterpret_cast<half2_t*>(base + 64 * e), from_bits<half2_t>(mine | (other << 16)));
+                if (!(lane & 1)) row_add(reinterpret_cast<half2_t*>(row + lane), from_bits<half2_t>(mine | (other << 16)));
             } else {
-                row_store<COH>(base + 64 * e, (uint16_t)bits((half_t)now[e]));
+                row_store<COH>(row + lane, (uint16_t)now);
             }
         }
     }
+    // ((row 0 + row 1) + row 2) + row 3 of the wavefront's four rows of 16 lanes, in every lane
+    static __device__ __forceinline__ float sum_rows_in_order(float x)
+    {
+        auto halves = __builtin_amdgcn_permlane32_swap(bits(x), bits(x), false, false);      // [0]: rows 0 1 0 1, [1]: rows 2 3 2 3
+        auto lo = __builtin_amdgcn_permlane16_swap(halves[0], halves[0], false, false);      // [0]: row 0 everywhere, [1]: row 1
+        auto hi = __builtin_amdgcn_permlane16_swap(halves[1], halves[1], false, false);      // [0]: row 2 everywhere, [1]: row 3
+        float s = from_bits<float>(lo[0]) + from_bits<float>(lo[1]);
+        s = s + from_bits<float>(hi[0]);
+        return s + from_bits<float>(hi[1]);
+    }
     template <int CLS> __device__ __forceinline__ void update(Row& row, const Info& i, uint32_t) const
     {
+        float pf[E], qf[E];
+        widen(pf, row.p); widen(qf, row.q);
         float dot;
         if constexpr (E == 1) {
-            dot = reduce_wave(row.p[0] * row.q[0], OpAdd());                // k = 64: p1*q1 + p2*q2, then the tree
+            dot = reduce_wave(pf[0] * qf[0], OpAdd());                // k = 64: p1*q1 + p2*q2, then the tree
         } else {
-            const float m0 = row.p[0] * row.q[0], m1 = row.p[1] * row.q[1];
-            const float o0 = lane_xor32(m0), o1 = lane_xor32(m1);
-            const bool upper = lane >= 32;
-            float s = m0 + o0;                                              // a + b
-            s = s + (upper ? o1 : m1);                                      // + c
-            s = s + (upper ? m1 : o1);                                      // + d
-            dot = reduce_half_wave(s, OpAdd());
+            const float even = reduce_row16(sum_rows_in_order(pf[0] * qf[0]), OpAdd());
+            const float odd = reduce_row16(sum_rows_in_order(pf[1] * qf[1]), OpAdd());
+            dot = even + odd;
         }
         const float ruv = i.r - dot;
-        float dp[E], dq[E];
+        float dp[E], dq[E], np[E], nq[E];
 #pragma unroll
         for (int e = 0; e < E; ++e) {
-            const float pe = row.p[e], qe = row.q[e];
-            dp[e] = lrate * (ruv * qe - lambda * pe);
-            dq[e] = lrate * (ruv * pe - lambda * qe);
-            // the register copy is what the row holds afterwards: the sum rounded to binary16
-            row.p[e] = (i.thin & 1u) ? pe : (float)(half_t)(pe + dp[e]);
-            row.q[e] = (i.thin & 2u) ? qe : (float)(half_t)(qe + dq[e]);
+            dp[e] = lrate * (ruv * qf[e] - lambda * pf[e]);
+            dq[e] = lrate * (ruv * pf[e] - lambda * qf[e]);
+            np[e] = pf[e] + dp[e];
+            nq[e] = qf[e] + dq[e];
         }
-        if (!(i.thin & 1u)) write_side(P + (size_t)i.u * K + lane, row.p, dp, i.thin & 4u);
-        if (!(i.thin & 2u)) write_side(Q + (size_t)i.v * K + lane, row.q, dq, i.thin & 8u);
+        // the register copy is what the row holds afterwards: the sum rounded to binary16
+        if (!(i.thin & 1u)) { row.p = narrow(np); write_side(P + (size_t)i.u * K, row.p, dp, i.thin & 4u); }
+        if (!(i.thin & 2u)) { row.q = narrow(nq); write_side(Q + (size_t)i.v * K, row.q, dq, i.thin & 8u); }
     }
     __device__ __forceinline__ void finish(const Params&, uint32_t) const {}
 };
