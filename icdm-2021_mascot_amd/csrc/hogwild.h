@@ -28,7 +28,7 @@ template <int I, int N, class F> __device__ __forceinline__ void static_for(F&& 
     }
 }
 
-template <class Rule, int CLS>
+template <class Rule, int CLS, bool HOT>
 __device__ __forceinline__ void process_chunk(Rule& rule, const Rating& my, const typename Rule::Prep& prep, int n, uint32_t processed)
 {
     constexpr int A = Rule::kAhead;
@@ -56,7 +56,7 @@ __device__ __forceinline__ void process_chunk(Rule& rule, const Rating& my, cons
                     constexpr int sh = (d - h + 2 * S) % S;
                     if (j >= h) rule.forward(ring[d], inf[d], ring[sh], inf[sh]);
                 });
-                rule.template update<CLS>(ring[d], inf[d], processed + (uint32_t)j);
+                rule.template update<CLS, HOT>(ring[d], inf[d], processed + (uint32_t)j);
             }
         });
     }
@@ -89,7 +89,7 @@ __device__ __forceinline__ void process_full_chunk(Rule& rule, const Rating& my,
             constexpr int sh = (d - h + 2 * S) % S;
             rule.forward(ring[d], inf[d], ring[sh], inf[sh]);
         });
-        rule.template update<CLS>(ring[d], inf[d], processed + (uint32_t)j);
+        rule.template update<CLS, HOT>(ring[d], inf[d], processed + (uint32_t)j);
     };
     static_for<0, A>([&](auto D) { fetch_rows(D, decltype(D)::value); });
     for (int j0 = 0; j0 < kWave - S; j0 += S) {
@@ -188,13 +188,13 @@ __global__ __launch_bounds__(kMaxBlock) void hogwild_kernel(Schedule s, typename
             // chunks of those run the straight-line pipeline, everything else the general one
             if (Rule::kClasses > 1 && cls == 1) {
                 if (n == kWave) process_full_chunk<Rule, 1, HOT>(rule, my, prep, processed);
-                else process_chunk<Rule, 1>(rule, my, prep, n, processed);
+                else process_chunk<Rule, 1, HOT>(rule, my, prep, n, processed);
             } else if (Rule::kClasses > 2 && cls == 2 && n == kWave) {
                 process_full_chunk<Rule, 2, HOT>(rule, my, prep, processed);
             } else if (Rule::kClasses == 1 && n == kWave) {
                 process_full_chunk<Rule, 0, HOT>(rule, my, prep, processed);
             } else {
-                process_chunk<Rule, 0>(rule, my, prep, n, processed);
+                process_chunk<Rule, 0, HOT>(rule, my, prep, n, processed);
             }
             if (!more) break;
             processed = nprocessed; c = nc; ite = nite; start = nstart; n = nn; my = nmy;

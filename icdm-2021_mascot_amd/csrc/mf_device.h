@@ -40,7 +40,8 @@ template <class T> __device__ __forceinline__ T lane_xor32(T x)
 // Value held by lane ((L + N) mod 16) of the same row of 16 lanes.
 template <int N, class T> __device__ __forceinline__ T row_ror(T x)
 {
-    return from_bits<T>((uint32_t)__builtin_amdgcn_update_dpp(0, (int)bits(x), 0x120 + N, 0xf, 0xf, false));
+    // every lane has a source lane, so no previous value is needed (mov_dpp leaves it undefined: no register to clear)
+    return from_bits<T>((uint32_t)__builtin_amdgcn_mov_dpp((int)bits(x), 0x120 + N, 0xf, 0xf, true));
 }
 
 // Reduction steps: every lane ends with op(own, partner); op must be commutative.
@@ -127,6 +128,31 @@ __device__ __forceinline__ void row_add(float* p, float d)
 __device__ __forceinline__ void row_add(half2_t* p, half2_t d)
 {
     (void)__builtin_amdgcn_global_atomic_fadd_v2f16(global_ptr(p), d);
+}
+
+// A row seen through a buffer resource of `bytes` bytes: accesses past the end are dropped by the hardware,
+// so a window of 0 bytes turns a store into a no-op without a branch.  The fp32 rules' kernels with hot-row
+// code store rows this way: the store of a rating that is thinned, or whose change is added instead, is still
+// issued (and dropped), every rating then issues the same number of memory instructions on the straight path
+// and the compiler's counted waits (s_waitcnt vmcnt(N)) keep the look-ahead of the row loads.
+typedef __amdgpu_buffer_rsrc_t row_window_t;
+__device__ __forceinline__ row_window_t row_window(uint64_t row, uint32_t bytes)
+{
+    return __builtin_amdgcn_make_buffer_rsrc((void*)row, 0, (int)bytes, 0x00020000 /* 32-bit data format, raw addressing */);
+}
+// COH: the sc1 cache policy of row_store's agent-scope stores
+template <bool COH> __device__ __forceinline__ void window_store(row_window_t w, uint32_t byte_offset, uint32_t v)
+{
+    __builtin_amdgcn_raw_buffer_store_b32(v, w, (int)byte_offset, 0, COH ? 16 : 0);
+}
+template <bool COH> __device__ __forceinline__ void window_store(row_window_t w, uint32_t byte_offset, uint16_t v)
+{
+    __builtin_amdgcn_raw_buffer_store_b16(v, w, (int)byte_offset, 0, COH ? 16 : 0);
+}
+template <bool COH> __device__ __forceinline__ void window_store(row_window_t w, uint32_t byte_offset, uint64_t v)
+{
+    typedef uint32_t uint2_t __attribute__((ext_vector_type(2)));
+    __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(uint2_t, v), w, (int)byte_offset, 0, COH ? 16 : 0);
 }
 
 // ---- counter-based generator -----------------------------------------------------------

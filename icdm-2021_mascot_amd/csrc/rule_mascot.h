@@ -121,8 +121,9 @@ template <int K, bool COH, bool SAMPLED> struct MascotRuleT {
             const uint32_t urow = ug ? my.u - uend_s[ug - 1] - 1 : my.u;
             const uint32_t irow = ig ? my.v - iend_s[ig - 1] - 1 : my.v;
             const uint32_t up = uprec_s[ug] ? 1u : 0u, ip = iprec_s[ig] ? 1u : 0u;
-            pr.pptr = pptr_s[ug] + (uint64_t)urow * (K * (up ? 4u : 2u));
-            pr.qptr = qptr_s[ig] + (uint64_t)irow * (K * (ip ? 4u : 2u));
+            // a rating that is skipped carries null pointers: forward() then matches it with no row
+            pr.pptr = ok ? pptr_s[ug] + (uint64_t)urow * (K * (up ? 4u : 2u)) : 0ull;
+            pr.qptr = ok ? qptr_s[ig] + (uint64_t)irow * (K * (ip ? 4u : 2u)) : 0ull;
             pr.flags = up | (ip << 1) | (ok ? 0u : kSkip) | (ug << 3) | (ig << 17);
         }
         return pr;
@@ -132,7 +133,7 @@ template <int K, bool COH, bool SAMPLED> struct MascotRuleT {
         if (__builtin_amdgcn_ballot_w64(valid && (pr.flags & kSkip) != 0u) != 0ull) return 0;
         return __builtin_amdgcn_ballot_w64(valid && (pr.flags & 3u) != 0u) == 0ull ? 1 : 2;
     }
-    static __device__ __forceinline__ Info no_row() { return Info{0.f, 0ull, 0ull, kSkip, 0u}; }      // forward() ignores skipped slots
+    static __device__ __forceinline__ Info no_row() { return Info{0.f, 0ull, 0ull, kSkip, 0u}; }      // null pointers: forward() matches no row
     __device__ __forceinline__ Info info(const Rating& my, const Prep& pr, int j) const
     {
         Info i;
@@ -148,41 +149,41 @@ template <int K, bool COH, bool SAMPLED> struct MascotRuleT {
     {
         if (fp32) {
             if constexpr (E == 2) {
-                const uint64_t v = row_load(reinterpret_cast<const uint64_t*>(ptr + (uint64_t)lane * 8));
+                const uint64_t v = row_load((reinterpret_cast<const uint64_t*>(ptr) + lane));
                 r[0] = (uint32_t)v; r[1] = (uint32_t)(v >> 32);
             } else {
-                r[0] = row_load(reinterpret_cast<const uint32_t*>(ptr + (uint64_t)lane * 4));
+                r[0] = row_load((reinterpret_cast<const uint32_t*>(ptr) + lane));
             }
         } else {
-            if constexpr (E == 2) r[0] = row_load(reinterpret_cast<const uint32_t*>(ptr + (uint64_t)lane * 4));
-            else r[0] = row_load(reinterpret_cast<const uint16_t*>(ptr + (uint64_t)lane * 2));
+            if constexpr (E == 2) r[0] = row_load((reinterpret_cast<const uint32_t*>(ptr) + lane));
+            else r[0] = row_load((reinterpret_cast<const uint16_t*>(ptr) + lane));
         }
     }
     // hot row (Schedule::keep_u): add the change of this lane's elements to the row in memory
     static __device__ __forceinline__ void add_side_half(uint64_t ptr, HV d, int lane)
     {
         if constexpr (E == 2) {
-            row_add(reinterpret_cast<half2_t*>(ptr + (uint64_t)lane * 4), d);
+            row_add((reinterpret_cast<half2_t*>(ptr) + lane), d);
         } else {
             // one element per lane: even lanes add the pair (own, right neighbour)
             const uint32_t mine = (uint32_t)bits(d);
             const uint32_t other = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)mine, 0xB1 /* quad_perm 1,0,3,2 */, 0xf, 0xf, false);
-            if (!(lane & 1)) row_add(reinterpret_cast<half2_t*>(ptr + (uint64_t)lane * 2), from_bits<half2_t>(mine | (other << 16)));
+            if (!(lane & 1)) row_add(reinterpret_cast<half2_t*>(reinterpret_cast<uint16_t*>(ptr) + lane), from_bits<half2_t>(mine | (other << 16)));
         }
     }
     static __device__ __forceinline__ void add_side_float(uint64_t ptr, const float* d, int lane)
     {
 #pragma unroll
-        for (int e = 0; e < E; ++e) row_add(reinterpret_cast<float*>(ptr + (uint64_t)lane * (4 * E)) + e, d[e]);
+        for (int e = 0; e < E; ++e) row_add((reinterpret_cast<float*>(ptr) + lane * E + e), d[e]);
     }
     static __device__ __forceinline__ void store_side(const uint32_t* r, uint64_t ptr, bool fp32, int lane)
     {
         if (fp32) {
-            if constexpr (E == 2) row_store<COH>(reinterpret_cast<uint64_t*>(ptr + (uint64_t)lane * 8), (uint64_t)r[0] | ((uint64_t)r[1] << 32));
-            else row_store<COH>(reinterpret_cast<uint32_t*>(ptr + (uint64_t)lane * 4), r[0]);
+            if constexpr (E == 2) row_store<COH>((reinterpret_cast<uint64_t*>(ptr) + lane), (uint64_t)r[0] | ((uint64_t)r[1] << 32));
+            else row_store<COH>((reinterpret_cast<uint32_t*>(ptr) + lane), r[0]);
         } else {
-            if constexpr (E == 2) row_store<COH>(reinterpret_cast<uint32_t*>(ptr + (uint64_t)lane * 4), r[0]);
-            else row_store<COH>(reinterpret_cast<uint16_t*>(ptr + (uint64_t)lane * 2), (uint16_t)r[0]);
+            if constexpr (E == 2) row_store<COH>((reinterpret_cast<uint32_t*>(ptr) + lane), r[0]);
+            else row_store<COH>((reinterpret_cast<uint16_t*>(ptr) + lane), (uint16_t)r[0]);
         }
     }
     template <int CLS> __device__ __forceinline__ void load(Row& row, const Info& i) const
@@ -201,8 +202,8 @@ template <int K, bool COH, bool SAMPLED> struct MascotRuleT {
     // selects, no branches: a branch here would sit between the row loads and their first use
     __device__ __forceinline__ void forward(Row& nxt, const Info& in, const Row& cur, const Info& ic) const
     {
-        const bool live = !((in.flags | ic.flags) & kSkip);
-        const bool same_p = live && in.pptr == ic.pptr, same_q = live && in.qptr == ic.qptr;
+        // skipped ratings and empty slots have null pointers; copies between two of those are never used
+        const bool same_p = in.pptr == ic.pptr, same_q = in.qptr == ic.qptr;
 #pragma unroll
         for (int e = 0; e < E; ++e) {
             nxt.p[e] = same_p ? cur.p[e] : nxt.p[e];
@@ -308,7 +309,7 @@ template <int K, bool COH, bool SAMPLED> struct MascotRuleT {
         }
     }
 
-    template <int CLS> __device__ __forceinline__ void update(Row& row, const Info& i, uint32_t processed) const
+    template <int CLS, bool HOT> __device__ __forceinline__ void update(Row& row, const Info& i, uint32_t processed) const
     {
         if (CLS == 0 && (i.flags & kSkip)) return;
         const bool up = CLS != 1 && (i.flags & 1u), ip = CLS != 1 && (i.flags & 2u);

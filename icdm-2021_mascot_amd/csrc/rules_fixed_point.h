@@ -100,7 +100,7 @@ template <int K, bool COH> struct MuppetRule : DenseBase<K, COH> {
         if constexpr (E == 2) { const float b = step_xor32(sq[1], OpAdd()); a = a + b; }
         return a;
     }
-    template <int CLS> __device__ __forceinline__ void update(Row& row, const Info& i, uint32_t processed)
+    template <int CLS, bool HOT> __device__ __forceinline__ void update(Row& row, const Info& i, uint32_t processed)
     {
         const float* p = row.p; const float* q = row.q;
         float p_min = 0, p_max = 0, q_min = 0, q_max = 0, sp = 0, sq = 0, pred;
@@ -275,7 +275,7 @@ template <int K, bool COH> struct AfpRule : DenseBase<K, COH> {
         q.r = ufirst(q.r); q.n = ufirst(q.n); q.itv = ufirst(q.itv); q.mov_avg_range = ufirst(q.mov_avg_range);
         return q;
     }
-    template <int CLS> __device__ __forceinline__ void update(Row& row, const Info& i, uint32_t)
+    template <int CLS, bool HOT> __device__ __forceinline__ void update(Row& row, const Info& i, uint32_t)
     {
         const float* p = row.p; const float* q = row.q;
         float p_abs = fabsf(p[0]), q_abs = fabsf(q[0]);
