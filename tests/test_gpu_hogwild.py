@@ -107,7 +107,7 @@ def test_afp_bit_exact(orc, k, afp_epoch):
     assert np.array_equal(gq.view(np.uint32), Q.view(np.uint32))
 
 
-def _mascot_case(orc, k, W, uc, window, user_groups, item_groups, prec_mode, first_sample, seed):
+def _mascot_case(orc, k, W, uc, window, user_groups, item_groups, prec_mode, first_sample, seed, lr=LR):
     import torch
     h = mfutil.hip()
     R, starts, P, Q = mfutil.conflict_free_problem(seed, k, W, uc, window)
@@ -128,7 +128,7 @@ def _mascot_case(orc, k, W, uc, window, user_groups, item_groups, prec_mode, fir
     d_gsq = torch.zeros(item_groups * k, dtype=torch.float32, device="cuda")
     d_nsp = torch.full((user_groups * nb,), -3.0, dtype=torch.float32, device="cuda")
     d_nsq = torch.full((item_groups * nb,), -3.0, dtype=torch.float32, device="cuda")
-    h.mf_mascot_sgd_hogwild(dR.data_ptr(), R.size, dp.ptrs.data_ptr(), dq.ptrs.data_ptr(), k, W, uc, window, LR, LAM,
+    h.mf_mascot_sgd_hogwild(dR.data_ptr(), R.size, dp.ptrs.data_ptr(), dq.ptrs.data_ptr(), k, W, uc, window, lr, LAM,
                             dp.end.data_ptr(), dq.end.data_ptr(), dp.prec.data_ptr(), dq.prec.data_ptr(),
                             d_gsp.data_ptr(), d_gsq.data_ptr(), d_nsp.data_ptr(), d_nsq.data_ptr(),
                             first_sample, user_groups, item_groups, 0, 0, dS.data_ptr(), mfutil.stream_ptr())
@@ -136,7 +136,7 @@ def _mascot_case(orc, k, W, uc, window, user_groups, item_groups, prec_mode, fir
     gsp, gsq = np.zeros(user_groups * k, np.float32), np.zeros(item_groups * k, np.float32)
     nsp, nsq = np.zeros(user_groups, np.float32), np.zeros(item_groups, np.float32)
     orc.lib.orc_mascot_epoch(k, R.ctypes.data, R.size, gmp.ptrs, gmq.ptrs, gmp.end_idx.ctypes.data, gmq.end_idx.ctypes.data,
-                             gmp.prec.ctypes.data, gmq.prec.ctypes.data, user_groups, item_groups, W, uc, window, LR, LAM,
+                             gmp.prec.ctypes.data, gmq.prec.ctypes.data, user_groups, item_groups, W, uc, window, lr, LAM,
                              first_sample, gsp.ctypes.data, gsq.ctypes.data, nsp.ctypes.data, nsq.ctypes.data,
                              0, 0, starts.ctypes.data, 1)
     for got, want in zip(dp.download() + dq.download(), gmp.arrays + gmq.arrays):
@@ -161,6 +161,16 @@ def test_mascot_bit_exact(orc, k, prec_mode):
         assert nsp.sum() > 0 and nsq.sum() > 0
     if prec_mode == "float":
         assert nsp.sum() == 0 and nsq.sum() == 0
+
+
+@pytest.mark.parametrize("k", [64, 128])
+def test_mascot_sampled_ranges_in_pieces(orc, k):
+    """More workers than the sampled launch has wavefronts (4096): every worker's sampled range is cut into pieces
+    that different wavefronts play.  With a learning rate of 0 the model does not move, so the pieces may run in
+    any order and the sums must still hold every sampled rating exactly once."""
+    W, uc, window = 4100, 2, 192
+    nsp, nsq = _mascot_case(orc, k, W, uc, window, 9, 6, "half", first_sample=100, seed=90 + k, lr=0.0)
+    assert nsp.sum() > 0 and nsq.sum() > 0
 
 
 @pytest.mark.parametrize("k", [64, 128])
