@@ -14,25 +14,23 @@
 
 namespace mf {
 
+// Saturating conversions (CUDA's float-to-integer casts saturate and map NaN to 0).  Written without branches:
+// the value is clamped first, so the conversion itself is always in range, and selects pick the special cases;
+// nested ifs became nested exec-mask regions, a dozen scalar instructions per converted element.
 __device__ __forceinline__ uint32_t f2u_sat(float f)
 {
-    if (!(f > 0.0f)) return 0u;
-    if (f >= 4294967296.0f) return 0xffffffffu;
-    return (uint32_t)f;
+    const uint32_t r = (uint32_t)__builtin_amdgcn_fmed3f(f, 0.0f, 4294967040.0f);
+    return (f > 0.0f) ? (f >= 4294967296.0f ? 0xffffffffu : r) : 0u;
 }
 __device__ __forceinline__ int f2i_sat(float f)
 {
-    if (f != f) return 0;
-    if (f >= 2147483648.0f) return 2147483647;
-    if (f <= -2147483648.0f) return (int)0x80000000;
-    return (int)f;
+    const int r = (int)__builtin_amdgcn_fmed3f(f, -2147483648.0f, 2147483520.0f);
+    return (f != f) ? 0 : (f >= 2147483648.0f ? 2147483647 : r);
 }
 __device__ __forceinline__ int f2i8_sat(float f)
 {
-    if (f != f) return 0;
-    if (f > 127.0f) return 127;
-    if (f < -128.0f) return -128;
-    return (int)f;
+    const int r = (int)__builtin_amdgcn_fmed3f(f, -128.0f, 127.0f);
+    return (f != f) ? 0 : r;
 }
 // 2^n for an integer-valued exponent, exact (exp2f of an integer in the reference).
 __device__ __forceinline__ float pow2u(uint32_t n) { return __builtin_ldexpf(1.0f, n > 1000u ? 1000 : (int)n); }
@@ -68,6 +66,42 @@ __device__ __forceinline__ uint32_t muppet_scale_index(unsigned bitwidth, float 
     return f2u_sat(floorf(__builtin_log2f(range_best)));
 }
 __device__ __forceinline__ half_t grid_h(float v, float s, float s_rev) { return (half_t)(roundf(v * s) * s_rev); }
+// 1 / 2^n as the reference's division yields it: 2^n is infinite from n = 128 on, and 1 / inf = 0
+__device__ __forceinline__ float pow2_reciprocal(uint32_t n) { return n > 127u ? 0.0f : __builtin_ldexpf(1.0f, -(int)n); }
+// x / 2^n, likewise: scaling by a power of two is exact (and rounds like the division where the result is subnormal)
+__device__ __forceinline__ float div_pow2(float x, uint32_t n) { return n > 127u ? x * 0.0f : __builtin_ldexpf(x, -(int)n); }
+
+// IEEE 754-2019 maximum: equal to fmaxf for numbers, and one v_maximum3_f32 on gfx950 where fmaxf first
+// canonicalises both operands (three instructions after every cross-lane move)
+struct OpMaximum { __device__ __forceinline__ float operator()(float a, float b) const { return __builtin_elementwise_maximum(a, b); } };
+struct OpMinimum { __device__ __forceinline__ float operator()(float a, float b) const { return __builtin_elementwise_minimum(a, b); } };
+
+// Four wave-wide maxima in one reduction.  In: every lane's own a, b, c, d.  Out: the maximum over all lanes of a in
+// rows 0 (lanes 0-15), of c in row 1, of b in row 2 and of d in row 3.  v_permlane32_swap(a, b) leaves [a.lower, b.lower]
+// and [a.upper, b.upper], whose maximum folds the half-waves of a into the lower half and those of b into the upper
+// half; v_permlane16_swap folds the rows the same way; four rotations finish inside the rows.
+__device__ __forceinline__ float max4_by_rows(float a, float b, float c, float d)
+{
+    auto ab = __builtin_amdgcn_permlane32_swap(bits(a), bits(b), false, false);
+    auto cd = __builtin_amdgcn_permlane32_swap(bits(c), bits(d), false, false);
+    const float x = OpMaximum()(from_bits<float>(ab[0]), from_bits<float>(ab[1]));      // rows 0,1: a   rows 2,3: b
+    const float y = OpMaximum()(from_bits<float>(cd[0]), from_bits<float>(cd[1]));      // rows 0,1: c   rows 2,3: d
+    auto xy = __builtin_amdgcn_permlane16_swap(bits(x), bits(y), false, false);          // [x.r0 y.r0 x.r2 y.r2], [x.r1 y.r1 x.r3 y.r3]
+    const float z = OpMaximum()(from_bits<float>(xy[0]), from_bits<float>(xy[1]));
+    return reduce_row16(z, OpMaximum());
+}
+// get_only_scaling_factor (muppet_sgd_kernel.h:7-18) for two value ranges at once.  `extreme` holds, by half-wave, the
+// largest value (lower) and the negated smallest value (upper) of a range, the same in both rows of a half-wave or a
+// different range in each; the result is the scale index of the lane's range.
+__device__ __forceinline__ uint32_t muppet_scale_index_by_rows(unsigned bitwidth, float extreme, bool upper)
+{
+    const float val = (float)(1 << (bitwidth - 1));
+    const float bound = upper ? (-val) - 0.5f : (val - 1) + 0.5f;
+    const float ratio = fabsf(bound / extreme);                                        // |min_val / min| = |min_val / -min|
+    const float range_best = step_xor32(ratio, OpMinimum());
+    const bool both_zero = step_xor32(fabsf(extreme), OpMaximum()) == 0.0f;
+    return both_zero ? 0u : f2u_sat(floorf(__builtin_log2f(range_best)));
+}
 
 template <int K, bool COH> struct MuppetRule : DenseBase<K, COH> {
     using Base = DenseBase<K, COH>;
@@ -103,31 +137,34 @@ template <int K, bool COH> struct MuppetRule : DenseBase<K, COH> {
     template <int CLS, bool HOT> __device__ __forceinline__ void update(Row& row, const Info& i, uint32_t processed)
     {
         const float* p = row.p; const float* q = row.q;
-        float p_min = 0, p_max = 0, q_min = 0, q_max = 0, sp = 0, sq = 0, pred;
+        const bool upper = this->lane >= 32;
+        // extrema by rows of 16 lanes: max p, max q, -min p, -min q (all 0 when the forward pass is binary32, as in the reference)
+        float extrema = 0, sp = 0, sq = 0, pred;
+        uint32_t ip = 0, iq = 0;
         if (fwd != 32) {
-            p_min = p_max = p[0]; q_min = q_max = q[0];
+            float a = p[0], b = -p[0], c = q[0], d = -q[0];
             if constexpr (E == 2) {
-                p_min = fminf(p_min, p[1]); p_max = fmaxf(p_max, p[1]);
-                q_min = fminf(q_min, q[1]); q_max = fmaxf(q_max, q[1]);
+                a = OpMaximum()(a, p[1]); b = OpMaximum()(b, -p[1]);
+                c = OpMaximum()(c, q[1]); d = OpMaximum()(d, -q[1]);
             }
-            p_min = reduce_wave(p_min, OpMin()); q_min = reduce_wave(q_min, OpMin());
-            p_max = reduce_wave(p_max, OpMax()); q_max = reduce_wave(q_max, OpMax());
-            sp = pow2u(muppet_scale_index((unsigned)fwd, p_max, p_min));
-            sq = pow2u(muppet_scale_index((unsigned)fwd, q_max, q_min));
+            extrema = max4_by_rows(a, b, c, d);
+            const uint32_t idx = muppet_scale_index_by_rows((unsigned)fwd, extrema, upper);      // rows 0,2: p   rows 1,3: q
+            ip = bcast(idx, 0); iq = bcast(idx, 16);
+            sp = pow2u(ip); sq = pow2u(iq);
         }
         if (fwd == 8) {
             int acc = 0;
 #pragma unroll
             for (int e = 0; e < E; ++e) acc += f2i8_sat(roundf(p[e] * sp)) * f2i8_sat(roundf(q[e] * sq));
             acc = reduce_wave(acc, OpAdd());
-            pred = acc / (sp * sq);
+            pred = div_pow2((float)acc, ip + iq);                        // acc / (sp * sq)
         } else if (fwd == 32) {
             float m[E];
 #pragma unroll
             for (int e = 0; e < E; ++e) m[e] = p[e] * q[e];
             pred = dot_reference_order<E, float>(m);
         } else {
-            const float sp_rev = 1 / sp, sq_rev = 1 / sq;
+            const float sp_rev = pow2_reciprocal(ip), sq_rev = pow2_reciprocal(iq);
             // the reference's half2 lanes: .x sums elements l, l+64 (lower half-wave here), .y elements l+32, l+96 (upper)
             half_t t = grid_h(p[0], sp, sp_rev) * grid_h(q[0], sq, sq_rev);
             if constexpr (E == 2) t = t + grid_h(p[1], sp, sp_rev) * grid_h(q[1], sq, sq_rev);
@@ -136,15 +173,18 @@ template <int K, bool COH> struct MuppetRule : DenseBase<K, COH> {
         }
         const float ruv = i.r - pred;
         float sb = 0;
+        uint32_t ib = 0;
         if (bwd != 32) {
+            // max(p_max, q_max, -lambda, ruv) in the lower half-wave, -min(p_min, q_min, -lambda, ruv) in the upper one
             const float neg_lambda = -1 * lambda;
-            const float bmin = fminf(fminf(p_min, q_min), fminf(neg_lambda, ruv));
-            const float bmax = fmaxf(fmaxf(p_max, q_max), fmaxf(neg_lambda, ruv));
-            sb = pow2u(muppet_scale_index((unsigned)bwd, bmax, bmin));
+            const float pq = step_xor16(extrema, OpMaximum());
+            const float lr_ = upper ? OpMaximum()(-neg_lambda, -ruv) : OpMaximum()(neg_lambda, ruv);
+            ib = bcast(muppet_scale_index_by_rows((unsigned)bwd, OpMaximum()(pq, lr_), upper), 0);
+            sb = pow2u(ib);
         }
         float gp[E], gq[E];
         if (bwd == 8) {
-            const float sq_rev = 1 / (sb * sb);
+            const float sq_rev = pow2_reciprocal(2u * ib);
             const int ruv_i = f2i8_sat(roundf(ruv * sb));
             const int lam_i = f2i8_sat(roundf(-1.0f * lambda * sb));
 #pragma unroll
@@ -160,7 +200,7 @@ template <int K, bool COH> struct MuppetRule : DenseBase<K, COH> {
                 gq[e] = ruv * p[e] - lambda * q[e];
             }
         } else {
-            const float sb_rev = 1 / sb;
+            const float sb_rev = pow2_reciprocal(ib);
             const half_t t_ruv = grid_h(ruv, sb, sb_rev), t_lam = grid_h(-1 * lambda, sb, sb_rev);
 #pragma unroll
             for (int e = 0; e < E; ++e) {
