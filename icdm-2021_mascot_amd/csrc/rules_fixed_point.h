@@ -109,6 +109,10 @@ template <int K, bool COH> struct MuppetRule : DenseBase<K, COH> {
     using typename Base::Info;
     static constexpr int E = Base::E;
     static constexpr int J = K / 32;
+    // One rating of look-ahead: every race on a row is resolved last-writer-wins here (the plain store() below), and
+    // each further rating a wavefront has in flight loses more updates of the popular rows.  Measured at 100M
+    // ratings: three ratings ahead leave MuPPET's epoch unchanged (bound by its arithmetic), make AFP's 11 % shorter
+    // and cost both 0.006 to 0.015 of test RMSE after four epochs.
     static constexpr int kAhead = 1, kRing = 4;
     struct Params {
         float* p; float* q; float lrate; float lambda; uint32_t first_sample;
@@ -319,12 +323,12 @@ template <int K, bool COH> struct AfpRule : DenseBase<K, COH> {
     {
         const float* p = row.p; const float* q = row.q;
         float p_abs = fabsf(p[0]), q_abs = fabsf(q[0]);
-        if constexpr (E == 2) { p_abs = fmaxf(p_abs, fabsf(p[1])); q_abs = fmaxf(q_abs, fabsf(q[1])); }
+        if constexpr (E == 2) { p_abs = OpMaximum()(p_abs, fabsf(p[1])); q_abs = OpMaximum()(q_abs, fabsf(q[1])); }
         // the three re-measurements below happen every itv-th update of the worker; they sum their error terms per
         // lane from left to right over all four values, so they work on the 32-lane view
         if (cur_iter == upd_u) {
             Mirror<K> pm; pm.build(row.p, upper);
-            const float mx = reduce_wave(p_abs, OpMax());
+            const float mx = reduce_wave(p_abs, OpMaximum());
             const float diff = qem(pm.v, mx);
             if (cur_iter == 0) uq.mov_avg_range = mx;
             uq = uniform(afp_qpa(diff, mx, uq.mov_avg_range));
@@ -334,7 +338,7 @@ template <int K, bool COH> struct AfpRule : DenseBase<K, COH> {
         }
         if (cur_iter == upd_i) {
             Mirror<K> qm; qm.build(row.q, upper);
-            const float mx = reduce_wave(q_abs, OpMax());
+            const float mx = reduce_wave(q_abs, OpMaximum());
             const float diff = qem(qm.v, mx);
             if (cur_iter == 0) iq.mov_avg_range = mx;
             iq = uniform(afp_qpa(diff, mx, iq.mov_avg_range));
@@ -348,9 +352,9 @@ template <int K, bool COH> struct AfpRule : DenseBase<K, COH> {
 #pragma unroll
             for (int e = 0; e < E; ++e) acc += afp_sat8(roundf(p[e] * sp)) * afp_sat8(roundf(q[e] * sq));
             acc = reduce_wave(acc, OpAdd());
-            pred = acc / (sp * sq);
+            pred = div_pow2((float)acc, (uint32_t)uq.r + (uint32_t)iq.r);            // acc / (sp * sq); r >= 0
         } else {
-            const float sp_rev = 1 / sp, sq_rev = 1 / sq;
+            const float sp_rev = pow2_reciprocal((uint32_t)uq.r), sq_rev = pow2_reciprocal((uint32_t)iq.r);
             // the reference's half2 lanes: .x sums elements l, l+64 (lower half-wave here), .y elements l+32, l+96 (upper)
             half_t t = (half_t)afp_grid(p[0], sp, sp_rev) * (half_t)afp_grid(q[0], sq, sq_rev);
             if constexpr (E == 2) t = t + (half_t)afp_grid(p[1], sp, sp_rev) * (half_t)afp_grid(q[1], sq, sq_rev);
@@ -360,9 +364,9 @@ template <int K, bool COH> struct AfpRule : DenseBase<K, COH> {
         const float ruv = i.r - pred;
         if (cur_iter == upd_b) {
             Mirror<K> pm, qm; pm.build(row.p, upper); qm.build(row.q, upper);
-            float mx = fmaxf(p_abs, q_abs);
-            mx = fmaxf(fmaxf(mx, fabsf(lambda)), fabsf(ruv));
-            mx = reduce_wave(mx, OpMax());
+            float mx = OpMaximum()(p_abs, q_abs);
+            mx = OpMaximum()(OpMaximum()(mx, fabsf(lambda)), fabsf(ruv));
+            mx = reduce_wave(mx, OpMaximum());
             const float diff = qem_bp(pm.v, qm.v, ruv, mx);
             if (cur_iter == 0) bq.mov_avg_range = mx;
             bq = uniform(afp_qpa(diff, mx, bq.mov_avg_range));
@@ -374,7 +378,7 @@ template <int K, bool COH> struct AfpRule : DenseBase<K, COH> {
         if (bq.n == 8) {
             const int lam_i = afp_sat8(roundf(-1.0f * lambda * sb));
             const int ruv_i = afp_sat8(roundf(ruv * sb));
-            const float sq_rev = 1 / (sb * sb);
+            const float sq_rev = pow2_reciprocal(2u * (uint32_t)bq.r);
 #pragma unroll
             for (int e = 0; e < E; ++e) {
                 const int pi = afp_sat8(roundf(p[e] * sb)), qi = afp_sat8(roundf(q[e] * sb));
@@ -382,7 +386,7 @@ template <int K, bool COH> struct AfpRule : DenseBase<K, COH> {
                 gq[e] = (float)(pi * ruv_i + qi * lam_i) * sq_rev;
             }
         } else {
-            const float sb_rev = 1 / sb;
+            const float sb_rev = pow2_reciprocal((uint32_t)bq.r);
             const half_t t_ruv = (half_t)afp_grid(ruv, sb, sb_rev), t_lam = (half_t)afp_grid(-1.0f * lambda, sb, sb_rev);
 #pragma unroll
             for (int e = 0; e < E; ++e) {
