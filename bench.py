@@ -234,6 +234,25 @@ def time_steps(torch, prob, W, warmup, steps, cfg, seed):
     return per, wall, uc, float(np.mean(kept))
 
 
+def access_pattern_ceiling(torch, h, prob, W, tables, coherent, seed, reps=3):
+    """Time of mf_row_traffic_probe on the same ratings, hot-row tables and store policy: the epoch's memory traffic
+    without the arithmetic (all rows binary16, as in the timed epochs)."""
+    dev = prob.R.device
+    n = prob.R.shape[0]
+    P = torch.zeros(prob.n_users * prob.k, dtype=torch.float16, device=dev)
+    Q = torch.zeros(prob.n_items * prob.k, dtype=torch.float16, device=dev)
+    ku, kv = (tables[0].data_ptr(), tables[1].data_ptr()) if tables is not None else (None, None)
+    st = torch.cuda.current_stream().cuda_stream
+    run = lambda: h.mf_row_traffic_probe(prob.R.data_ptr(), n, P.data_ptr(), Q.data_ptr(), prob.k * 2, W, ku, kv, seed, 1 if coherent else 0, st)
+    run()
+    torch.cuda.synchronize()
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(reps)]
+    for a, b in ev:
+        a.record(); run(); b.record()
+    torch.cuda.synchronize()
+    return float(np.mean([a.elapsed_time(b) for a, b in ev]))
+
+
 def cpu_baseline(prob, cfg, seed, threads, target_updates):
     """The checker's MASCOT epoch (reference update rule, binary16 through F16C) as a Hogwild CPU loop."""
     from oracle import oracle as om
@@ -340,6 +359,7 @@ def main():
     ap.add_argument("--pmc-copy", action="store_true",
                     help="profiling aid: also run three 1 GiB device copies, the known-size kernel that FETCH_SIZE / WRITE_SIZE are scaled by")
     ap.add_argument("--skip-fp32", action="store_true", help="skip the fp32-SGD leg")
+    ap.add_argument("--skip-ceiling", action="store_true", help="skip the access-pattern probe")
     ap.add_argument("--reference-rmse", action="store_true",
                     help="also train with the reference rule on the CPU for warmup+steps epochs (minutes) and report the test RMSE delta")
     ap.add_argument("--seed", type=int, default=2021)
@@ -413,6 +433,16 @@ def main():
         "ms_steps": main_leg["ms_steps"],
         "test_rmse_after_timed_epochs": {"value": main_leg["rmse"], "epochs": a.warmup + a.steps, "test_ratings": n_test},
     }
+    if not a.skip_ceiling:
+        # what the memory system sustains for this epoch's addresses and store policy, beside the plain (non-check) epochs
+        is_check = lambda e: e >= 5 and e % cfg["interval"] == 5 % cfg["interval"] and e != cfg["epochs"] - 1
+        plain = [ms for i, ms in enumerate(main_leg["ms_steps"]) if not is_check(a.warmup + i)] or main_leg["ms_steps"]
+        tables = None if a.skip_coherent or not a.hot_row_inflight else prob.hot_tables(main_leg["workers"], a.hot_row_inflight)
+        ceil_ms = access_pattern_ceiling(torch, h, prob, main_leg["workers"], tables, not a.skip_coherent, a.seed)
+        out["roofline"]["access_pattern_ceiling"] = {
+            "note": "mf_row_traffic_probe: the same ratings, workers, hot-row tables and store policy, rows read and written "
+                    "back without the arithmetic; kernel_vs_ceiling = this time / mean plain epoch",
+            "ms": ceil_ms, "plain_epoch_ms": float(np.mean(plain)), "kernel_vs_ceiling": ceil_ms / float(np.mean(plain))}
     if not a.skip_coherent and not a.skip_exact and a.hot_row_inflight:
         e = leg(True, a.workers, 0.0)
         out["exact_coherent"] = {"note": "same workload, device-coherent rows, every row update carried out (no hot-row thinning): bound by "

@@ -30,6 +30,7 @@ SIGNATURES = {
     "mf_window_start": (u32, [u64, u32, u32, u32, u32]),
     "mf_single_sgd_hogwild": (i32, [vp, u32, vp, vp, i32, u32, u32, u32, f32, f32, u64, u32, vp, vp]),
     "mf_mem_quant_sgd_hogwild": (i32, [vp, u32, vp, vp, i32, u32, u32, u32, f32, f32, u64, u32, vp, vp]),
+    "mf_row_traffic_probe": (i32, [vp, u32, vp, vp, u32, u32, vp, vp, u64, i32, vp]),
     "mf_mpt_sgd_hogwild": (i32, [vp, u32, vp, vp, i32, u32, u32, u32, f32, u16, f32, u64, u32, vp, vp]),
     "mf_muppet_sgd_hogwild": (i32, [vp, u32, vp, vp, i32, u32, u32, u32, f32, f32, u32, vp, vp, u8, u8, u64, u32, vp, vp]),
     "mf_afp_sgd_hogwild": (i32, [vp, u32, vp, vp, i32, u32, u32, u32, f32, f32, i32, u64, u32, vp, vp]),

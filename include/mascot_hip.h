@@ -68,6 +68,16 @@ uint32_t mf_get_epoch_splits(void);
  * mf_params.hot_row_inflight > 0 (MuPPET and AFP ignore them).  No counterpart in the reference.  The tables must
  * stay valid while launches that use them are in flight. */
 int mf_set_hot_row_thinning(const uint8_t* user_keep, const uint8_t* item_keep);
+/* Measurement aid, no counterpart in the reference: the memory traffic of one epoch of updates without the
+ * arithmetic.  Worker w (one wavefront) walks ratings [w*ceil(n/W), (w+1)*ceil(n/W)); per rating it reads row u of p
+ * and row i of q (row_bytes = 128, 256 or 512 bytes each: k = 64 binary16, k = 128 binary16 / k = 64 binary32,
+ * k = 128 binary32) and writes both back unchanged, with the store policy of mf_set_row_coherence's value
+ * `coherent`.  With keep tables (as for mf_set_hot_row_thinning; both or neither) a thinned update only reads its
+ * row; an update of a hot row that is kept is a store here as well.  p and q keep their contents (writes of other
+ * code that race with the probe may be lost).  The time of this launch is what the memory system sustains for the
+ * sequence of addresses and the write policy of an epoch; bench.py reports the update kernel's time beside it. */
+int mf_row_traffic_probe(const mf_node* R, uint32_t n, void* p, void* q, uint32_t row_bytes, uint32_t num_workers,
+                         const uint8_t* user_keep, const uint8_t* item_keep, uint64_t seed, int coherent, void* stream);
 /* Number of per-block columns mf_mascot_sgd_hogwild writes into norm_sum_p / norm_sum_q
  * (the reference's `block_num`, mf_methods.cu:109). */
 uint32_t mf_mascot_norm_blocks(uint32_t num_workers);

@@ -235,3 +235,32 @@ def test_group_error_matches_host_formula(orc, k):
     # the accumulators of binary16 groups are cleared for the next check epoch (mf_methods.cu:333)
     left = from_dev(dgs, np.float32).reshape(G, k)
     assert np.all(left[prec == 0] == 0)
+
+
+@pytest.mark.parametrize("row_bytes", [128, 256, 512])
+@pytest.mark.parametrize("coherent", [0, 1])
+def test_row_traffic_probe_leaves_rows_unchanged(row_bytes, coherent):
+    """The access-pattern probe reads the two rows of every rating and writes kept ones back as they are."""
+    import torch
+    h = mfutil.hip()
+    rng = np.random.default_rng(row_bytes + coherent)
+    n_users, n_items, n = 300, 70, 20_001
+    R = np.zeros(n, mfutil.NODE)
+    R["u"] = rng.integers(0, n_users, n); R["i"] = rng.integers(0, n_items, n); R["r"] = 1.0
+    P = rng.integers(0, 256, n_users * row_bytes, dtype=np.uint8)
+    Q = rng.integers(0, 256, n_items * row_bytes, dtype=np.uint8)
+    ku = rng.choice(np.array([0, 100, 254, 255], np.uint8), n_users)
+    kv = rng.choice(np.array([0, 100, 254, 255], np.uint8), n_items)
+    dR, dP, dQ, dku, dkv = to_dev(R), to_dev(P), to_dev(Q), to_dev(ku), to_dev(kv)
+    for tables in ((None, None), (dku.data_ptr(), dkv.data_ptr())):
+        for workers in (1, 7, 4096):
+            h.mf_row_traffic_probe(dR.data_ptr(), n, dP.data_ptr(), dQ.data_ptr(), row_bytes, workers, tables[0], tables[1], 5, coherent, mfutil.stream_ptr())
+    torch.cuda.synchronize()
+    assert np.array_equal(from_dev(dP, np.uint8), P) and np.array_equal(from_dev(dQ, np.uint8), Q)
+    from importlib import import_module
+    MfError = import_module("icdm-2021_mascot_amd.capi").MfError
+    with pytest.raises(MfError, match="row_bytes must be"):
+        h.mf_row_traffic_probe(dR.data_ptr(), n, dP.data_ptr(), dQ.data_ptr(), 64, 4, None, None, 5, coherent, mfutil.stream_ptr())
+    with pytest.raises(MfError, match="both keep tables"):
+        h.mf_row_traffic_probe(dR.data_ptr(), n, dP.data_ptr(), dQ.data_ptr(), row_bytes, 4, dku.data_ptr(), None, 5, coherent, mfutil.stream_ptr())
+    h.mf_row_traffic_probe(None, 0, None, None, row_bytes, 4, None, None, 5, coherent, mfutil.stream_ptr())      # nothing to do
