@@ -8,6 +8,7 @@
 #include <iostream>
 #include <sstream>
 #include <sys/stat.h>
+#include <thread>
 
 namespace {
 
@@ -163,12 +164,46 @@ bool read_test_dataset(Dataset& d, const std::string& path)
     return true;
 }
 
+// The text of `rows` model rows: row r is k numbers from row(r), or k zeros where row(r) is null, each followed by a
+// blank -- what `f << value << " "` writes with the stream's default formatting (%g, six significant digits; the
+// reference's writers, io_utils.h:276-297,320-330).  A model of config 4 holds 64M numbers, so blocks of rows are
+// formatted by all hardware threads into their own buffers and written in order.
+template <class RowOf>
+static bool write_rows(std::ofstream& f, size_t rows, uint32_t k, RowOf row)
+{
+    const unsigned threads = std::max(1u, std::min(16u, std::thread::hardware_concurrency()));
+    const size_t block = 2048;                                   // rows per thread and round
+    std::vector<std::string> text(threads);
+    for (size_t base = 0; base < rows; base += block * threads) {
+        auto format = [&](unsigned t) {
+            std::string& out = text[t];
+            out.clear();
+            const size_t lo = std::min(rows, base + block * t), hi = std::min(rows, lo + block);
+            out.reserve((hi - lo) * k * 13);
+            char buf[40];
+            for (size_t r = lo; r < hi; ++r) {
+                const float* v = row(r);
+                if (!v) { for (uint32_t j = 0; j < k; ++j) out.append("0 ", 2); continue; }
+                for (uint32_t j = 0; j < k; ++j) out.append(buf, (size_t)std::snprintf(buf, sizeof buf, "%g ", (double)v[j]));
+            }
+        };
+        std::vector<std::thread> pool;
+        for (unsigned t = 1; t < threads; ++t) pool.emplace_back(format, t);
+        format(0);
+        for (auto& th : pool) th.join();
+        for (unsigned t = 0; t < threads; ++t) f.write(text[t].data(), (std::streamsize)text[t].size());
+        if (!f) return false;
+    }
+    return true;
+}
+
 bool save_trained_model(const Dataset& d, const float* p, const float* q, uint32_t k, const std::string& outfile)
 {
     std::cout << "Save trained model..." << std::endl;
     const std::string outpath = outfile + ".txt";
     std::ofstream f(outpath);
     if (f.fail()) { std::cout << "fail to write file named " << outpath << std::endl; std::cerr << "Error: " << std::strerror(errno); return false; }
+    // rows are indexed by original id up to the largest one; ids that never occurred have no row (zeros in the file)
     auto sorted_by_orig = [](const std::vector<uint32_t>& orig) {       // (original id, dense id), ascending original id
         std::vector<std::pair<uint32_t, uint32_t>> v(orig.size());
         for (uint32_t i = 0; i < orig.size(); ++i) v[i] = {orig[i], i};
@@ -176,20 +211,16 @@ bool save_trained_model(const Dataset& d, const float* p, const float* q, uint32
         return v;
     };
     const auto users = sorted_by_orig(d.user_orig), items = sorted_by_orig(d.item_orig);
-    f << users.back().first + 1 << " " << items.back().first + 1 << " " << k << std::endl;
-    auto dump = [&](const std::vector<std::pair<uint32_t, uint32_t>>& ids, const float* m) {
-        int prev = 0;
-        for (const auto& kv : ids) {
-            const int orig = (int)kv.first;
-            for (int c = prev; c <= orig - 1; ++c) for (uint32_t j = 0; j < k; ++j) f << 0 << " ";
-            for (uint32_t j = 0; j < k; ++j) f << m[(size_t)kv.second * k + j] << " ";
-            prev = orig + 1;
-        }
+    auto row_of = [k](const std::vector<std::pair<uint32_t, uint32_t>>& ids, const float* m, size_t orig) -> const float* {
+        auto it = std::lower_bound(ids.begin(), ids.end(), std::make_pair((uint32_t)orig, 0u));
+        return it != ids.end() && it->first == orig ? m + (size_t)it->second * k : nullptr;
     };
-    dump(users, p);
+    const size_t user_rows = users.empty() ? 0 : (size_t)users.back().first + 1, item_rows = items.empty() ? 0 : (size_t)items.back().first + 1;
+    f << user_rows << " " << item_rows << " " << k << std::endl;
+    bool ok = write_rows(f, user_rows, k, [&](size_t r) { return row_of(users, p, r); });
     f << std::endl;
-    dump(items, q);
-    return true;
+    ok = ok && write_rows(f, item_rows, k, [&](size_t r) { return row_of(items, q, r); });
+    return ok && (bool)f;
 }
 
 bool save_trained_model_reconst(uint32_t n_users, uint32_t n_items, const float* p, const float* q, uint32_t k, const std::string& outfile)
@@ -199,10 +230,10 @@ bool save_trained_model_reconst(uint32_t n_users, uint32_t n_items, const float*
     std::ofstream f(outpath);
     if (f.fail()) { std::cout << "fail to write file named " << outpath << std::endl; std::cerr << "Error: " << std::strerror(errno); return false; }
     f << n_users << " " << n_items << " " << k << std::endl;
-    for (size_t i = 0; i < (size_t)n_users * k; ++i) f << p[i] << " ";
+    bool ok = write_rows(f, n_users, k, [&](size_t r) { return p + r * k; });
     f << std::endl;
-    for (size_t i = 0; i < (size_t)n_items * k; ++i) f << q[i] << " ";
-    return true;
+    ok = ok && write_rows(f, n_items, k, [&](size_t r) { return q + r * k; });
+    return ok && (bool)f;
 }
 
 bool save_reconst_testset(const std::vector<mf_node>& test, const std::string& testfile)

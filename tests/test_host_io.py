@@ -1,0 +1,101 @@
+"""The command line's host I/O layer (csrc/io_utils.cpp) on the CPU: the TSV readers' id mapping and test-set rules
+(io_utils.h:81-111,183-238) and the two model-file layouts (io_utils.h:242-332), whose numbers must read exactly as
+`ostream << float` writes them (%g)."""
+import os
+import subprocess
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+CSRC = os.path.join(ROOT, "icdm-2021_mascot_amd", "csrc")
+
+
+@pytest.fixture(scope="module")
+def driver(tmp_path_factory):
+    exe = str(tmp_path_factory.mktemp("host_io") / "host_io_check")
+    subprocess.run(["g++", "-O1", "-std=c++17", "-pthread", "-o", exe, os.path.join(ROOT, "tests", "host_io_check.cpp"),
+                    os.path.join(CSRC, "io_utils.cpp")], check=True)
+    return exe
+
+
+def c_format(v):
+    """'%g' of a binary32 value, as printf and the stream's default float formatting give it."""
+    return "%g" % float(v)
+
+
+@pytest.mark.parametrize("k", [4, 64])
+def test_readers_and_model_files(driver, tmp_path, k):
+    train = tmp_path / "train.tsv"
+    test = tmp_path / "test.tsv"
+    # users 40, 7, 1000 and items 5, 900, 3 in first-seen order; item 2 and user 8 never occur in training
+    train_lines = [(40, 5, 3.0), (7, 900, 4.5), (40, 900, 1.0), (1000, 3, 5.0), (7, 5, 2.0), (1000, 900, 0.5)]
+    train.write_text("".join("%d\t%d\t%g\n" % t for t in train_lines))
+    # an unseen user, an unseen item, a duplicate (the later line wins), and lines out of (user, item) order
+    test_lines = [(1000, 900, 2.0), (8, 5, 1.0), (40, 2, 1.0), (7, 3, 3.5), (40, 3, 4.0), (7, 3, 2.5), (40, 5, 1.5)]
+    test.write_text("".join("%d\t%d\t%g\n" % t for t in test_lines))
+    out = str(tmp_path / "model")
+    r = subprocess.run([driver, str(train), str(test), out, str(k)], capture_output=True, text=True)
+    assert r.returncode == 0, r.stdout + r.stderr
+    lines = r.stdout.splitlines()
+    summary = [l for l in lines if l.startswith("users ")][0].split()
+    assert summary[1] == "3" and summary[3] == "3" and summary[5] == "6"
+    users = {int(l.split()[1]): int(l.split()[3]) for l in lines if l.startswith("user ")}
+    items = {int(l.split()[1]): int(l.split()[3]) for l in lines if l.startswith("item ")}
+    assert users == {0: 40, 1: 7, 2: 1000} and items == {0: 5, 1: 900, 2: 3}              # first-seen order
+    got_train = [tuple(l.split()[1:]) for l in lines if l.startswith("train ")]
+    u2d, i2d = {v: key for key, v in users.items()}, {v: key for key, v in items.items()}
+    assert got_train == [(str(u2d[u]), str(i2d[i]), "%.9g" % r_) for u, i, r_ in train_lines]
+    # test set: unseen ids dropped (and listed), duplicates folded, ordered by dense user then dense item
+    got_test = [(int(a), int(b), float(c)) for a, b, c in (l.split()[1:] for l in lines if l.startswith("test "))]
+    want = {}
+    for u, i, r_ in test_lines:
+        if u in u2d and i in i2d:
+            want[(u2d[u], i2d[i])] = r_
+    assert got_test == [(u, i, want[(u, i)]) for u, i in sorted(want)]
+    assert (tmp_path / "remove_user.txt").read_text().split() == ["8"]
+    assert (tmp_path / "remove_item.txt").read_text().split() == ["2"]
+    # the values the driver put into P and Q
+    vals = np.fromfile(out + ".values", np.float32)
+    P, Q = vals[:3 * k].reshape(3, k), vals[3 * k:].reshape(3, k)
+    # <out>_reconst.txt: header, then the rows in dense order
+    text = open(out + "_reconst.txt").read()
+    head, body_p, body_q = text.split("\n")
+    assert head == "3 3 %d" % k
+    assert body_p == "".join(c_format(v) + " " for v in P.reshape(-1))
+    assert body_q == "".join(c_format(v) + " " for v in Q.reshape(-1))
+    # <out>.txt: rows by original id, zeros for ids that never occurred
+    text = open(out + ".txt").read()
+    head, body_p, body_q = text.split("\n")
+    assert head == "1001 901 %d" % k
+    tok = body_p.split(" ")
+    assert tok[-1] == "" and len(tok) == 1001 * k + 1
+    for orig in range(1001):
+        row = tok[orig * k:(orig + 1) * k]
+        assert row == ([c_format(v) for v in P[u2d[orig]]] if orig in u2d else ["0"] * k), orig
+    tok = body_q.split(" ")
+    assert len(tok) == 901 * k + 1
+    for orig in (0, 2, 3, 4, 5, 6, 899, 900):
+        row = tok[orig * k:(orig + 1) * k]
+        assert row == ([c_format(v) for v in Q[i2d[orig]]] if orig in i2d else ["0"] * k), orig
+    # reconst_<testfile>: the kept test ratings in the dense index space, user first
+    rec = (tmp_path / "reconst_test.tsv").read_text().splitlines()
+    assert rec == ["%d\t%d\t%s" % (u, i, c_format(np.float32(want[(u, i)]))) for u, i in sorted(want)]
+    assert [l for l in lines if l.startswith("reread ")][0] == "reread users 3 items 3 k %d p %d q %d" % (k, 3 * k, 3 * k)
+
+
+def test_many_rows_are_written_in_order(driver, tmp_path):
+    """More rows than one formatting block per thread: the blocks must land in the file in row order."""
+    n_users, n_items, k = 70_001, 3, 2
+    train = tmp_path / "train.tsv"
+    train.write_text("".join("%d\t%d\t1\n" % (u, u % n_items) for u in range(n_users)))
+    test = tmp_path / "test.tsv"
+    test.write_text("0\t0\t1\n")
+    out = str(tmp_path / "m")
+    r = subprocess.run([driver, str(train), str(test), out, str(k)], capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr
+    vals = np.fromfile(out + ".values", np.float32)
+    P = vals[:n_users * k]
+    head, body_p, body_q = open(out + "_reconst.txt").read().split("\n")
+    assert head == "%d %d %d" % (n_users, n_items, k)
+    assert body_p == "".join(c_format(v) + " " for v in P)
