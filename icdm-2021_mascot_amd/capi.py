@@ -31,6 +31,9 @@ SIGNATURES = {
     "mf_single_sgd_hogwild": (i32, [vp, u32, vp, vp, i32, u32, u32, u32, f32, f32, u64, u32, vp, vp]),
     "mf_mem_quant_sgd_hogwild": (i32, [vp, u32, vp, vp, i32, u32, u32, u32, f32, f32, u64, u32, vp, vp]),
     "mf_row_traffic_probe": (i32, [vp, u32, vp, vp, u32, u32, vp, vp, u64, i32, vp]),
+    "mf_synth_baseline_config": (i32, [i32, vp]),
+    "mf_generate_ratings": (i32, [vp, u64, u64, u64, vp, vp]),
+    "mf_generate_ratings_host": (i32, [vp, u64, u64, u64, vp]),
     "mf_mpt_sgd_hogwild": (i32, [vp, u32, vp, vp, i32, u32, u32, u32, f32, u16, f32, u64, u32, vp, vp]),
     "mf_muppet_sgd_hogwild": (i32, [vp, u32, vp, vp, i32, u32, u32, u32, f32, f32, u32, vp, vp, u8, u8, u64, u32, vp, vp]),
     "mf_afp_sgd_hogwild": (i32, [vp, u32, vp, vp, i32, u32, u32, u32, f32, f32, i32, u64, u32, vp, vp]),
@@ -57,6 +60,12 @@ SIGNATURES = {
 
 
 f64 = C.c_double
+
+
+class SynthConfig(C.Structure):
+    """mf_synth_config of include/mascot_hip.h."""
+    _fields_ = [("n_users", u32), ("n_items", u32), ("n_train", u64), ("n_test", u64), ("user_alpha", f32), ("item_alpha", f32),
+                ("rank", u32), ("noise", f32), ("mean", f32), ("step", f32), ("lo", f32), ("hi", f32), ("bimodal", u32)]
 
 
 class MfParams(C.Structure):
@@ -120,6 +129,12 @@ class MascotHip:
         raise AttributeError(name)
 
     # ---- host-level helpers over numpy arrays ----------------------------------------------
+    def synth_config(self, config):
+        """The synthetic stand-in of BASELINE.json's configuration `config` (1..5)."""
+        c = SynthConfig()
+        self.mf_synth_baseline_config(config, C.addressof(c))
+        return c
+
     def default_params(self, **kw):
         prm = MfParams()
         self.lib.mf_default_params(C.byref(prm))

@@ -4,6 +4,8 @@
 #include "mf_host.h"
 #include "mf_device.h"
 #include <type_traits>
+#include <cmath>
+#include <vector>
 
 namespace mf {
 
@@ -273,17 +275,61 @@ __device__ __forceinline__ double det_cos2pi(double t)
     s = a * s;
     switch (q & 3) { case 0: return c; case 1: return -s; case 2: return -c; default: return s; }
 }
-__global__ __launch_bounds__(kStreamBlock) void init_normal_kernel(float* __restrict__ out, uint64_t n, uint64_t base)
+// N(0,1) from 64 bits (Box-Muller over the two 32-bit halves)
+__device__ __forceinline__ double det_normal(uint64_t h)
+{
+    const uint32_t a = (uint32_t)(h >> 32), b = (uint32_t)h;
+    const double u1 = ((double)a + 1.0) * 2.3283064365386962890625e-10;
+    const double u2 = (double)b * 2.3283064365386962890625e-10;
+    const double rad = __builtin_sqrt(-2.0 * det_log(u1));
+    return rad * det_cos2pi(u2);
+}
+__global__ __launch_bounds__(kStreamBlock) void init_normal_kernel(float* __restrict__ out, uint64_t n, uint64_t base, double scale)
 {
     const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
-    for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
-        const uint64_t h = mix64(base ^ i);
-        const uint32_t a = (uint32_t)(h >> 32), b = (uint32_t)h;
-        const double u1 = ((double)a + 1.0) * 2.3283064365386962890625e-10;
-        const double u2 = (double)b * 2.3283064365386962890625e-10;
-        const double rad = __builtin_sqrt(-2.0 * det_log(u1));
-        const double z = rad * det_cos2pi(u2);
-        out[i] = (float)(z * 0.01);
+    for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride)
+        out[i] = (float)(det_normal(mix64(base ^ i)) * scale);
+}
+
+// ---- seeded synthetic ratings (mf_generate_ratings) ------------------------------------------------
+struct SynthTables {
+    const double* user_cdf; const double* item_cdf;       // cumulative Zipf weights, last entry 1.0
+    const uint32_t* user_perm; const uint32_t* item_perm; // popularity rank -> id
+    const float* U; const float* V;                       // [rows][rank] factors, or null (bimodal)
+};
+// smallest index whose cumulative weight exceeds x (x in [0,1), cdf[count-1] = 1)
+__device__ __forceinline__ uint32_t cdf_rank(const double* cdf, uint32_t count, double x)
+{
+    uint32_t lo = 0, hi = count - 1;
+    while (lo < hi) {
+        const uint32_t mid = (lo + hi) >> 1;
+        if (x < cdf[mid]) hi = mid; else lo = mid + 1;
+    }
+    return lo;
+}
+__global__ __launch_bounds__(kStreamBlock) void generate_ratings_kernel(mf_synth_config c, SynthTables t, uint64_t key, uint64_t first, uint64_t count,
+                                                                      float inv_step, mf_node* __restrict__ out)
+{
+    const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+    for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += stride) {
+        const uint64_t j = first + i;
+        const double xu = (double)(mix64(key ^ (j * 4 + 0)) >> 11) * 1.1102230246251565404e-16;      // 53 bits in [0,1)
+        const double xi = (double)(mix64(key ^ (j * 4 + 1)) >> 11) * 1.1102230246251565404e-16;
+        const uint32_t u = t.user_perm[cdf_rank(t.user_cdf, c.n_users, xu)];
+        const uint32_t v = t.item_perm[cdf_rank(t.item_cdf, c.n_items, xi)];
+        const float nz = (float)(det_normal(mix64(key ^ (j * 4 + 2))) * (double)c.noise);
+        float r;
+        if (c.bimodal) {
+            const double xm = (double)(mix64(key ^ (j * 4 + 3)) >> 11) * 1.1102230246251565404e-16;
+            const float m = xm < 0.5 ? 20.0f : 80.0f;
+            r = fminf(fmaxf(roundf(m + nz), c.lo), c.hi) * 0.04f + 1.0f;
+        } else {
+            float dot = 0.0f;
+            for (uint32_t k = 0; k < c.rank; ++k) dot = dot + t.U[(size_t)u * c.rank + k] * t.V[(size_t)v * c.rank + k];
+            const float val = (dot + c.mean) + nz;
+            r = fminf(fmaxf(roundf(val * inv_step) * c.step, c.lo), c.hi);
+        }
+        out[i].r = r; out[i].u = u; out[i].i = v;
     }
 }
 
@@ -395,6 +441,45 @@ __global__ __launch_bounds__(kBlock) void row_traffic_probe_kernel(const mf_node
     }
 }
 
+namespace {
+// cumulative weights (rank+1)^-alpha, normalised by their sum; summed in rank order in double
+std::vector<double> zipf_cdf(uint32_t count, float alpha)
+{
+    std::vector<double> cdf(count);
+    double sum = 0.0;
+    for (uint32_t i = 0; i < count; ++i) { sum += std::pow((double)(i + 1), -(double)alpha); cdf[i] = sum; }
+    for (uint32_t i = 0; i < count; ++i) cdf[i] = cdf[i] / sum;
+    return cdf;
+}
+// Fisher-Yates with the counter-based generator
+std::vector<uint32_t> seeded_permutation(uint32_t count, uint64_t base)
+{
+    std::vector<uint32_t> p(count);
+    for (uint32_t i = 0; i < count; ++i) p[i] = i;
+    for (uint32_t i = count; i-- > 1;) { const uint32_t j = (uint32_t)(mix64(base ^ (uint64_t)i) % ((uint64_t)i + 1)); std::swap(p[i], p[j]); }
+    return p;
+}
+struct DeviceTables {      // frees what it allocated when it goes out of scope
+    std::vector<void*> owned;
+    ~DeviceTables() { for (void* p : owned) (void)hipFree(p); }
+    template <class T> int upload(const std::vector<T>& h, const T** d, hipStream_t st)
+    {
+        void* p = nullptr;
+        if (int rc = check_hip(hipMalloc(&p, h.size() * sizeof(T) + 16), "hipMalloc(synthetic tables)")) return rc;
+        owned.push_back(p);
+        if (int rc = check_hip(hipMemcpyAsync(p, h.data(), h.size() * sizeof(T), hipMemcpyHostToDevice, st), "hipMemcpyAsync(synthetic tables)")) return rc;
+        *d = static_cast<const T*>(p);
+        return MF_OK;
+    }
+    int alloc(size_t bytes, void** d)
+    {
+        if (int rc = check_hip(hipMalloc(d, bytes + 16), "hipMalloc(synthetic factors)")) return rc;
+        owned.push_back(*d);
+        return MF_OK;
+    }
+};
+}  // namespace
+
 extern "C" {
 
 int mf_transform_float2half(const float* in, uint16_t* out, uint64_t n, void* stream)
@@ -484,7 +569,7 @@ int mf_init_rand_feature(float* array, uint64_t n, uint64_t seed, uint64_t strea
     if (n == 0) return MF_OK;
     if (!array) return invalid("mf_init_rand_feature: null pointer");
     const uint64_t base = mix64(mix64(seed ^ 0x494E49544E4F524Dull) + stream_id);
-    hipLaunchKernelGGL(init_normal_kernel, dim3(stream_grid(n)), dim3(kStreamBlock), 0, as_stream(stream), array, n, base);
+    hipLaunchKernelGGL(init_normal_kernel, dim3(stream_grid(n)), dim3(kStreamBlock), 0, as_stream(stream), array, n, base, 0.01);
     return launch_status("mf_init_rand_feature");
 }
 
@@ -535,6 +620,67 @@ int mf_row_traffic_probe(const mf_node* R, uint32_t n, void* p, void* q, uint32_
     else { if (coherent) MF_PROBE(8, true); else MF_PROBE(8, false); }
 #undef MF_PROBE
     return launch_status("mf_row_traffic_probe");
+}
+
+int mf_synth_baseline_config(int config, mf_synth_config* out)
+{
+    if (!out) return invalid("mf_synth_baseline_config: null pointer");
+    //                          users    items    train       test     alpha_u alpha_i rank noise  mean  step  lo    hi   bimodal
+    static const mf_synth_config table[5] = {
+        {5000u, 2000u, 400000ull, 100000ull, 1.0f, 1.0f, 8u, 0.8f, 3.5f, 1.0f, 1.0f, 5.0f, 0u},
+        {70000u, 10700u, 8000000ull, 2000000ull, 0.9f, 0.9f, 16u, 0.8f, 3.5f, 0.5f, 0.5f, 5.0f, 0u},
+        {162000u, 59000u, 20000000ull, 5000000ull, 1.0f, 1.0f, 16u, 0.8f, 3.5f, 0.5f, 0.5f, 5.0f, 0u},
+        {480000u, 17800u, 100000000ull, 1400000ull, 0.8f, 1.1f, 32u, 0.9f, 3.6f, 1.0f, 1.0f, 5.0f, 0u},
+        {1000000u, 625000u, 250000000ull, 4000000ull, 1.2f, 1.2f, 0u, 15.0f, 0.0f, 1.0f, 0.0f, 100.0f, 1u},
+    };
+    if (config < 1 || config > 5) return invalid("mf_synth_baseline_config: configurations are numbered 1..5 (got %d)", config);
+    *out = table[config - 1];
+    return MF_OK;
+}
+
+int mf_generate_ratings(const mf_synth_config* cfg, uint64_t seed, uint64_t first, uint64_t count, mf_node* out, void* stream)
+{
+    if (!cfg) return invalid("mf_generate_ratings: null configuration");
+    if (count == 0) return MF_OK;
+    if (!out) return invalid("mf_generate_ratings: null output");
+    const mf_synth_config c = *cfg;
+    if (c.n_users == 0 || c.n_items == 0) return invalid("mf_generate_ratings: no users or no items");
+    if (!c.bimodal && (c.rank == 0 || c.rank > 1024u)) return invalid("mf_generate_ratings: rank must be 1..1024 (got %u)", c.rank);
+    if (!(c.step > 0.0f) || !(c.lo <= c.hi)) return invalid("mf_generate_ratings: step must be positive and lo <= hi");
+    hipStream_t st = as_stream(stream);
+    const uint64_t key = mix64(seed ^ 0x53594E5448455449ull);
+    DeviceTables dev;
+    SynthTables t = {};
+    const std::vector<double> ucdf = zipf_cdf(c.n_users, c.user_alpha), icdf = zipf_cdf(c.n_items, c.item_alpha);
+    const std::vector<uint32_t> uperm = seeded_permutation(c.n_users, mix64(key + 1)), iperm = seeded_permutation(c.n_items, mix64(key + 2));
+    if (int rc = dev.upload(ucdf, &t.user_cdf, st)) return rc;
+    if (int rc = dev.upload(icdf, &t.item_cdf, st)) return rc;
+    if (int rc = dev.upload(uperm, &t.user_perm, st)) return rc;
+    if (int rc = dev.upload(iperm, &t.item_perm, st)) return rc;
+    if (!c.bimodal) {
+        void *U = nullptr, *V = nullptr;
+        const uint64_t nu = (uint64_t)c.n_users * c.rank, nv = (uint64_t)c.n_items * c.rank;
+        if (int rc = dev.alloc(nu * sizeof(float), &U)) return rc;
+        if (int rc = dev.alloc(nv * sizeof(float), &V)) return rc;
+        hipLaunchKernelGGL(init_normal_kernel, dim3(stream_grid(nu)), dim3(kStreamBlock), 0, st, static_cast<float*>(U), nu, mix64(key + 3), 0.5);
+        hipLaunchKernelGGL(init_normal_kernel, dim3(stream_grid(nv)), dim3(kStreamBlock), 0, st, static_cast<float*>(V), nv, mix64(key + 4), 0.5);
+        t.U = static_cast<const float*>(U); t.V = static_cast<const float*>(V);
+    }
+    hipLaunchKernelGGL(generate_ratings_kernel, dim3(stream_grid(count)), dim3(kStreamBlock), 0, st, c, t, key, first, count, 1.0f / c.step, out);
+    if (int rc = launch_status("mf_generate_ratings")) return rc;
+    return check_hip(hipStreamSynchronize(st), "mf_generate_ratings: hipStreamSynchronize");       // the tables are freed on return
+}
+
+int mf_generate_ratings_host(const mf_synth_config* cfg, uint64_t seed, uint64_t first, uint64_t count, mf_node* host_out)
+{
+    if (count == 0) return MF_OK;
+    if (!host_out) return invalid("mf_generate_ratings_host: null output");
+    void* dev = nullptr;
+    if (int rc = check_hip(hipMalloc(&dev, count * sizeof(mf_node)), "mf_generate_ratings_host: hipMalloc")) return rc;
+    int rc = mf_generate_ratings(cfg, seed, first, count, static_cast<mf_node*>(dev), nullptr);
+    if (rc == MF_OK) rc = check_hip(hipMemcpy(host_out, dev, count * sizeof(mf_node), hipMemcpyDeviceToHost), "mf_generate_ratings_host: hipMemcpy");
+    (void)hipFree(dev);
+    return rc;
 }
 
 }  // extern "C"

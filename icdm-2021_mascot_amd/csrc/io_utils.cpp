@@ -164,6 +164,26 @@ bool read_test_dataset(Dataset& d, const std::string& path)
     return true;
 }
 
+void dataset_from_ratings(Dataset& d, std::vector<mf_node>&& train, const std::vector<mf_node>& test, uint32_t n_users, uint32_t n_items)
+{
+    d = Dataset();
+    d.R = std::move(train);
+    d.max_user = n_users; d.max_item = n_items;
+    d.user_orig.resize(n_users); d.item_orig.resize(n_items);
+    for (uint32_t i = 0; i < n_users; ++i) d.user_orig[i] = i;
+    for (uint32_t i = 0; i < n_items; ++i) d.item_orig[i] = i;
+    std::vector<uint8_t> user_seen(n_users, 0), item_seen(n_items, 0);
+    for (const mf_node& t : d.R) { user_seen[t.u] = 1; item_seen[t.i] = 1; }
+    std::vector<std::map<uint32_t, float>> test_R(n_users);
+    for (const mf_node& t : test) {
+        if (t.u < n_users && t.i < n_items && user_seen[t.u] && item_seen[t.i]) { test_R[t.u][t.i] = t.r; d.test_lines_kept++; }
+        else if (t.u >= n_users || !user_seen[t.u]) { d.test_missing++; d.remove_user.push_back(t.u); }
+        else { d.test_missing++; d.remove_item.push_back(t.i); }
+    }
+    for (uint32_t u = 0; u < n_users; ++u)
+        for (const auto& kv : test_R[u]) d.test.push_back({kv.second, u, kv.first});
+}
+
 // The text of `rows` model rows: row r is k numbers from row(r), or k zeros where row(r) is null, each followed by a
 // blank -- what `f << value << " "` writes with the stream's default formatting (%g, six significant digits; the
 // reference's writers, io_utils.h:276-297,320-330).  A model of config 4 holds 64M numbers, so blocks of rows are

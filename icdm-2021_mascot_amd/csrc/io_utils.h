@@ -29,6 +29,11 @@ bool read_test_dataset(Dataset& d, const std::string& path);
 // times) loads that instead of parsing, prints the same "Missing the number of ratings" line and rewrites the two
 // remove_*.txt files.  Without use_cache this is read_training_dataset followed by read_test_dataset.
 bool load_dataset(Dataset& d, const std::string& train_path, const std::string& test_path, bool use_cache, bool* from_cache = nullptr);
+// A data set from ratings that are already in memory with dense ids (the synthetic generator): `train` is taken as
+// it is; `test` goes through the test-set rules of read_test_dataset (ratings of users or items without a training
+// rating are dropped and counted, one rating per (user, item) with the later one winning, ordered by user then
+// item).  Original ids are the dense ids; no remove_*.txt files are written.
+void dataset_from_ratings(Dataset& d, std::vector<mf_node>&& train, const std::vector<mf_node>& test, uint32_t n_users, uint32_t n_items);
 // save_trained_model, io_utils.h:242-303: <out>.txt, rows by original id, zero rows for absent ids
 bool save_trained_model(const Dataset& d, const float* p, const float* q, uint32_t k, const std::string& outfile);
 // save_trained_model_reconst, io_utils.h:305-332: <out>_reconst.txt, rows in the order given

@@ -1,7 +1,9 @@
 // quantized_mf: the reference's command line (main.cu:15-175) over libmascot_hip.
 // Same flags, same stdout lines, same model files.  Additions: `-seed <n>` (the reference seeds from
 // time(0) and clock(), so two of its runs never agree; here the default seed is fixed), `-cached <0|1>`
-// and `-split <n>` (row access policy and kernel launches per epoch, see include/mascot_hip.h).
+// and `-split <n>` (row access policy and kernel launches per epoch, see include/mascot_hip.h), `-synth <c>[,<n>]`
+// (no input files: the seeded synthetic stand-in of BASELINE configuration c, optionally with n training ratings
+// and the test set scaled alike, generated on the device; mf_generate_ratings).
 #include <sys/stat.h>
 #include <cstdlib>
 #include <cstdio>
@@ -19,6 +21,7 @@ int main(int argc, const char* argv[])
     mf_default_params(&prm);
     unsigned reconst_save = 0;
     int use_cache = 0;                                // -cache 1: keep the parsed ratings in <input>.mfcache
+    int synth = 0; unsigned long long synth_train = 0;  // -synth <config>[,<training ratings>]
     const char* usage = " [-t <threads> -p <predictions/user> -o <output-tsv>] <input-tsv>";
     if (argc < 2) { std::cout << argv[0] << usage << std::endl; return 0; }
     if (argc == 2) infile = argv[1];
@@ -55,10 +58,20 @@ int main(int argc, const char* argv[])
                 if (got >= 3) prm.hot_row_early_epochs = ep;
             }
             if (a == "-cache" && has) use_cache = std::atoi(argv[i + 1]);
+            if (a == "-synth" && has) std::sscanf(argv[i + 1], "%d,%llu", &synth, &synth_train);
             if (a == "-h") { std::cout << argv[0] << usage << std::endl; return 0; }
         }
     }
-    if (!exists(infile)) { std::cout << infile << " doesn't exist!" << std::endl; return 0; }
+    mf_synth_config sc = {};
+    if (synth) {
+        if (int rc = mf_synth_baseline_config(synth, &sc)) { std::cerr << "quantized_mf: " << mf_last_error() << std::endl; return rc > 0 ? rc : 1; }
+        if (synth_train && synth_train < sc.n_train) {
+            sc.n_test = (uint64_t)((double)sc.n_test * (double)synth_train / (double)sc.n_train);
+            sc.n_train = synth_train;
+        }
+        infile = "synthetic configuration " + std::to_string(synth);
+        if (synth == 5) prm.is_yahoo = 1;               // 0..100 ratings, rescaled like the reference's Yahoo set
+    } else if (!exists(infile)) { std::cout << infile << " doesn't exist!" << std::endl; return 0; }
 
     std::cout << std::endl;
     std::cout << "Input file                  : " << infile << std::endl;
@@ -78,14 +91,23 @@ int main(int argc, const char* argv[])
 
     Dataset d;
     bool from_cache = false;
-    load_dataset(d, infile, testfile, use_cache != 0, &from_cache);
+    if (synth) {
+        std::vector<mf_node> all(sc.n_train + sc.n_test);
+        if (int rc = mf_generate_ratings_host(&sc, prm.seed, 0, all.size(), all.data())) { std::cerr << "quantized_mf: " << mf_last_error() << std::endl; return rc > 0 ? rc : 1; }
+        std::vector<mf_node> test(all.begin() + (std::ptrdiff_t)sc.n_train, all.end());
+        all.resize(sc.n_train);
+        dataset_from_ratings(d, std::move(all), test, sc.n_users, sc.n_items);
+        std::cout << "Missing the number of ratings : " << d.test_missing << std::endl;
+    } else {
+        load_dataset(d, infile, testfile, use_cache != 0, &from_cache);
+    }
     if (from_cache) std::cout << "Ratings loaded from " << infile << ".mfcache" << std::endl;
     std::cout << "The number of nonzeros      : " << d.R.size() << std::endl;
     std::cout << "The number of users         : " << d.max_user << std::endl;
     std::cout << "The number of items         : " << d.max_item << std::endl;
     std::cout << "The number of test nonzeros : " << d.test.size() << std::endl;
 
-    prm.is_yahoo = infile.find("Yahoo") != std::string::npos;
+    if (!synth) prm.is_yahoo = infile.find("Yahoo") != std::string::npos;
     prm.verbose = 1;
     if (prm.version == 0) prm.version = 5;          // "-v 0" is accepted as plain fp32 SGD
     const size_t pn = (size_t)d.max_user * prm.k, qn = (size_t)d.max_item * prm.k;
@@ -128,6 +150,6 @@ int main(int argc, const char* argv[])
         if (prm.version == 1 || prm.version == 6) save_trained_model_reconst(d.max_user, d.max_item, p.data(), q.data(), prm.k, outfile);
         else save_trained_model(d, p.data(), q.data(), prm.k, outfile);
     }
-    if ((prm.version == 1 || prm.version == 6) && reconst_save == 1) save_reconst_testset(test_reconst, testfile);
+    if ((prm.version == 1 || prm.version == 6) && reconst_save == 1 && !synth) save_reconst_testset(test_reconst, testfile);
     return 0;
 }

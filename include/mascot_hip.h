@@ -68,6 +68,29 @@ uint32_t mf_get_epoch_splits(void);
  * mf_params.hot_row_inflight > 0 (MuPPET and AFP ignore them).  No counterpart in the reference.  The tables must
  * stay valid while launches that use them are in flight. */
 int mf_set_hot_row_thinning(const uint8_t* user_keep, const uint8_t* item_keep);
+/* Seeded synthetic ratings (no counterpart in the reference, whose data sets are downloaded): users and items are
+ * drawn independently from Zipf(alpha) over a random permutation of the ids; a rating is
+ * clamp(round_to_step(U_u . V_i + mean + noise * N(0,1)), lo, hi) with rank-`rank` factors U, V ~ N(0, 0.5^2), or,
+ * with bimodal != 0, clamp(round(m + noise * N(0,1)), lo, hi) * 0.04 + 1 with m = 20 or 80 (the 0..100 ratings of
+ * BASELINE.json's fifth configuration mapped like the reference maps its 0..100 data set, io_utils.h:75).  Rating j
+ * depends on (seed, j) only, so any range [first, first + count) of the stream can be generated on its own; the
+ * command line takes the first n_train ratings for training and the next n_test for the test set. */
+typedef struct {
+    uint32_t n_users, n_items;
+    uint64_t n_train, n_test;
+    float user_alpha, item_alpha;
+    uint32_t rank;
+    float noise, mean, step, lo, hi;
+    uint32_t bimodal;
+} mf_synth_config;
+/* The synthetic stand-ins of BASELINE.json's configurations 1..5; MF_EINVAL for any other number. */
+int mf_synth_baseline_config(int config, mf_synth_config* out);
+/* Writes ratings [first, first + count) of the stream to the device array `out` (ids are dense, 0-based).
+ * Builds its tables (two CDFs, two permutations, the factors) on every call and frees them before returning, so it
+ * synchronises the stream. */
+int mf_generate_ratings(const mf_synth_config* cfg, uint64_t seed, uint64_t first, uint64_t count, mf_node* out, void* stream);
+/* The same into a host array (allocates, generates on the default stream, copies back, frees). */
+int mf_generate_ratings_host(const mf_synth_config* cfg, uint64_t seed, uint64_t first, uint64_t count, mf_node* host_out);
 /* Measurement aid, no counterpart in the reference: the memory traffic of one epoch of updates without the
  * arithmetic.  Worker w (one wavefront) walks ratings [w*ceil(n/W), (w+1)*ceil(n/W)); per rating it reads row u of p
  * and row i of q (row_bytes = 128, 256 or 512 bytes each: k = 64 binary16, k = 128 binary16 / k = 64 binary32,

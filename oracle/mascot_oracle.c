@@ -300,18 +300,90 @@ static double det_cos2pi(double t)
 /* init_rand_feature_single, model_init.cu:19-28: array[i] = (float)(N(0,1) * 0.01).
  * The normal deviate is a Box-Muller transform of this build's counter-based bits
  * (the reference draws from cuRAND states seeded with clock()).  parity unpinned. */
+static double det_normal(uint64_t h)
+{
+    uint32_t a = (uint32_t)(h >> 32), b = (uint32_t)h;
+    double u1 = ((double)a + 1.0) * 2.3283064365386962890625e-10;
+    double u2 = (double)b * 2.3283064365386962890625e-10;
+    double rad = sqrt(-2.0 * det_log(u1));
+    return rad * det_cos2pi(u2);
+}
+static void normal_array(uint64_t base, double scale, float* out, uint64_t n)
+{
+    for (uint64_t i = 0; i < n; i++) out[i] = (float)(det_normal(mix64(base ^ i)) * scale);
+}
 void orc_init_normal(uint64_t seed, uint64_t stream, float* out, uint64_t n)
 {
-    uint64_t base = mix64(mix64(seed ^ 0x494E49544E4F524Dull) + stream);
-    for (uint64_t i = 0; i < n; i++) {
-        uint64_t h = mix64(base ^ i);
-        uint32_t a = (uint32_t)(h >> 32), b = (uint32_t)h;
-        double u1 = ((double)a + 1.0) * 2.3283064365386962890625e-10;
-        double u2 = (double)b * 2.3283064365386962890625e-10;
-        double rad = sqrt(-2.0 * det_log(u1));
-        double z = rad * det_cos2pi(u2);
-        out[i] = (float)(z * 0.01);
+    normal_array(mix64(mix64(seed ^ 0x494E49544E4F524Dull) + stream), 0.01, out, n);
+}
+
+/* Seeded synthetic ratings: the CPU twin of this build's generator (the reference has none; its data sets are
+ * downloaded).  Users and items from Zipf(alpha) over a seeded permutation of the ids, ratings from a low-rank
+ * truth plus noise rounded to the rating grid, or bimodal 0..100 ratings mapped to r * 0.04 + 1.  parity unpinned
+ * against the reference by construction; pinned against the distribution it claims (tests/test_oracle_host.py). */
+static uint32_t cdf_rank(const double* cdf, uint32_t count, double x)
+{
+    uint32_t lo = 0, hi = count - 1;
+    while (lo < hi) {
+        uint32_t mid = (lo + hi) >> 1;
+        if (x < cdf[mid]) hi = mid; else lo = mid + 1;
     }
+    return lo;
+}
+static double* zipf_cdf(uint32_t count, float alpha)
+{
+    double* cdf = (double*)malloc((size_t)count * sizeof(double));
+    double sum = 0.0;
+    for (uint32_t i = 0; i < count; i++) { sum += pow((double)(i + 1), -(double)alpha); cdf[i] = sum; }
+    for (uint32_t i = 0; i < count; i++) cdf[i] = cdf[i] / sum;
+    return cdf;
+}
+static uint32_t* seeded_permutation(uint32_t count, uint64_t base)
+{
+    uint32_t* p = (uint32_t*)malloc((size_t)count * sizeof(uint32_t));
+    for (uint32_t i = 0; i < count; i++) p[i] = i;
+    for (uint32_t i = count; i-- > 1;) {
+        uint32_t j = (uint32_t)(mix64(base ^ (uint64_t)i) % ((uint64_t)i + 1));
+        uint32_t t = p[i]; p[i] = p[j]; p[j] = t;
+    }
+    return p;
+}
+void orc_generate_ratings(const orc_synth_config* c, uint64_t seed, uint64_t first, uint64_t count, orc_node* out)
+{
+    uint64_t key = mix64(seed ^ 0x53594E5448455449ull);
+    double* ucdf = zipf_cdf(c->n_users, c->user_alpha);
+    double* icdf = zipf_cdf(c->n_items, c->item_alpha);
+    uint32_t* uperm = seeded_permutation(c->n_users, mix64(key + 1));
+    uint32_t* iperm = seeded_permutation(c->n_items, mix64(key + 2));
+    float *U = NULL, *V = NULL;
+    if (!c->bimodal) {
+        U = (float*)malloc((size_t)c->n_users * c->rank * sizeof(float));
+        V = (float*)malloc((size_t)c->n_items * c->rank * sizeof(float));
+        normal_array(mix64(key + 3), 0.5, U, (uint64_t)c->n_users * c->rank);
+        normal_array(mix64(key + 4), 0.5, V, (uint64_t)c->n_items * c->rank);
+    }
+    float inv_step = 1.0f / c->step;
+    for (uint64_t i = 0; i < count; i++) {
+        uint64_t j = first + i;
+        double xu = (double)(mix64(key ^ (j * 4 + 0)) >> 11) * 1.1102230246251565404e-16;
+        double xi = (double)(mix64(key ^ (j * 4 + 1)) >> 11) * 1.1102230246251565404e-16;
+        uint32_t u = uperm[cdf_rank(ucdf, c->n_users, xu)];
+        uint32_t v = iperm[cdf_rank(icdf, c->n_items, xi)];
+        float nz = (float)(det_normal(mix64(key ^ (j * 4 + 2))) * (double)c->noise);
+        float r;
+        if (c->bimodal) {
+            double xm = (double)(mix64(key ^ (j * 4 + 3)) >> 11) * 1.1102230246251565404e-16;
+            float m = xm < 0.5 ? 20.0f : 80.0f;
+            r = fminf(fmaxf(roundf(m + nz), c->lo), c->hi) * 0.04f + 1.0f;
+        } else {
+            float dot = 0.0f;
+            for (uint32_t k = 0; k < c->rank; k++) dot = dot + U[(size_t)u * c->rank + k] * V[(size_t)v * c->rank + k];
+            float val = (dot + c->mean) + nz;
+            r = fminf(fmaxf(roundf(val * inv_step) * c->step, c->lo), c->hi);
+        }
+        out[i].r = r; out[i].u = u; out[i].i = v;
+    }
+    free(ucdf); free(icdf); free(uperm); free(iperm); free(U); free(V);
 }
 
 /* ------------------------------------------------------------------------ */

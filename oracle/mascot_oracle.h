@@ -63,6 +63,16 @@ void orc_group_lookup(uint32_t idx, const uint32_t* end_idx, uint32_t groups, ui
 void orc_shuffle_keys(uint64_t seed, uint64_t n, uint64_t* keys);
 void orc_shuffle(uint64_t seed, const orc_node* in, orc_node* out, uint64_t n);
 void orc_init_normal(uint64_t seed, uint64_t stream, float* out, uint64_t n);
+/* Seeded synthetic ratings, the twin of the build's mf_generate_ratings (same field order as mf_synth_config). */
+typedef struct {
+    uint32_t n_users, n_items;
+    uint64_t n_train, n_test;
+    float user_alpha, item_alpha;
+    uint32_t rank;
+    float noise, mean, step, lo, hi;
+    uint32_t bimodal;
+} orc_synth_config;
+void orc_generate_ratings(const orc_synth_config* c, uint64_t seed, uint64_t first, uint64_t count, orc_node* out);
 
 /* ---- single updates (in place on one P row and one Q row) -------------- */
 void orc_sgd_update(int k, float* p, float* q, float r, float lr, float lambda);

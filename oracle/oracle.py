@@ -27,6 +27,13 @@ class AfpQ(C.Structure):
     _fields_ = [("r", C.c_int), ("n", C.c_int), ("itv", C.c_int), ("mov_avg_range", C.c_float)]
 
 
+class SynthConfig(C.Structure):
+    """orc_synth_config (= mf_synth_config of the library)."""
+    _fields_ = [("n_users", C.c_uint32), ("n_items", C.c_uint32), ("n_train", C.c_uint64), ("n_test", C.c_uint64),
+                ("user_alpha", C.c_float), ("item_alpha", C.c_float), ("rank", C.c_uint32), ("noise", C.c_float), ("mean", C.c_float),
+                ("step", C.c_float), ("lo", C.c_float), ("hi", C.c_float), ("bimodal", C.c_uint32)]
+
+
 class AfpState(C.Structure):
     _fields_ = [("user", AfpQ), ("item", AfpQ), ("backward", AfpQ),
                 ("update_user_params_iter", C.c_int), ("update_item_params_iter", C.c_int),
@@ -65,6 +72,7 @@ class Oracle:
             "orc_group_lookup": (None, [u32, vp, u32, C.POINTER(u32), C.POINTER(u32)]),
             "orc_shuffle_keys": (None, [u64, u64, vp]), "orc_shuffle": (None, [u64, vp, vp, u64]),
             "orc_init_normal": (None, [u64, u64, vp, u64]),
+            "orc_generate_ratings": (None, [vp, u64, u64, u64, vp]),
             "orc_sgd_update": (None, [i32, vp, vp, f32, f32, f32]),
             "orc_mem_quant_update": (None, [i32, vp, vp, f32, f32, f32]),
             "orc_mem_quant_epoch": (None, [i32, vp, u32, vp, vp, u32, u32, u32, f32, f32, u64, u32, vp, i32]),
@@ -145,6 +153,13 @@ class Oracle:
     def shuffle(self, seed, R):
         out = np.empty_like(R)
         self.lib.orc_shuffle(seed, _ptr(R), _ptr(out), R.size)
+        return out
+
+    def generate_ratings(self, cfg, seed, first, count):
+        """Ratings [first, first + count) of the seeded synthetic stream; cfg: any ctypes structure laid out like SynthConfig."""
+        out = np.empty(count, NODE)
+        c = SynthConfig.from_buffer_copy(bytes(cfg))
+        self.lib.orc_generate_ratings(C.addressof(c), seed, first, count, _ptr(out))
         return out
 
     def init_normal(self, seed, stream, n):

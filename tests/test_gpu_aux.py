@@ -264,3 +264,28 @@ def test_row_traffic_probe_leaves_rows_unchanged(row_bytes, coherent):
     with pytest.raises(MfError, match="both keep tables"):
         h.mf_row_traffic_probe(dR.data_ptr(), n, dP.data_ptr(), dQ.data_ptr(), row_bytes, 4, dku.data_ptr(), None, 5, coherent, mfutil.stream_ptr())
     h.mf_row_traffic_probe(None, 0, None, None, row_bytes, 4, None, None, 5, coherent, mfutil.stream_ptr())      # nothing to do
+
+
+@pytest.mark.parametrize("config", [1, 4, 5])
+def test_generated_ratings_match_the_checker(orc, config):
+    """mf_generate_ratings against its CPU twin, bit for bit, on scaled-down BASELINE configurations; any range of the
+    stream can be generated on its own."""
+    import torch
+    from oracle import oracle as om
+    h = mfutil.hip()
+    c = h.synth_config(config)
+    if config != 1:                      # keep the checker's tables small
+        c.n_users, c.n_items = 30_000, 4_000
+    n = 150_000
+    want = orc.generate_ratings(c, 11, 0, n)
+    out = torch.empty(n * 12, dtype=torch.uint8, device="cuda")
+    import ctypes as C
+    h.mf_generate_ratings(C.addressof(c), 11, 0, n, out.data_ptr(), mfutil.stream_ptr())
+    got = from_dev(out, mfutil.NODE)
+    assert np.array_equal(got.view(np.uint8), want.view(np.uint8))
+    part = torch.empty(1000 * 12, dtype=torch.uint8, device="cuda")
+    h.mf_generate_ratings(C.addressof(c), 11, 77_777, 1000, part.data_ptr(), mfutil.stream_ptr())
+    assert np.array_equal(from_dev(part, mfutil.NODE).view(np.uint8), want[77_777:78_777].view(np.uint8))
+    host = np.empty(500, mfutil.NODE)
+    h.mf_generate_ratings_host(C.addressof(c), 11, 10, 500, host.ctypes.data)
+    assert np.array_equal(host.view(np.uint8), want[10:510].view(np.uint8))

@@ -285,3 +285,34 @@ def test_command_line_rating_cache(tmp_path):
     out3, facts3 = run()
     assert "Ratings loaded from" not in out3
     assert facts3 != facts1
+
+
+def test_command_line_synthetic_configuration(orc, tmp_path):
+    """-synth 1: no input files; BASELINE configuration 1 (5000 x 2000, 400k / 100k ratings) is generated on the
+    device, the test set goes through the reference's test-set rules, training reports a falling RMSE and the model
+    file holds one row per id."""
+    assert os.path.exists(CLI), "quantized_mf is not built"
+    out = str(tmp_path / "model")
+    cmd = [CLI, "-synth", "1", "-o", out, "-v", "5", "-k", "64", "-l", "6", "-wg", "0", "-a", "0.01", "-b", "0.05", "-d", "0.1", "-seed", "4"]
+    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=300)
+    assert res.returncode == 0, res.stderr
+    assert "The number of nonzeros      : 400000" in res.stdout
+    assert "The number of users         : 5000" in res.stdout and "The number of items         : 2000" in res.stdout
+    # the same stream from the checker: the test set the command line must have kept
+    from oracle import oracle as om
+    h = mfutil.hip()
+    c = h.synth_config(1)
+    allr = orc.generate_ratings(c, 4, 0, 500_000)
+    train, test = allr[:400_000], allr[400_000:]
+    keep = np.isin(test["u"], train["u"]) & np.isin(test["i"], train["i"])
+    kept = mfutil.test_set_order(test[keep])
+    assert "The number of test nonzeros : %d" % kept.size in res.stdout
+    assert "Missing the number of ratings : %d" % int((~keep).sum()) in res.stdout
+    epochs = [l.split() for l in res.stdout.splitlines() if len(l.split()) == 3 and l.split()[0].isdigit()]
+    rm = np.array([float(l[2]) for l in epochs])
+    assert len(rm) == 6 and rm[-1] < rm[0]
+    rows = open(out + ".txt").read().split("\n")
+    assert rows[0].split() == ["5000", "2000", "64"]
+    P = np.array(rows[1].split(), np.float32).reshape(5000, 64)
+    Q = np.array(rows[2].split(), np.float32).reshape(2000, 64)
+    assert abs(orc.rmse(64, kept, P, Q) - rm[-1]) < 2e-4

@@ -461,3 +461,66 @@ def test_argument_checks_need_no_gpu(lib):
         p = np.zeros(128, np.float32); out = C.c_double(0)
         lib.call("mf_gpu_test_rmse", node.ctypes.data, 1, p.ctypes.data, p.ctypes.data, 1, 1, 128, C.byref(out))
     assert lib.mf_set_row_coherence(1) == 0 and lib.mf_get_row_coherence() == 1
+
+
+# ---- seeded synthetic ratings (the generator behind `quantized_mf -synth`) ------------------------------------------
+def _zipf_share(count, alpha, rank):
+    w = np.arange(1, count + 1, dtype=np.float64) ** -alpha
+    return w[rank] / w.sum()
+
+
+def test_generated_ratings_follow_the_stated_distribution(orc):
+    """Pins the generator's CPU twin against what it claims: Zipf popularity over a permutation of the ids, ratings on
+    the grid, a low-rank signal under the noise, and rating j depending on (seed, j) only."""
+    from oracle import oracle as om
+    c = om.SynthConfig(3000, 800, 0, 0, 0.9, 1.1, 8, 0.8, 3.5, 0.5, 0.5, 5.0, 0)
+    n = 600_000
+    R = orc.generate_ratings(c, 5, 0, n)
+    assert R["u"].max() < 3000 and R["i"].max() < 800
+    assert np.array_equal(np.unique(R["r"]), np.arange(1, 11) * 0.5)               # the 0.5 .. 5.0 grid, nothing else
+    for ids, count, alpha in ((R["u"], 3000, 0.9), (R["i"], 800, 1.1)):
+        cnt = np.sort(np.bincount(ids, minlength=count))[::-1].astype(np.float64)
+        for rank in (0, 1, 9, 99):                                                   # binomial, 5 sigma
+            p = _zipf_share(count, alpha, rank)
+            assert abs(cnt[rank] - n * p) < 5 * np.sqrt(n * p) + 0.02 * n * p, (rank, cnt[rank], n * p)
+        slope = np.polyfit(np.log(np.arange(1, 101)), np.log(cnt[:100]), 1)[0]
+        assert abs(slope + alpha) < 0.05
+        top = np.argsort(np.bincount(ids, minlength=count))[::-1][:20]
+        assert not np.array_equal(np.sort(top), np.arange(20))                      # popularity is not in id order
+    # the truth is low rank: the per-(user, item) means of repeated pairs vary far more than noise / sqrt(repeats) would
+    key = R["u"].astype(np.int64) * 800 + R["i"]
+    order = np.argsort(key, kind="stable")
+    k_sorted, r_sorted = key[order], R["r"][order].astype(np.float64)
+    uniq, start, reps = np.unique(k_sorted, return_index=True, return_counts=True)
+    many = reps >= 30
+    means = np.add.reduceat(r_sorted, start)[many] / reps[many]
+    assert many.sum() > 50 and means.std() > 3 * 0.8 / np.sqrt(30)
+    # any range on its own; another seed gives other ratings
+    assert np.array_equal(orc.generate_ratings(c, 5, 123_456, 777).view(np.uint8), R[123_456:124_233].view(np.uint8))
+    assert not np.array_equal(orc.generate_ratings(c, 6, 0, 1000).view(np.uint8), R[:1000].view(np.uint8))
+
+
+def test_generated_bimodal_ratings(orc):
+    from oracle import oracle as om
+    c = om.SynthConfig(500, 300, 0, 0, 1.2, 1.2, 0, 15.0, 0.0, 1.0, 0.0, 100.0, 1)
+    R = orc.generate_ratings(c, 9, 0, 200_000)
+    raw = np.round((R["r"].astype(np.float64) - 1.0) / 0.04)                          # back to 0..100
+    assert raw.min() >= 0 and raw.max() <= 100 and np.allclose((raw * 0.04 + 1.0).astype(np.float32), R["r"])
+    low, high = raw[raw < 50], raw[raw >= 50]
+    assert abs(low.size / raw.size - 0.5) < 0.01
+    # clamping at 0 / 100 (9 % of each mode) pulls the means about 0.5 inwards and the deviations to about 13
+    assert abs(low.mean() - 20.5) < 0.5 and abs(high.mean() - 79.5) < 0.5
+    assert 12 < low.std() < 15 and 12 < high.std() < 15
+
+
+def test_synth_baseline_configs():
+    """mf_synth_baseline_config: the five shapes (users, items, training and test ratings) of BASELINE.json's configurations."""
+    capi = importlib.import_module("icdm-2021_mascot_amd.capi")
+    h = capi.load()
+    sizes = {1: (5000, 2000, 400_000, 100_000), 2: (70_000, 10_700, 8_000_000, 2_000_000), 3: (162_000, 59_000, 20_000_000, 5_000_000),
+             4: (480_000, 17_800, 100_000_000, 1_400_000), 5: (1_000_000, 625_000, 250_000_000, 4_000_000)}
+    for cfg, (nu, ni, ntr, nte) in sizes.items():
+        c = h.synth_config(cfg)
+        assert (c.n_users, c.n_items, c.n_train, c.n_test) == (nu, ni, ntr, nte)
+    with pytest.raises(capi.MfError, match="numbered 1..5"):
+        h.synth_config(6)
