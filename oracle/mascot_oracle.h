@@ -11,6 +11,11 @@
  *     unseeded (clock()/time(0) seeds, cuRAND XORWOW), so these restate this
  *     build's own seeded generators, not the reference's streams.
  *     parity unpinned (by construction; only the index mapping is closed form).
+ *   - orc_generate_ratings: synthetic data has no counterpart in the reference
+ *     (its data sets are downloaded); this is the twin of the build's own
+ *     generator.  parity unpinned against the reference by construction; the
+ *     distribution it claims (Zipf marginals, rating grid, low-rank signal,
+ *     range independence) is pinned in tests/test_oracle_host.py.
  *   - MuPPET / AFP: floor/ceil(log2f(x)) for x within one ulp of a power of
  *     two, and float -> int8 conversion of values outside [-128,127], depend on
  *     CUDA's libdevice / cvt behaviour.  parity unpinned for those inputs.
