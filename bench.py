@@ -332,9 +332,9 @@ def measured_traffic(a, leg):
     if a.config != 4 or a.k != 128 or a.ratings != 100_000_000 or a.seed != 2021:
         return None
     if a.skip_coherent:
-        return (14_008_952 * 2.0 + 24_135_386) * 1024 if leg["workers"] == 16384 else None
+        return (13_996_993 * 2.0 + 24_209_347) * 1024 if leg["workers"] == 16384 else None
     if leg["workers"] == 6104 and a.hot_row_inflight == 2.0 and a.warmup >= a.hot_row_early_epochs:
-        return (15_955_472 * 2.0 + 27_558_058) * 1024
+        return (15_952_590 * 2.0 + 27_557_537) * 1024
     return None
 
 
