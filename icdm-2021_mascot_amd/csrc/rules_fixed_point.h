@@ -109,10 +109,8 @@ template <int K, bool COH> struct MuppetRule : DenseBase<K, COH> {
     using typename Base::Info;
     static constexpr int E = Base::E;
     static constexpr int J = K / 32;
-    // One rating of look-ahead: every race on a row is resolved last-writer-wins here (the plain store() below), and
-    // each further rating a wavefront has in flight loses more updates of the popular rows.  Measured at 100M
-    // ratings: three ratings ahead leave MuPPET's epoch unchanged (bound by its arithmetic), make AFP's 11 % shorter
-    // and cost both 0.006 to 0.015 of test RMSE after four epochs.
+    // One rating of look-ahead: the rule is bound by its arithmetic, and three ratings in flight per wavefront measured
+    // slower (the longer register ring costs more than the loads' latency, which the other wavefronts already cover).
     static constexpr int kAhead = 1, kRing = 4;
     struct Params {
         float* p; float* q; float lrate; float lambda; uint32_t first_sample;
@@ -213,12 +211,15 @@ template <int K, bool COH> struct MuppetRule : DenseBase<K, COH> {
                 gq[e] = (float)(half_t)(ph * t_ruv + qh * t_lam);
             }
         }
+        float dp[E], dq[E];
 #pragma unroll
         for (int e = 0; e < E; ++e) {
-            row.p[e] = row.p[e] + lrate * gp[e];
-            row.q[e] = row.q[e] + lrate * gq[e];
+            dp[e] = lrate * gp[e];
+            dq[e] = lrate * gq[e];
+            row.p[e] = (i.thin & 1u) ? row.p[e] : row.p[e] + dp[e];
+            row.q[e] = (i.thin & 2u) ? row.q[e] : row.q[e] + dq[e];
         }
-        this->store(row, i);
+        this->template store<HOT>(row, i, dp, dq);
         if (fwd != 32 && bwd != 32 && processed >= first_sample) {
             float sp2[E], sq2[E];
 #pragma unroll
@@ -274,7 +275,7 @@ template <int K, bool COH> struct AfpRule : DenseBase<K, COH> {
     using typename Base::Info;
     static constexpr int E = Base::E;
     static constexpr int J = K / 32;
-    static constexpr int kAhead = 1, kRing = 4;
+    static constexpr int kAhead = 1, kRing = 4;    // as for MuPPET: three ratings ahead measured no faster (k = 128) or slower (k = 64)
     static constexpr bool kSplittable = false;    // the per-worker quantiser state lives for one launch
     struct Params { float* p; float* q; float lrate; float lambda; int afp_epoch; int init_threshold; bool accumulate; };
     float lrate, lambda; int afp_epoch, init_threshold;
@@ -395,12 +396,15 @@ template <int K, bool COH> struct AfpRule : DenseBase<K, COH> {
                 gq[e] = (float)(half_t)(ph * t_ruv + qh * t_lam);
             }
         }
+        float dp[E], dq[E];
 #pragma unroll
         for (int e = 0; e < E; ++e) {
-            row.p[e] = row.p[e] + lrate * gp[e];
-            row.q[e] = row.q[e] + lrate * gq[e];
+            dp[e] = lrate * gp[e];
+            dq[e] = lrate * gq[e];
+            row.p[e] = (i.thin & 1u) ? row.p[e] : row.p[e] + dp[e];
+            row.q[e] = (i.thin & 2u) ? row.q[e] : row.q[e] + dq[e];
         }
-        this->store(row, i);
+        this->template store<HOT>(row, i, dp, dq);
         cur_iter += 1;
     }
     __device__ __forceinline__ void finish(const Params&, uint32_t) const {}

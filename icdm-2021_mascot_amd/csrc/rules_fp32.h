@@ -78,20 +78,6 @@ template <int K, bool COH> struct DenseBase {
             }
         }
     }
-    // rules that keep last-writer-wins on every row
-    __device__ __forceinline__ void store(const Row& row, const Info& i) const
-    {
-        float* pp = P + (size_t)i.u * K + lane;
-        float* qq = Q + (size_t)i.v * K + lane;
-        if (!(i.thin & 1u)) {
-#pragma unroll
-            for (int e = 0; e < E; ++e) row_store<COH>(pp + 64 * e, row.p[e]);
-        }
-        if (!(i.thin & 2u)) {
-#pragma unroll
-            for (int e = 0; e < E; ++e) row_store<COH>(qq + 64 * e, row.q[e]);
-        }
-    }
     __device__ __forceinline__ void forward(Row& nxt, const Info& in, const Row& cur, const Info& ic) const
     {
         if (in.u == ic.u) {

@@ -271,7 +271,7 @@ int train_dense(Common& c, float* p, float* q)
     if (version == 8) MF_TRY(whole.init(c, d_p.as<float>(), d_q.as<float>(), prm.num_workers));
 
     HotRows hot;
-    if (prm.hot_row_inflight > 0 && (version == 5 || version == 4 || version == 7 || version == 8)) {
+    if (prm.hot_row_inflight > 0) {
         DevBuf d_ucnt, d_icnt;
         MF_TRY(d_ucnt.alloc((size_t)c.n_users * 4, "hipMalloc(user counts)"));
         MF_TRY(d_icnt.alloc((size_t)c.n_items * 4, "hipMalloc(item counts)"));

@@ -57,7 +57,7 @@ int mf_get_row_coherence(void);
  * Default 1.  No counterpart in the reference. */
 int mf_set_epoch_splits(uint32_t splits);
 uint32_t mf_get_epoch_splits(void);
-/* Hot rows for the fp32-SGD / MPT / MASCOT update calls (process-wide, both NULL = off, the default).
+/* Hot rows for the update calls (process-wide, both NULL = off, the default).
  * user_keep[row], item_keep[row] are device arrays of bytes indexed like P and Q rows (for MASCOT: sorted row
  * order).  255 marks an ordinary row.  A row with a smaller value is a hot row, meant for rows that have several
  * updates in flight at any time: (1) a rating updates the row with probability (keep+1)/255 and otherwise only
@@ -65,7 +65,7 @@ uint32_t mf_get_epoch_splits(void);
  * (an atomic add per element) instead of storing the new row, so concurrent updates add up where
  * last-writer-wins would keep one of them.  The sum of C stale gradients is a step C times as long, which is why
  * rows with many updates in flight are thinned.  mf_train builds the tables from the rating counts when
- * mf_params.hot_row_inflight > 0 (MuPPET and AFP ignore them).  No counterpart in the reference.  The tables must
+ * mf_params.hot_row_inflight > 0.  No counterpart in the reference.  The tables must
  * stay valid while launches that use them are in flight. */
 int mf_set_hot_row_thinning(const uint8_t* user_keep, const uint8_t* item_keep);
 /* Seeded synthetic ratings (no counterpart in the reference, whose data sets are downloaded): users and items are
