@@ -106,8 +106,15 @@ __device__ __forceinline__ void process_full_chunk(Rule& rule, const Rating& my,
     });
 }
 
+// A rule may ask for a minimum number of resident wavefronts per SIMD (kMinWavesPerSimd): the compiler then keeps the
+// kernel's registers within 512 / that many.  For rules whose natural allocation lands just above a step (85 VGPRs
+// is 5 wavefronts per SIMD, 80 is 6) this decides whether all workers of a launch are resident at once.
+template <class Rule, class = void> struct min_waves_per_simd { static constexpr int value = 1; };
+template <class Rule> struct min_waves_per_simd<Rule, std::void_t<decltype(Rule::kMinWavesPerSimd)>> { static constexpr int value = Rule::kMinWavesPerSimd; };
+
 template <class Rule, bool HOT>
-__global__ __launch_bounds__(kMaxBlock) void hogwild_kernel(Schedule s, typename Rule::Params prm)
+__global__ __launch_bounds__(kMaxBlock) __attribute__((amdgpu_waves_per_eu(min_waves_per_simd<Rule>::value)))
+void hogwild_kernel(Schedule s, typename Rule::Params prm)
 {
     extern __shared__ __align__(16) uint8_t smem[];
     const int lane = threadIdx.x & (kWave - 1);
