@@ -365,8 +365,8 @@ def main():
     ap.add_argument("--seed", type=int, default=2021)
     a = ap.parse_args()
     if a.gpus != 1:
-        print("bench.py: this build runs on one GPU only (every box has one; the multi-GPU sharding is a design note "
-              "in DESIGN.md); run with --gpus 1", file=sys.stderr)
+        print("bench.py: this build runs on one GPU only (one process, one device; sharding over several GPUs is a design "
+              "note, not code); run with --gpus 1", file=sys.stderr)
         sys.exit(2)
     import torch
     h = importlib.import_module("icdm-2021_mascot_amd").load()
@@ -452,7 +452,7 @@ def main():
     if not a.skip_cached:
         c = leg(False, a.cached_workers)
         out["cached_rows"] = {"note": "same workload with ordinary cached row accesses (each XCD trains its own L2-resident copy of hot "
-                                      "rows; faster, converges worse, see DESIGN.md); its algorithmic bytes can exceed the HBM peak because "
+                                      "rows; faster, converges worse); its algorithmic bytes can exceed the HBM peak because "
                                       "hot rows are served and overwritten in L2 without reaching memory",
                               "value": c["ratings_per_s"], "unit": "ratings/s", "ms_per_step": c["ms_per_step"], "workers": c["workers"],
                               "roofline": {"bound": "hbm", "achieved": c["gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": c["gbs"] / PEAK_HBM_GBS,
