@@ -142,13 +142,12 @@ class MascotProblem:
         """Hot-row tables from the rating counts (rows are in popularity-sorted order), as mf_train builds them:
         255 = ordinary row; rows with more than one update in flight are hot rows (updates added in memory), thinned to
         at most `inflight_cap` updates in flight.  Returns (user table, item table, fraction of row updates carried out)."""
-        F = min(W, 8192) * 4.0
         tabs, kept = [], 0.0
         for s in self.sides:
-            inflight = F * s["sorted_cnt"].astype(np.float64) / self.n
-            keep = np.where(inflight > inflight_cap, inflight_cap / np.maximum(inflight, 1e-30), 1.0)
-            t = np.where(inflight > 1.0, np.clip(np.floor(keep * 255.0) - 1, 0, 254), 255).astype(np.uint8)
-            kept += float((s["sorted_cnt"].astype(np.float64) * np.where(t == 255, 1.0, (t.astype(np.float64) + 1) / 255.0)).sum()) / self.n
+            cnt = np.ascontiguousarray(s["sorted_cnt"], np.uint32)
+            t = np.empty(cnt.size, np.uint8)
+            self.h.mf_hot_row_table(cnt.ctypes.data, cnt.size, self.n, W, inflight_cap, t.ctypes.data)
+            kept += float((cnt.astype(np.float64) * np.where(t == 255, 1.0, (t.astype(np.float64) + 1) / 255.0)).sum()) / self.n
             tabs.append(self.torch.from_numpy(t).to(self.R.device))
         return tabs[0], tabs[1], kept / 2
 

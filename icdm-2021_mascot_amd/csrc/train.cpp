@@ -699,6 +699,17 @@ int mf_gpu_test_rmse(const mf_node* test, uint32_t test_n, const float* p, const
     return MF_OK;
 }
 
+int mf_hot_row_table(const uint32_t* counts, uint32_t rows, uint32_t n, uint32_t num_workers, float inflight_cap, uint8_t* table)
+{
+    if (rows == 0) return MF_OK;
+    if (!counts || !table) return invalid("mf_hot_row_table: null pointer");
+    if (n == 0 || num_workers == 0) return invalid("mf_hot_row_table: no ratings or no workers");
+    if (!(inflight_cap > 0)) return invalid("mf_hot_row_table: the cap must be positive");
+    const std::vector<uint8_t> t = keep_table(counts, rows, n, num_workers, inflight_cap);
+    std::memcpy(table, t.data(), rows);
+    return MF_OK;
+}
+
 uint32_t mf_auto_workers(uint32_t n)
 {
     // about 128 windows of 128 ratings per worker: the ratio at which the runs on 8M and on 100M ratings stay

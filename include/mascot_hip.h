@@ -68,6 +68,11 @@ uint32_t mf_get_epoch_splits(void);
  * mf_params.hot_row_inflight > 0.  No counterpart in the reference.  The tables must
  * stay valid while launches that use them are in flight. */
 int mf_set_hot_row_thinning(const uint8_t* user_keep, const uint8_t* item_keep);
+/* The table mf_train builds for one side (host arrays): counts[row] ratings of `n` fall on the row; with
+ * F = min(num_workers, 8192) * 4 updates in flight on the device a row has about F * counts[row] / n of them.
+ * Rows with at most one stay ordinary (255); the others become hot rows, kept with probability
+ * min(1, inflight_cap / in flight): table value clip(floor(keep * 255) - 1, 0, 254). */
+int mf_hot_row_table(const uint32_t* counts, uint32_t rows, uint32_t n, uint32_t num_workers, float inflight_cap, uint8_t* table);
 /* Seeded synthetic ratings (no counterpart in the reference, whose data sets are downloaded): users and items are
  * drawn independently from Zipf(alpha) over a random permutation of the ids; a rating is
  * clamp(round_to_step(U_u . V_i + mean + noise * N(0,1)), lo, hi) with rank-`rank` factors U, V ~ N(0, 0.5^2), or,
