@@ -99,3 +99,12 @@ def test_many_rows_are_written_in_order(driver, tmp_path):
     head, body_p, body_q = open(out + "_reconst.txt").read().split("\n")
     assert head == "%d %d %d" % (n_users, n_items, k)
     assert body_p == "".join(c_format(v) + " " for v in P)
+
+
+def test_round_half_away_identity_is_exhaustive(tmp_path):
+    """The fixed-point kernels round with trunc(x + copysign(pred(0.5), x)); the reference calls roundf.  All 2^32 bit
+    patterns agree."""
+    exe = str(tmp_path / "round_identity_check")
+    subprocess.run(["gcc", "-O2", "-fopenmp", "-ffp-contract=off", "-o", exe, os.path.join(ROOT, "tests", "round_identity_check.c"), "-lm"], check=True)
+    r = subprocess.run([exe], capture_output=True, text=True, timeout=600)
+    assert r.returncode == 0 and r.stdout.strip() == "0", r.stdout + r.stderr
