@@ -226,11 +226,14 @@ template <int K, bool COH, bool SAMPLED> struct MascotRuleT {
     static __device__ __forceinline__ float dot_float(const float* m)
     {
         if constexpr (E == 2) {
-            float a = m[0], b = m[1];
-            a = step_xor16(a, OpAdd()); b = step_xor16(b, OpAdd());
-            a = step_xor32(a, OpAdd()); b = step_xor32(b, OpAdd());
-            a = reduce_row16(a, OpAdd()); b = reduce_row16(b, OpAdd());
-            return a + b;
+            // both element sums in one register: v_permlane16_swap(a, b) leaves [a.r0 b.r0 a.r2 b.r2] and
+            // [a.r1 b.r1 a.r3 b.r3], whose sum is the lane ^ 16 step of a in rows 0, 2 and of b in rows 1, 3; the
+            // lane ^ 32 step and the rotations inside the rows follow as for one value, a + b is the last step
+            auto ab = __builtin_amdgcn_permlane16_swap(bits(m[0]), bits(m[1]), false, false);
+            float s = from_bits<float>(ab[0]) + from_bits<float>(ab[1]);
+            s = step_xor32(s, OpAdd());
+            s = reduce_row16(s, OpAdd());
+            return step_xor16(s, OpAdd());
         } else {
             return reduce_wave(m[0], OpAdd());
         }

@@ -251,15 +251,21 @@ template <int K, bool COH> struct MemQuantRule {
             }
         }
     }
-    // ((row 0 + row 1) + row 2) + row 3 of the wavefront's four rows of 16 lanes, in every lane
-    static __device__ __forceinline__ float sum_rows_in_order(float x)
+    // The dot product at k = 128 from the products of the even (x) and odd (y) elements of every lane.  Per 16-lane
+    // position the four rows are summed in order, ((row 0 + row 1) + row 2) + row 3, x in the lower half-wave and y in
+    // the upper one at the same time: v_permlane32_swap(x, y) leaves [x.rows01, y.rows01] and [x.rows23, y.rows23],
+    // v_permlane16_swap of each with itself spreads its even and its odd row.  Then the tree inside the rows
+    // (rotations by 8, 4, 2, 1) and the last step, even + odd, across the half-waves.
+    static __device__ __forceinline__ float dot_rows_in_order(float x, float y)
     {
-        auto halves = __builtin_amdgcn_permlane32_swap(bits(x), bits(x), false, false);      // [0]: rows 0 1 0 1, [1]: rows 2 3 2 3
-        auto lo = __builtin_amdgcn_permlane16_swap(halves[0], halves[0], false, false);      // [0]: row 0 everywhere, [1]: row 1
-        auto hi = __builtin_amdgcn_permlane16_swap(halves[1], halves[1], false, false);      // [0]: row 2 everywhere, [1]: row 3
+        auto halves = __builtin_amdgcn_permlane32_swap(bits(x), bits(y), false, false);
+        auto lo = __builtin_amdgcn_permlane16_swap(halves[0], halves[0], false, false);      // [0]: rows 0 0 | 0 0 of x | y, [1]: rows 1
+        auto hi = __builtin_amdgcn_permlane16_swap(halves[1], halves[1], false, false);      // [0]: rows 2, [1]: rows 3
         float s = from_bits<float>(lo[0]) + from_bits<float>(lo[1]);
         s = s + from_bits<float>(hi[0]);
-        return s + from_bits<float>(hi[1]);
+        s = s + from_bits<float>(hi[1]);
+        s = reduce_row16(s, OpAdd());
+        return step_xor32(s, OpAdd());
     }
     template <int CLS, bool HOT> __device__ __forceinline__ void update(Row& row, const Info& i, uint32_t) const
     {
@@ -269,9 +275,7 @@ template <int K, bool COH> struct MemQuantRule {
         if constexpr (E == 1) {
             dot = reduce_wave(pf[0] * qf[0], OpAdd());                // k = 64: p1*q1 + p2*q2, then the tree
         } else {
-            const float even = reduce_row16(sum_rows_in_order(pf[0] * qf[0]), OpAdd());
-            const float odd = reduce_row16(sum_rows_in_order(pf[1] * qf[1]), OpAdd());
-            dot = even + odd;
+            dot = dot_rows_in_order(pf[0] * qf[0], pf[1] * qf[1]);
         }
         const float ruv = i.r - dot;
         float dp[E], dq[E], np[E], nq[E];
