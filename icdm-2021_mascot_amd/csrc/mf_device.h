@@ -46,8 +46,6 @@ template <int N, class T> __device__ __forceinline__ T row_ror(T x)
 
 // Reduction steps: every lane ends with op(own, partner); op must be commutative.
 struct OpAdd { template <class T> __device__ __forceinline__ T operator()(T a, T b) const { return a + b; } };
-struct OpMin { __device__ __forceinline__ float operator()(float a, float b) const { return fminf(a, b); } };
-struct OpMax { __device__ __forceinline__ float operator()(float a, float b) const { return fmaxf(a, b); } };
 
 template <class T, class Op> __device__ __forceinline__ T step_xor32(T x, Op op)
 {
