@@ -178,6 +178,8 @@ def test_mascot_group_table_sizes(orc, k):
     # one group per side, and more groups than a 64-lane compare could hold
     _mascot_case(orc, k, 4, 1, 128, 1, 1, "half", first_sample=128, seed=61)
     _mascot_case(orc, k, 40, 1, 64, 150, 101, "mixed", first_sample=0, seed=62)
+    # more groups than the sampled sums have room for in LDS: the whole epoch runs with the sums in global memory
+    _mascot_case(orc, k, 100, 1, 64, 400, 350, "mixed", first_sample=10, seed=63)
 
 
 @pytest.mark.parametrize("k", [64, 128])
