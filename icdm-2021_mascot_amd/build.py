@@ -23,7 +23,8 @@ ARCH = "gfx950"
 DEVICE_FLAGS = ["--offload-arch=" + ARCH, "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off", "-munsafe-fp-atomics",
                 "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
                 "-Xclang", "-target-feature", "-Xclang", "-fma-mix-insts", "-Wall", "-Wno-unused-function"]
-KERNEL_SOURCES = ["hogwild_launch.hip", "aux_kernels.hip", "sort_shuffle.hip"]
+KERNEL_SOURCES = ["launch_mascot_plain.hip", "launch_mascot_sampled.hip", "launch_muppet.hip", "launch_afp.hip", "hogwild_launch.hip", "launch_mem_quant.hip", "aux_kernels.hip",
+                  "sort_shuffle.hip", "launch_mascot.hip"]
 HOST_SOURCES = ["train.cpp"]
 CLI_SOURCES = ["main.cpp", "io_utils.cpp"]
 EVAL_SOURCES = ["test_mf_main.cpp", "io_utils.cpp"]
@@ -47,7 +48,7 @@ def _compile(src):
 def build(verbose=False):
     os.makedirs(OBJ, exist_ok=True)
     lib_sources = [s for s in KERNEL_SOURCES + HOST_SOURCES if os.path.exists(os.path.join(CSRC, s))]
-    with ThreadPoolExecutor(max_workers=4) as ex:
+    with ThreadPoolExecutor(max_workers=8) as ex:
         objs = list(ex.map(_compile, lib_sources))
     _run([HIPCC, "--offload-arch=" + ARCH, "-shared", "-fPIC", "-o", LIB] + objs)
     if all(os.path.exists(os.path.join(CSRC, s)) for s in CLI_SOURCES):
