@@ -297,6 +297,66 @@ def time_fp32_sgd(torch, h, prob, W, warmup, steps, cfg, seed):
     return np.array([a.elapsed_time(b) for a, b in ev]), uc, rmse, float(np.mean(kept))
 
 
+def time_every_rule(torch, h, prob, W, cfg, seed, epochs=6):
+    """Every update kernel on the same ratings, workers and hot-row schedule (dense P and Q in the rule's storage format):
+    mean time of the steady plain epochs 2..epochs-1 and the test RMSE after `epochs` epochs, with the access-pattern
+    probe of the rule's row size beside it."""
+    dev, k, st = prob.R.device, prob.k, torch.cuda.current_stream().cuda_stream
+    uc = h.mf_update_count(prob.n, W, 128)
+    lr = lambda e: h.mf_lr_schedule(cfg["lr"], cfg["decay"], e)
+    lam_h = int(np.array([np.float32(cfg["lam"]) * np.float32(1000.0)], np.float32).astype(np.float16).view(np.uint16)[0])
+    R, n = prob.R.data_ptr(), prob.n
+    sums = torch.zeros(k, dtype=torch.float32, device=dev)
+    norms = torch.zeros(W, dtype=torch.float32, device=dev)
+    rules = {
+        "fp32_sgd": (4, lambda P, Q, e: h.mf_single_sgd_hogwild(R, n, P, Q, k, W, uc, 128, lr(e), cfg["lam"], seed, e, None, st)),
+        "mpt": (4, lambda P, Q, e: h.mf_mpt_sgd_hogwild(R, n, P, Q, k, W, uc, 128, lr(e), lam_h, 1000.0, seed, e, None, st)),
+        "muppet_8bit": (4, lambda P, Q, e: h.mf_muppet_sgd_hogwild(R, n, P, Q, k, W, uc, 128, lr(e), cfg["lam"], uc * 128, sums.data_ptr(),
+                                                                  norms.data_ptr(), 8, 8, seed, e, None, st)),
+        "muppet_16bit": (4, lambda P, Q, e: h.mf_muppet_sgd_hogwild(R, n, P, Q, k, W, uc, 128, lr(e), cfg["lam"], uc * 128, sums.data_ptr(),
+                                                                   norms.data_ptr(), 16, 16, seed, e, None, st)),
+        "afp": (4, lambda P, Q, e: h.mf_afp_sgd_hogwild(R, n, P, Q, k, W, uc, 128, lr(e), cfg["lam"], e, seed, e, None, st)),
+        "mem_quant": (2, lambda P, Q, e: h.mf_mem_quant_sgd_hogwild(R, n, P, Q, k, W, uc, 128, lr(e), cfg["lam"], seed, e, None, st)),
+    }
+    out, ceilings = {}, {}
+    steady = prob.hot["steady"] if prob.hot else None
+    for name, (elem, call) in rules.items():
+        P32 = torch.empty(prob.n_users * k, dtype=torch.float32, device=dev)
+        Q32 = torch.empty(prob.n_items * k, dtype=torch.float32, device=dev)
+        h.mf_init_rand_feature(P32.data_ptr(), P32.numel(), seed, 0, st)
+        h.mf_init_rand_feature(Q32.data_ptr(), Q32.numel(), seed, 1, st)
+        P, Q = P32, Q32
+        if elem == 2:
+            P, Q = torch.empty(P32.numel(), dtype=torch.float16, device=dev), torch.empty(Q32.numel(), dtype=torch.float16, device=dev)
+            h.mf_transform_float2half(P32.data_ptr(), P.data_ptr(), P32.numel(), st)
+            h.mf_transform_float2half(Q32.data_ptr(), Q.data_ptr(), Q32.numel(), st)
+        ms = []
+        for e in range(epochs):
+            prob.select_hot_rows(e)
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record(); call(P.data_ptr(), Q.data_ptr(), e); b.record()
+            torch.cuda.synchronize()
+            ms.append(a.elapsed_time(b))
+        if elem == 2:
+            h.mf_transform_half2float(P.data_ptr(), P32.data_ptr(), P32.numel(), st)
+            h.mf_transform_half2float(Q.data_ptr(), Q32.data_ptr(), Q32.numel(), st)
+        acc = torch.zeros(1, dtype=torch.float64, device=dev)
+        h.mf_test_rmse(prob.test.data_ptr(), prob.test.shape[0], P32.data_ptr(), Q32.data_ptr(), k, acc.data_ptr(), st)
+        row_bytes = k * elem
+        if row_bytes not in ceilings:
+            ku, kv = (steady[0].data_ptr(), steady[1].data_ptr()) if steady else (None, None)
+            probe = lambda: h.mf_row_traffic_probe(R, n, P.data_ptr(), Q.data_ptr(), row_bytes, W, ku, kv, seed, h.mf_get_row_coherence(), st)
+            probe(); torch.cuda.synchronize()
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record(); probe(); probe(); b.record(); torch.cuda.synchronize()
+            ceilings[row_bytes] = a.elapsed_time(b) / 2
+        steady_ms = float(np.mean(ms[2:]))
+        out[name] = {"ms_per_epoch": steady_ms, "row_bytes": row_bytes, "access_pattern_ceiling_ms": ceilings[row_bytes],
+                     "kernel_vs_ceiling": ceilings[row_bytes] / steady_ms, "test_rmse": float(np.sqrt(acc.item() / prob.test.shape[0])), "epochs": epochs}
+        del P, Q, P32, Q32
+    return out
+
+
 def reference_rule_rmse(prob, h, cfg, seed, threads, epochs, workers):
     """Test RMSE of the reference update rule (the checker's MASCOT epoch as an OpenMP Hogwild loop, `threads` updates
     in flight) after `epochs` epochs on the same shuffled ratings, initial model, schedule and learning rates."""
@@ -359,6 +419,8 @@ def main():
                     help="profiling aid: also run three 1 GiB device copies, the known-size kernel that FETCH_SIZE / WRITE_SIZE are scaled by")
     ap.add_argument("--skip-fp32", action="store_true", help="skip the fp32-SGD leg")
     ap.add_argument("--skip-ceiling", action="store_true", help="skip the access-pattern probe")
+    ap.add_argument("--every-rule", action="store_true",
+                    help="also time every update kernel (fp32 SGD, MPT, MuPPET, AFP, mem_quant) for six epochs on the same workload")
     ap.add_argument("--reference-rmse", action="store_true",
                     help="also train with the reference rule on the CPU for warmup+steps epochs (minutes) and report the test RMSE delta")
     ap.add_argument("--seed", type=int, default=2021)
@@ -469,6 +531,11 @@ def main():
                            "value": a.ratings / (ms / 1e3), "unit": "ratings/s", "ms_per_step": ms, "workers": a.workers,
                            "roofline_frac": a.workers * uc * 128 * bpu / (ms / 1e3) / 1e9 / PEAK_HBM_GBS,
                            "test_rmse_after_timed_epochs": rmse, "mascot_speedup": ms / main_leg["ms_per_step"]}
+    if a.every_rule and not a.skip_coherent:
+        h.mf_set_row_coherence(1)
+        prob.set_hot_rows(a.workers, a.hot_row_inflight, a.hot_row_inflight_early, a.hot_row_early_epochs)
+        out["every_rule"] = time_every_rule(torch, h, prob, a.workers, cfg, a.seed)
+        prob.set_hot_rows(a.workers, 0.0)
     if a.reference_rmse:
         threads = min(os.cpu_count() or 1, 16)
         ref = reference_rule_rmse(prob, h, cfg, a.seed, threads, a.warmup + a.steps, a.workers)
