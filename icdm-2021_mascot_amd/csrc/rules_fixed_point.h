@@ -33,10 +33,27 @@ __device__ __forceinline__ int f2i_sat(float f)
     const int r = (int)__builtin_amdgcn_fmed3f(f, -2147483648.0f, 2147483520.0f);
     return (f != f) ? 0 : (f >= 2147483648.0f ? 2147483647 : r);
 }
-__device__ __forceinline__ int f2i8_sat(float f)
+// The hardware's own float-to-integer conversions truncate, saturate and map NaN to 0, which is what CUDA's casts do;
+// spelled as instructions because an out-of-range cast has no defined value in C++.
+// The compiler's hazard bookkeeping does not look inside an asm statement, so each one is self-contained: its input
+// comes from an ordinary VALU instruction (an add, a minimum), its result goes to one, and the one wait state a
+// transcendental's result needs before another VALU instruction reads it is spelled out.
+__device__ __forceinline__ int hw_cvt_i32(float f) { int r; asm("v_cvt_i32_f32_e32 %0, %1" : "=v"(r) : "v"(f)); return r; }
+// (unsigned)floorf(log2f(x)) for x that is not subnormal: the conversion truncates, and negative logarithms and NaN
+// give 0 with or without the floor
+__device__ __forceinline__ uint32_t floor_log2_u32(float x)
 {
-    const int r = (int)__builtin_amdgcn_fmed3f(f, -128.0f, 127.0f);
-    return (f != f) ? 0 : r;
+    uint32_t r;
+    asm("v_log_f32_e32 %0, %1\n\ts_nop 0\n\tv_cvt_u32_f32_e32 %0, %0" : "=v"(r) : "v"(x));
+    return r;
+}
+// (signed char) of roundf(x), saturating, NaN -> 0: the conversion truncates by itself, so round_half_away's own
+// truncation is not needed, and clamping the integer afterwards equals clamping the float before (four instructions
+// where rounding, clamping, converting and the NaN select took seven)
+__device__ __forceinline__ int round_to_i8(float x)
+{
+    const int v = hw_cvt_i32(x + __builtin_copysignf(0x1.fffffep-2f, x));
+    return v < -128 ? -128 : (v > 127 ? 127 : v);
 }
 // 2^n for an integer-valued exponent, exact (exp2f of an integer in the reference).
 __device__ __forceinline__ float pow2u(uint32_t n) { return __builtin_ldexpf(1.0f, n > 1000u ? 1000 : (int)n); }
@@ -106,7 +123,9 @@ __device__ __forceinline__ uint32_t muppet_scale_index_by_rows(unsigned bitwidth
     const float ratio = fabsf(bound / extreme);                                        // |min_val / min| = |min_val / -min|
     const float range_best = step_xor32(ratio, OpMinimum());
     const bool both_zero = step_xor32(fabsf(extreme), OpMaximum()) == 0.0f;
-    return both_zero ? 0u : f2u_sat(floorf(__builtin_log2f(range_best)));
+    // x is never subnormal (|bound| >= 127.5 over a finite extreme), so the bare v_log_f32 equals log2f
+    const uint32_t idx = floor_log2_u32(range_best);
+    return both_zero ? 0u : idx;
 }
 
 template <int K, bool COH> struct MuppetRule : DenseBase<K, COH> {
@@ -163,7 +182,7 @@ template <int K, bool COH> struct MuppetRule : DenseBase<K, COH> {
         if (fwd == 8) {
             int acc = 0;
 #pragma unroll
-            for (int e = 0; e < E; ++e) acc += f2i8_sat(round_half_away(p[e] * sp)) * f2i8_sat(round_half_away(q[e] * sq));
+            for (int e = 0; e < E; ++e) acc += round_to_i8(p[e] * sp) * round_to_i8(q[e] * sq);
             acc = reduce_wave(acc, OpAdd());
             pred = div_pow2((float)acc, ip + iq);                        // acc / (sp * sq)
         } else if (fwd == 32) {
@@ -193,11 +212,11 @@ template <int K, bool COH> struct MuppetRule : DenseBase<K, COH> {
         float gp[E], gq[E];
         if (bwd == 8) {
             const float sq_rev = pow2_reciprocal(2u * ib);
-            const int ruv_i = f2i8_sat(round_half_away(ruv * sb));
-            const int lam_i = f2i8_sat(round_half_away(-1.0f * lambda * sb));
+            const int ruv_i = round_to_i8(ruv * sb);
+            const int lam_i = round_to_i8(-1.0f * lambda * sb);
 #pragma unroll
             for (int e = 0; e < E; ++e) {
-                const int pi = f2i8_sat(round_half_away(p[e] * sb)), qi = f2i8_sat(round_half_away(q[e] * sb));
+                const int pi = round_to_i8(p[e] * sb), qi = round_to_i8(q[e] * sb);
                 gp[e] = (float)(qi * ruv_i + pi * lam_i) * sq_rev;
                 gq[e] = (float)(pi * ruv_i + qi * lam_i) * sq_rev;
             }
@@ -271,7 +290,6 @@ __device__ __forceinline__ AfpQ afp_qpa(float diff, float range, float prev)
     q.itv = f2i_sat((beta / fmaxf(i1, i2)) - gamma);
     return q;
 }
-__device__ __forceinline__ int afp_sat8(float t) { return (int)(t > 127.0f ? 127.0f : (t < -128.0f) ? -128.0f : t); }
 __device__ __forceinline__ float ufirst(float x) { return from_bits<float>((uint32_t)__builtin_amdgcn_readfirstlane((int)bits(x))); }
 __device__ __forceinline__ int ufirst(int x) { return __builtin_amdgcn_readfirstlane(x); }
 
@@ -358,7 +376,7 @@ template <int K, bool COH> struct AfpRule : DenseBase<K, COH> {
         if (uq.n == 8 && iq.n == 8) {
             int acc = 0;
 #pragma unroll
-            for (int e = 0; e < E; ++e) acc += afp_sat8(round_half_away(p[e] * sp)) * afp_sat8(round_half_away(q[e] * sq));
+            for (int e = 0; e < E; ++e) acc += round_to_i8(p[e] * sp) * round_to_i8(q[e] * sq);
             acc = reduce_wave(acc, OpAdd());
             pred = div_pow2((float)acc, (uint32_t)uq.r + (uint32_t)iq.r);            // acc / (sp * sq); r >= 0
         } else {
@@ -384,12 +402,12 @@ template <int K, bool COH> struct AfpRule : DenseBase<K, COH> {
         }
         float gp[E], gq[E];
         if (bq.n == 8) {
-            const int lam_i = afp_sat8(round_half_away(-1.0f * lambda * sb));
-            const int ruv_i = afp_sat8(round_half_away(ruv * sb));
+            const int lam_i = round_to_i8(-1.0f * lambda * sb);
+            const int ruv_i = round_to_i8(ruv * sb);
             const float sq_rev = pow2_reciprocal(2u * (uint32_t)bq.r);
 #pragma unroll
             for (int e = 0; e < E; ++e) {
-                const int pi = afp_sat8(round_half_away(p[e] * sb)), qi = afp_sat8(round_half_away(q[e] * sb));
+                const int pi = round_to_i8(p[e] * sb), qi = round_to_i8(q[e] * sb);
                 gp[e] = (float)(qi * ruv_i + pi * lam_i) * sq_rev;
                 gq[e] = (float)(pi * ruv_i + qi * lam_i) * sq_rev;
             }
