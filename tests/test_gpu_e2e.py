@@ -56,13 +56,20 @@ def test_config1_fp32_sgd_k64(orc):
     assert np.allclose(out["lr"], [orc.lib.orc_lr_schedule(0.01, 0.1, e) for e in range(E)], rtol=0, atol=0)
 
 
-@pytest.mark.parametrize("version,k", [(4, 128), (3, 64), (2, 128)])
-def test_dense_variants_track_the_checker(orc, version, k):
+# AFP (-v 2) keeps its quantiser state per worker, not per row: a worker measures the range of one row and uses that
+# scale for the next `itv` ratings, whatever rows they touch, so the order in which racing workers' updates land
+# changes which scales saturate and the runs spread (final test RMSE 0.825 .. 0.833 over 16 runs of four workers,
+# with or without hot rows; the checker's sequential run of the same four workers gives 0.8280).  One worker has no
+# races: its run is the same every time (0.82326 in 16 of 16 runs) and ends 0.0015 from the checker's (scale
+# decisions that sit within an ulp of a power of two fall differently for v_log_f32 and the host's log2f, and every
+# such decision moves the trajectory); four workers are held to a bar above their spread.
+@pytest.mark.parametrize("version,k,W,tol", [(4, 128, 4, 0.005), (3, 64, 4, 0.005), (2, 128, 1, 0.003), (2, 128, 4, 0.012)])
+def test_dense_variants_track_the_checker(orc, version, k, W, tol):
     h = mfutil.hip()
     n_users, n_items = 3000, 1200
     R = mfutil.make_ratings(77 + version, n_users, n_items, 250_000, rank=8, alpha=1.0)
     train, test = _split(R, 200_000)
-    W, E = 4, 10
+    E = 10
     prm = h.default_params(k=k, num_workers=W, epoch=E, learning_rate=0.01, lam=0.05, decay=0.1, version=version, seed=5, sample_ratio=0.05)
     half = version == 4
     p, q = h.init_model(n_users, n_items, k, 5, half_rounded=half)
@@ -74,7 +81,7 @@ def test_dense_variants_track_the_checker(orc, version, k):
     ref, info = mfutil.oracle_train_dense(orc, version, train, test, p0, q0, k, W, E, 0.01, 0.05, 0.1, 5, sample_ratio=0.05)
     print("gpu", out["rmse"], "\ncpu", ref)
     assert out["rmse"][-1] < out["rmse"][0]
-    assert abs(out["rmse"][-1] - ref[-1]) < 0.005
+    assert abs(out["rmse"][-1] - ref[-1]) < tol
     if version == 3:
         assert out["report"].muppet_final_bits in (8, 12, 14, 16, 32)
 
