@@ -107,6 +107,60 @@ def test_afp_bit_exact(orc, k, afp_epoch):
     assert np.array_equal(gq.view(np.uint32), Q.view(np.uint32))
 
 
+def _special_rows(seed, k):
+    """A conflict-free problem whose workers own rows with special contents: all zeros (scale index 0 by definition),
+    huge values (the int8 conversion saturates), infinities (a ratio of 0, whose logarithm is -inf), exact .5 ties
+    after scaling (roundf's halves away from zero) and tiny values (scale indices near 100)."""
+    W, uc, window = 6, 1, 128
+    R, starts, P, Q = mfutil.conflict_free_problem(seed, k, W, uc, window)
+    up, ip = P.shape[0] // W, Q.shape[0] // W
+    P[1 * up] = 0.0; Q[1 * ip] = 0.0; P[1 * up + 1] = 0.0
+    P[2 * up, ::3] = 1e30; Q[2 * ip, 1::5] = -3e29
+    Q[3 * ip, 7] = np.inf; P[3 * up, 11] = -np.inf
+    P[4 * up] = (np.arange(k) % 9 - 4).astype(np.float32) * 0.0625 + 0.03125; Q[4 * ip] = 0.5 - (np.arange(k) % 5) * 0.25
+    P[5 * up:6 * up] *= 1e-29; Q[5 * ip:6 * ip] *= 1e-29
+    return R, starts, P, Q, uc, window
+
+
+def _same_values(got, want):
+    """Bit-exact where the checker's value is a number; the same positions hold NaN (payloads are not compared)."""
+    nan = np.isnan(want)
+    return np.array_equal(np.isnan(got), nan) and np.array_equal(got.view(np.uint32)[~nan], want.view(np.uint32)[~nan])
+
+
+@pytest.mark.parametrize("k", [64, 128])
+@pytest.mark.parametrize("bits", [8, 16])
+def test_muppet_special_values(orc, k, bits):
+    """The saturating conversions and the scale index on inputs that reach their edges (zeros, saturation, infinities,
+    ties, very small values): the kernel uses the hardware's conversions, the checker spells CUDA's cast rules out."""
+    import torch
+    h = mfutil.hip()
+    R, starts, P, Q, uc, window = _special_rows(700 + k + bits, k)
+    W = starts.shape[1]
+    dR, dS, dP, dQ = to_dev(R), to_dev(starts), to_dev(P), to_dev(Q)
+    d_sum = torch.zeros(k, dtype=torch.float32, device="cuda")
+    d_norm = torch.zeros(W, dtype=torch.float32, device="cuda")
+    h.mf_muppet_sgd_hogwild(dR.data_ptr(), R.size, dP.data_ptr(), dQ.data_ptr(), k, W, uc, window, LR, LAM, uc * window,
+                            d_sum.data_ptr(), d_norm.data_ptr(), bits, bits, 0, 0, dS.data_ptr(), mfutil.stream_ptr())
+    torch.cuda.synchronize()
+    sum_ref, norm_ref = np.zeros(k, np.float32), np.zeros(W, np.float32)
+    with np.errstate(all="ignore"):
+        orc.lib.orc_muppet_epoch(k, R.ctypes.data, R.size, P.ctypes.data, Q.ctypes.data, W, uc, window, LR, LAM, uc * window,
+                                 sum_ref.ctypes.data, norm_ref.ctypes.data, bits, bits, 0, 0, starts.ctypes.data, 1)
+    assert _same_values(from_dev(dP, np.float32, P.shape), P)
+    assert _same_values(from_dev(dQ, np.float32, Q.shape), Q)
+
+
+@pytest.mark.parametrize("k", [64, 128])
+def test_afp_special_values(orc, k):
+    R, starts, P, Q, uc, window = _special_rows(800 + k, k)
+    W = starts.shape[1]
+    gp, gq = _run_dense("afp", k, R, starts, P, Q, uc, window, (LR, LAM, 0))
+    orc.lib.orc_afp_epoch(k, R.ctypes.data, R.size, P.ctypes.data, Q.ctypes.data, W, uc, window, LR, LAM, 0, 0, 0, starts.ctypes.data, 1)
+    assert _same_values(gp, P)
+    assert _same_values(gq, Q)
+
+
 def _mascot_case(orc, k, W, uc, window, user_groups, item_groups, prec_mode, first_sample, seed, lr=LR):
     import torch
     h = mfutil.hip()
