@@ -261,6 +261,53 @@ def test_single_update_mascot_four_cases(orc, k):
             assert np.array_equal(dq.download()[0].view(np.uint8), gmq.arrays[0].view(np.uint8)), (up, ip)
 
 
+def _same_storage(got, want):
+    """Bit-exact where the checker's value is a number; NaN in the same positions (payloads are not compared)."""
+    if want.dtype == np.uint16:
+        nan = (want & 0x7fff) > 0x7c00
+        return np.array_equal((got & 0x7fff) > 0x7c00, nan) and np.array_equal(got[~nan], want[~nan])
+    return _same_values(got.view(np.float32), want.view(np.float32))
+
+
+@pytest.mark.parametrize("k", [64, 128])
+@pytest.mark.parametrize("case", ["subnormal", "overflow", "largest", "zeros"])
+def test_single_update_mascot_special_values(orc, k, case):
+    """One update in each of the four precision cases on rows at the edges of binary16: products and sums in the
+    subnormal range (nothing may be flushed to zero), values whose products overflow to infinity (and the NaN that
+    follows), the largest finite binary16 value, and signed zeros."""
+    import torch
+    h = mfutil.hip()
+    rng = np.random.default_rng(170 + k)
+    g = rng.standard_normal((2, 1, k)).astype(np.float32)
+    if case == "subnormal":
+        P, Q, r = g[0] * 3e-6, g[1] * 0.5, 1e-5
+    elif case == "overflow":
+        P, Q, r = g[0] * 200.0, g[1] * 300.0, 4.0
+    elif case == "largest":
+        P, Q, r = np.full((1, k), 65504.0, np.float32), g[1] * 1e-3, 4.0
+        P[0, ::2] = -65504.0
+    else:
+        P, Q, r = np.zeros((1, k), np.float32), g[1] * 0.1, 0.0
+        P[0, ::3] = -0.0
+    for up in (0, 1):
+        for ip in (0, 1):
+            R = np.zeros(1, mfutil.NODE); R["r"] = r
+            gmp = mfutil.host_grouped(orc, k, P.astype(np.float32), np.array([0], np.uint32), np.array([up], np.uint8))
+            gmq = mfutil.host_grouped(orc, k, Q.astype(np.float32), np.array([0], np.uint32), np.array([ip], np.uint8))
+            dp, dq = mfutil.DeviceGrouped(gmp), mfutil.DeviceGrouped(gmq)
+            dR = to_dev(R); dS = to_dev(np.zeros((1, 1), np.uint32))
+            z = torch.zeros(4 * k, dtype=torch.float32, device="cuda")
+            h.mf_mascot_sgd_hogwild(dR.data_ptr(), 1, dp.ptrs.data_ptr(), dq.ptrs.data_ptr(), k, 1, 1, 1, LR, LAM,
+                                    dp.end.data_ptr(), dq.end.data_ptr(), dp.prec.data_ptr(), dq.prec.data_ptr(),
+                                    z.data_ptr(), z[k:].data_ptr(), z[2 * k:].data_ptr(), z[3 * k:].data_ptr(),
+                                    1, 1, 1, 0, 0, dS.data_ptr(), mfutil.stream_ptr())
+            torch.cuda.synchronize()
+            with np.errstate(all="ignore"):
+                orc.lib.orc_mascot_update(k, gmp.arrays[0].ctypes.data, up, gmq.arrays[0].ctypes.data, ip, r, LR, LAM, None, None, None, None)
+            assert _same_storage(dp.download()[0], gmp.arrays[0]), (case, up, ip)
+            assert _same_storage(dq.download()[0], gmq.arrays[0]), (case, up, ip)
+
+
 @pytest.mark.parametrize("k", [64, 128])
 def test_counter_rng_schedule_matches_checker(orc, k):
     """window_start == NULL: the kernel's own generator must pick the windows the checker's twin picks."""
