@@ -128,6 +128,49 @@ def _same_values(got, want):
     return np.array_equal(np.isnan(got), nan) and np.array_equal(got.view(np.uint32)[~nan], want.view(np.uint32)[~nan])
 
 
+def _half_edge_rows(seed, k):
+    """A conflict-free problem whose workers own rows at the edges of binary16: zeros, values whose products and
+    scaled gradients overflow binary16, values in its subnormal range, and an infinity."""
+    W, uc, window = 5, 1, 128
+    R, starts, P, Q = mfutil.conflict_free_problem(seed, k, W, uc, window)
+    up, ip = P.shape[0] // W, Q.shape[0] // W
+    P[1 * up] = 0.0; Q[1 * ip] = -0.0
+    P[2 * up:3 * up] *= 3000.0; Q[2 * ip:3 * ip] *= 2000.0
+    P[3 * up:4 * up] *= 3e-5; Q[3 * ip:4 * ip] *= 1e-4
+    Q[4 * ip, 3] = np.inf
+    return R, starts, P, Q, uc, window
+
+
+@pytest.mark.parametrize("k", [64, 128])
+@pytest.mark.parametrize("variant", ["single", "mpt", "mem_quant"])
+def test_dense_rules_special_values(orc, k, variant):
+    """fp32 SGD, MPT (binary16 arithmetic on values scaled by 1000) and -v 7 (binary16 storage) on such rows."""
+    import torch
+    h = mfutil.hip()
+    R, starts, P, Q, uc, window = _half_edge_rows(900 + k, k)
+    W = starts.shape[1]
+    with np.errstate(all="ignore"):
+        if variant == "mem_quant":
+            Ph, Qh = orc.f2h(P).reshape(P.shape), orc.f2h(Q).reshape(Q.shape)
+            dR, dS, dP, dQ = to_dev(R), to_dev(starts), to_dev(Ph), to_dev(Qh)
+            h.mf_mem_quant_sgd_hogwild(dR.data_ptr(), R.size, dP.data_ptr(), dQ.data_ptr(), k, W, uc, window, LR, LAM, 1234, 0, dS.data_ptr(), mfutil.stream_ptr())
+            torch.cuda.synchronize()
+            orc.lib.orc_mem_quant_epoch(k, R.ctypes.data, R.size, Ph.ctypes.data, Qh.ctypes.data, W, uc, window, LR, LAM, 0, 0, starts.ctypes.data, 1)
+            assert _same_storage(from_dev(dP, np.uint16, P.shape), Ph)
+            assert _same_storage(from_dev(dQ, np.uint16, Q.shape), Qh)
+            return
+        if variant == "mpt":
+            P = orc.h2f(orc.f2h(P)).reshape(P.shape); Q = orc.h2f(orc.f2h(Q)).reshape(Q.shape)
+            lam_h = orc.lib.orc_float2half(np.float32(LAM) * np.float32(1000.0))
+            gp, gq = _run_dense("mpt", k, R, starts, P, Q, uc, window, (LR, lam_h, 1000.0))
+            orc.lib.orc_mpt_epoch(k, R.ctypes.data, R.size, P.ctypes.data, Q.ctypes.data, W, uc, window, LR, LAM, 1000.0, 0, 0, starts.ctypes.data, 1)
+        else:
+            gp, gq = _run_dense("single", k, R, starts, P, Q, uc, window, (LR, LAM))
+            orc.lib.orc_sgd_epoch(k, R.ctypes.data, R.size, P.ctypes.data, Q.ctypes.data, W, uc, window, LR, LAM, 0, 0, starts.ctypes.data, 1)
+    assert _same_values(gp, P)
+    assert _same_values(gq, Q)
+
+
 @pytest.mark.parametrize("k", [64, 128])
 @pytest.mark.parametrize("bits", [8, 16])
 def test_muppet_special_values(orc, k, bits):
