@@ -271,6 +271,21 @@ def cpu_baseline(prob, cfg, seed, threads, target_updates):
     return done / dt, done, dt
 
 
+def cpu_baseline_fp32(prob, h, cfg, seed, threads, target_updates):
+    """The checker's fp32 SGD epoch (reference rule of -v 5) as the same Hogwild CPU loop, dense fp32 P and Q."""
+    from oracle import oracle as om
+    orc = om.get()
+    R = prob.R.cpu().numpy().view(np.uint8).reshape(-1).view(om.NODE)
+    P = orc.init_normal(seed, 0, prob.n_users * prob.k)
+    Q = orc.init_normal(seed, 1, prob.n_items * prob.k)
+    W = threads * 8
+    uc = max(1, target_updates // (W * 128))
+    t0 = time.perf_counter()
+    orc.lib.orc_sgd_epoch(prob.k, R.ctypes.data, R.size, P.ctypes.data, Q.ctypes.data, W, uc, 128, cfg["lr"], cfg["lam"], seed, 0, None, threads)
+    dt = time.perf_counter() - t0
+    return W * uc * 128 / dt, W * uc * 128, dt
+
+
 def time_fp32_sgd(torch, h, prob, W, warmup, steps, cfg, seed):
     """The fp32-SGD update (-v 5) on the same ratings, schedule and hot-row tables: dense fp32 P and Q."""
     dev, k, st = prob.R.device, prob.k, torch.cuda.current_stream().cuda_stream
@@ -565,6 +580,10 @@ def main():
         out["cpu_baseline"] = {"value": rate, "unit": "ratings/s", "cores": threads, "kind": "port",
                                "sample": "%d updates of the same shuffled ratings and binary16 model (%d workers x %d windows of 128), "
                                          "%.1f s, OpenMP Hogwild loop of the checker" % (done, threads * 8, done // (threads * 8 * 128), dt)}
+        if not a.skip_fp32:
+            rate, done, dt = cpu_baseline_fp32(prob, h, cfg, a.seed, threads, a.cpu_updates // 2)
+            out["cpu_baseline"]["fp32_sgd"] = {"value": rate, "unit": "ratings/s", "cores": threads, "kind": "port",
+                                               "sample": "%d updates of the same shuffled ratings, dense fp32 model, %.1f s" % (done, dt)}
     print(json.dumps(out))
 
 
