@@ -127,14 +127,15 @@ def test_whole_model_switching_variant_tracks_the_checker(orc):
     assert gpu_switched == (switched >= 0)
 
 
-def test_mascot_reduced_config2(orc):
-    """BASELINE config 2 at one tenth: Zipf(0.9), rank-16 truth, ratings 0.5-5.0 in half steps; MASCOT k=128,
-    sample ratio 0.05, period 2; a low threshold so that groups do switch to binary32 within 12 epochs."""
+@pytest.mark.parametrize("name,n_users,n_items,alpha,k", [("config2", 7000, 1070, 0.9, 128), ("config3", 8100, 2950, 1.0, 64)])
+def test_mascot_reduced_configs(orc, name, n_users, n_items, alpha, k):
+    """BASELINE config 2 at one tenth (Zipf(0.9), k=128) and config 3 at one twentieth (Zipf(1.0), k=64): rank-16
+    truth, ratings 0.5-5.0 in half steps; MASCOT, sample ratio 0.05, period 2; a low threshold so that groups do
+    switch to binary32 within 12 epochs."""
     h = mfutil.hip()
-    n_users, n_items = 7000, 1070
-    R = mfutil.make_ratings(2, n_users, n_items, 1_000_000, rank=16, alpha=0.9, step=0.5, lo=0.5, hi=5.0, mean=3.5, noise=0.8)
+    R = mfutil.make_ratings(2, n_users, n_items, 1_000_000, rank=16, alpha=alpha, step=0.5, lo=0.5, hi=5.0, mean=3.5, noise=0.8)
     train, test = _split(R, 800_000)
-    k, W, E = 128, 8, 12
+    W, E = 8, 12
     kw = dict(k=k, num_workers=W, epoch=E, learning_rate=0.01, lam=0.015, decay=0.1, version=1, seed=3,
               user_group_num=20, item_group_num=20, sample_ratio=0.05, interval=2, error_threshold=1.5)
     prm = h.default_params(**kw)
