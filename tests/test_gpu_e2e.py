@@ -56,6 +56,69 @@ def test_config1_fp32_sgd_k64(orc):
     assert np.allclose(out["lr"], [orc.lib.orc_lr_schedule(0.01, 0.1, e) for e in range(E)], rtol=0, atol=0)
 
 
+@pytest.mark.parametrize("version,k", [(5, 64), (5, 128), (4, 128)])
+def test_single_worker_run_is_the_checkers_run(orc, version, k):
+    """One worker has no races and applies its updates in order, so a whole mf_train run (device shuffle, counter-based
+    windows, learning-rate schedule, update kernels over several epochs) must leave the very model the checker's
+    sequential run leaves: every value of P and Q bit for bit, for fp32 SGD and for MPT."""
+    h = mfutil.hip()
+    n_users, n_items = 900, 400
+    R = mfutil.make_ratings(11 + version + k, n_users, n_items, 60_000, rank=8, alpha=1.0)
+    train, test = _split(R, 50_000)
+    E = 3
+    prm = h.default_params(k=k, num_workers=1, epoch=E, learning_rate=0.01, lam=0.05, decay=0.1, version=version, seed=9)
+    half = version == 4
+    p, q = h.init_model(n_users, n_items, k, 9, half_rounded=half)
+    p0, q0 = p.copy(), q.copy()
+    out = h.train(prm, train, n_users, n_items, test, p, q)
+    ref, _ = mfutil.oracle_train_dense(orc, version, train, test, p0, q0, k, 1, E, 0.01, 0.05, 0.1, 9, threads=1)
+    assert np.array_equal(p.view(np.uint32), p0.view(np.uint32))
+    assert np.array_equal(q.view(np.uint32), q0.view(np.uint32))
+    assert np.allclose(out["rmse"], ref, rtol=1e-6, atol=0)
+
+
+@pytest.mark.parametrize("k", [64, 128])
+def test_single_worker_binary16_storage_run_is_the_checkers_run(orc, k):
+    """The same for -v 7 (binary16 storage, binary32 arithmetic)."""
+    h = mfutil.hip()
+    n_users, n_items = 900, 400
+    R = mfutil.make_ratings(17 + k, n_users, n_items, 60_000, rank=8, alpha=1.0)
+    train, test = _split(R, 50_000)
+    prm = h.default_params(k=k, num_workers=1, epoch=3, learning_rate=0.01, lam=0.05, decay=0.1, version=7, seed=9)
+    p, q = h.init_model(n_users, n_items, k, 9, half_rounded=True)
+    p0, q0 = p.copy(), q.copy()
+    out = h.train(prm, train, n_users, n_items, test, p, q)
+    ref = mfutil.oracle_train_mem_quant(orc, train, test, p0, q0, k, 1, 3, 0.01, 0.05, 0.1, 9, threads=1)
+    assert np.array_equal(p.view(np.uint32), p0.view(np.uint32))
+    assert np.array_equal(q.view(np.uint32), q0.view(np.uint32))
+    assert np.allclose(out["rmse"], ref, rtol=1e-6, atol=0)
+
+
+@pytest.mark.parametrize("k", [64, 128])
+def test_single_worker_mascot_run_is_the_checkers_run(orc, k):
+    """The same for MASCOT (-v 1) through pre-processing, grouping, scatter, seven epochs with two check epochs and the
+    switching they decide: every group ends in the checker's precision and holds the checker's values bit for bit.
+    (The sampled sums are added in a different order on the device; a decision would only differ for an error within
+    1e-5 of the threshold.)"""
+    h = mfutil.hip()
+    n_users, n_items = 900, 400
+    R = mfutil.make_ratings(23 + k, n_users, n_items, 60_000, rank=8, alpha=1.0)
+    train, test = _split(R, 50_000)
+    E = 9
+    prm = h.default_params(k=k, num_workers=1, epoch=E, learning_rate=0.01, lam=0.015, decay=0.1, version=1, seed=9,
+                           user_group_num=6, item_group_num=5, sample_ratio=0.05, interval=2, error_threshold=1.5)
+    p, q = h.init_model(n_users, n_items, k, 9)
+    p0, q0 = p.copy(), q.copy()
+    out = h.train(prm, train, n_users, n_items, test, p, q)
+    ref, info = mfutil.oracle_train_mascot(orc, train, test, p0, q0, k, 1, E, 0.01, 0.015, 0.1, 9, 6, 5, 0.05, 2, 1.5, threads=1)
+    print("gpu prec", out["user_prec"], out["item_prec"], "\ncpu prec", info["gu"].prec, info["gi"].prec)
+    assert np.array_equal(out["user_prec"], info["gu"].prec) and np.array_equal(out["item_prec"], info["gi"].prec)
+    for got, gm in ((p, info["gu"]), (q, info["gi"])):
+        want = np.concatenate([a.reshape(-1, k) if a.dtype == np.float32 else orc.h2f(a).reshape(-1, k) for a in gm.arrays])
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    assert np.allclose(out["rmse"], ref, rtol=1e-6, atol=0)
+
+
 # AFP (-v 2) keeps its quantiser state per worker, not per row: a worker measures the range of one row and uses that
 # scale for the next `itv` ratings, whatever rows they touch, so the order in which racing workers' updates land
 # changes which scales saturate and the runs spread (final test RMSE 0.825 .. 0.833 over 16 runs of four workers,
