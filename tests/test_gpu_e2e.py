@@ -78,6 +78,27 @@ def test_single_worker_run_is_the_checkers_run(orc, version, k):
 
 
 @pytest.mark.parametrize("k", [64, 128])
+def test_single_worker_muppet_run_is_the_checkers_run(orc, k):
+    """The same for MuPPET (-v 3) with its bit-width ladder: sixteen epochs, long enough for the ladder to move (its
+    diversity statistic sums the sampled gradients in another order on the device, which would only matter for a
+    ratio within 1e-5 of the switching bound)."""
+    h = mfutil.hip()
+    n_users, n_items = 900, 400
+    R = mfutil.make_ratings(29 + k, n_users, n_items, 60_000, rank=8, alpha=1.0)
+    train, test = _split(R, 50_000)
+    E = 16
+    prm = h.default_params(k=k, num_workers=1, epoch=E, learning_rate=0.01, lam=0.05, decay=0.1, version=3, seed=9, sample_ratio=0.05)
+    p, q = h.init_model(n_users, n_items, k, 9)
+    p0, q0 = p.copy(), q.copy()
+    out = h.train(prm, train, n_users, n_items, test, p, q)
+    ref, info = mfutil.oracle_train_dense(orc, 3, train, test, p0, q0, k, 1, E, 0.01, 0.05, 0.1, 9, threads=1, sample_ratio=0.05)
+    print("final bits", out["report"].muppet_final_bits, info["final_bits"])
+    assert out["report"].muppet_final_bits == info["final_bits"]
+    assert np.array_equal(p.view(np.uint32), p0.view(np.uint32))
+    assert np.array_equal(q.view(np.uint32), q0.view(np.uint32))
+
+
+@pytest.mark.parametrize("k", [64, 128])
 def test_single_worker_binary16_storage_run_is_the_checkers_run(orc, k):
     """The same for -v 7 (binary16 storage, binary32 arithmetic)."""
     h = mfutil.hip()
