@@ -98,6 +98,25 @@ def test_single_worker_muppet_run_is_the_checkers_run(orc, k):
     assert np.array_equal(q.view(np.uint32), q0.view(np.uint32))
 
 
+def test_single_worker_whole_model_switching_run_is_the_checkers_run(orc):
+    """The same for -v 8: the run switches the whole model to binary32 in the epoch the checker does."""
+    h = mfutil.hip()
+    n_users, n_items, k = 900, 400, 128
+    R = mfutil.make_ratings(37, n_users, n_items, 60_000, rank=8, alpha=1.0)
+    train, test = _split(R, 50_000)
+    E = 12
+    prm = h.default_params(k=k, num_workers=1, epoch=E, learning_rate=0.01, lam=0.05, decay=0.1, version=8, seed=9,
+                           sample_ratio=0.05, interval=2, error_threshold=0.3)
+    p, q = h.init_model(n_users, n_items, k, 9, half_rounded=True)
+    p0, q0 = p.copy(), q.copy()
+    out = h.train(prm, train, n_users, n_items, test, p, q)
+    ref, switched, errors = mfutil.oracle_train_switching_only(orc, train, test, p0, q0, k, 1, E, 0.01, 0.05, 0.1, 9, 0.05, 2, 0.3, threads=1)
+    print("switched at", switched, errors)
+    assert np.array_equal(p.view(np.uint32), p0.view(np.uint32))
+    assert np.array_equal(q.view(np.uint32), q0.view(np.uint32))
+    assert np.allclose(out["rmse"], ref, rtol=1e-6, atol=0)
+
+
 @pytest.mark.parametrize("k", [64, 128])
 def test_single_worker_binary16_storage_run_is_the_checkers_run(orc, k):
     """The same for -v 7 (binary16 storage, binary32 arithmetic)."""
