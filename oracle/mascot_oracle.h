@@ -19,6 +19,12 @@
  *   - MuPPET / AFP: floor/ceil(log2f(x)) for x within one ulp of a power of
  *     two, and float -> int8 conversion of values outside [-128,127], depend on
  *     CUDA's libdevice / cvt behaviour.  parity unpinned for those inputs.
+ *   - AFP's error measurement (QEM, afp/afp_sgd_kernel.h:32-59) uses the value
+ *     of log2f itself, not its floor: the last bit of the host's log2f, of
+ *     CUDA's and of a GPU's v_log_f32 may differ, and the re-measurement
+ *     interval computed from it then differs by one now and then.  parity
+ *     unpinned for whole AFP trajectories (single epochs on conflict-free
+ *     schedules are compared bit for bit with the GPU and agree).
  *   - orc_sgd_update / orc_mem_quant_update: binary32 arithmetic that nvcc may
  *     contract into fma where the source writes a*b - c*d; this restatement
  *     rounds every operation.  parity unpinned for that choice (the update is
