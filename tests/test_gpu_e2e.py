@@ -365,6 +365,54 @@ def test_quantized_mf_command_line(orc, tmp_path, version):
         assert abs(_evaluate(model, te, version) - orc.rmse(k, every, P, Q)) < 1e-5
 
 
+def test_command_line_single_worker_model_file_is_the_checkers(orc, tmp_path):
+    """quantized_mf -v 5 -wg 1 from TSV files to the model file: with one worker the run has no races, so every number
+    in <out>.txt is the text of the value the checker's run of the same rule leaves (ids re-mapped in first-seen
+    order, rows written back under their original ids, absent ids as zero rows)."""
+    assert os.path.exists(CLI), "quantized_mf is not built"
+    n_users, n_items, k, E, seed = 300, 120, 64, 3, 9
+    R = mfutil.make_ratings(53, n_users, n_items, 24_000)
+    train, test = R[:20_000], R[20_000:]
+    tr, te = str(tmp_path / "train.tsv"), str(tmp_path / "test.tsv")
+    _write_tsv(tr, train)
+    _write_tsv(te, test)
+    out = str(tmp_path / "model")
+    cmd = [CLI, "-i", tr, "-y", te, "-o", out, "-v", "5", "-k", str(k), "-l", str(E), "-wg", "1", "-a", "0.01", "-b", "0.05",
+           "-d", "0.1", "-seed", str(seed)]
+    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=300)
+    assert res.returncode == 0, res.stderr
+    printed = [l.split()[2] for l in res.stdout.splitlines() if len(l.split()) == 3 and l.split()[0].isdigit()]
+    # dense ids in first-seen order over the training file (io_utils.h:93-106)
+    def first_seen(x):
+        _, first = np.unique(x, return_index=True)
+        order = x[np.sort(first)]
+        return {int(v): j for j, v in enumerate(order)}
+    umap, imap = first_seen(train["u"]), first_seen(train["i"])
+    dense = train.copy()
+    dense["u"] = [umap[int(v)] for v in train["u"]]
+    dense["i"] = [imap[int(v)] for v in train["i"]]
+    keep = np.isin(test["u"], train["u"]) & np.isin(test["i"], train["i"])
+    dtest = test[keep].copy()
+    dtest["u"] = [umap[int(v)] for v in dtest["u"]]
+    dtest["i"] = [imap[int(v)] for v in dtest["i"]]
+    dtest = mfutil.test_set_order(dtest)
+    nu, ni = len(umap), len(imap)
+    P = orc.init_normal(seed, 0, nu * k).reshape(nu, k)
+    Q = orc.init_normal(seed, 1, ni * k).reshape(ni, k)
+    ref, _ = mfutil.oracle_train_dense(orc, 5, dense, dtest, P, Q, k, 1, E, 0.01, 0.05, 0.1, seed, threads=1)
+    assert len(printed) == E and np.allclose([float(x) for x in printed], ref, rtol=1e-5, atol=0)      # six digits are printed
+    rows = open(out + ".txt").read().split("\n")
+    max_u, max_i = int(train["u"].max()) * 3 + 1, int(train["i"].max()) * 2 + 5
+    assert rows[0].split() == [str(max_u + 1), str(max_i + 1), str(k)]
+    Pf, Qf = np.zeros((max_u + 1, k), np.float32), np.zeros((max_i + 1, k), np.float32)
+    for orig, j in umap.items():
+        Pf[orig * 3 + 1] = P[j]
+    for orig, j in imap.items():
+        Qf[orig * 2 + 5] = Q[j]
+    assert rows[1].split() == ["%g" % v for v in Pf.ravel()]
+    assert rows[2].split() == ["%g" % v for v in Qf.ravel()]
+
+
 def test_command_line_rating_cache(tmp_path):
     """-cache 1: the second run loads <train>.mfcache instead of parsing, reports the same data set, prints the same
     "Missing" line and rewrites remove_user.txt; touching the training file invalidates the cache."""
