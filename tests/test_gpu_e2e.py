@@ -413,6 +413,46 @@ def test_command_line_single_worker_model_file_is_the_checkers(orc, tmp_path):
     assert rows[2].split() == ["%g" % v for v in Qf.ravel()]
 
 
+def test_command_line_single_worker_mascot_model_file_is_the_checkers(orc, tmp_path):
+    """The same for -v 1: <out>_reconst.txt holds the checker's MASCOT model in popularity-sorted row order, number for
+    number, after nine epochs with check epochs and switching."""
+    assert os.path.exists(CLI), "quantized_mf is not built"
+    n_users, n_items, k, E, seed = 300, 120, 64, 9, 9
+    R = mfutil.make_ratings(59, n_users, n_items, 24_000)
+    train, test = R[:20_000], R[20_000:]
+    tr, te = str(tmp_path / "train.tsv"), str(tmp_path / "test.tsv")
+    _write_tsv(tr, train)
+    _write_tsv(te, test)
+    out = str(tmp_path / "model")
+    cmd = [CLI, "-i", tr, "-y", te, "-o", out, "-v", "1", "-k", str(k), "-l", str(E), "-wg", "1", "-a", "0.01", "-b", "0.015",
+           "-d", "0.1", "-ug", "5", "-ig", "4", "-s", "0.05", "-it", "2", "-e", "1.5", "-seed", str(seed)]
+    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=300)
+    assert res.returncode == 0, res.stderr
+    def first_seen(x):
+        _, first = np.unique(x, return_index=True)
+        order = x[np.sort(first)]
+        return {int(v): j for j, v in enumerate(order)}
+    umap, imap = first_seen(train["u"]), first_seen(train["i"])
+    dense = train.copy()
+    dense["u"] = [umap[int(v)] for v in train["u"]]
+    dense["i"] = [imap[int(v)] for v in train["i"]]
+    keep = np.isin(test["u"], train["u"]) & np.isin(test["i"], train["i"])
+    dtest = test[keep].copy()
+    dtest["u"] = [umap[int(v)] for v in dtest["u"]]
+    dtest["i"] = [imap[int(v)] for v in dtest["i"]]
+    dtest = mfutil.test_set_order(dtest)
+    nu, ni = len(umap), len(imap)
+    P = orc.init_normal(seed, 0, nu * k).reshape(nu, k)
+    Q = orc.init_normal(seed, 1, ni * k).reshape(ni, k)
+    ref, info = mfutil.oracle_train_mascot(orc, dense, dtest, P, Q, k, 1, E, 0.01, 0.015, 0.1, seed, 5, 4, 0.05, 2, 1.5, threads=1)
+    rows = open(out + "_reconst.txt").read().split("\n")
+    assert rows[0].split() == [str(nu), str(ni), str(k)]
+    for row, gm in ((rows[1], info["gu"]), (rows[2], info["gi"])):
+        want = np.concatenate([a.reshape(-1, k) if a.dtype == np.float32 else orc.h2f(a).reshape(-1, k) for a in gm.arrays])
+        assert row.split() == ["%g" % v for v in want.ravel()]
+    assert info["gu"].prec.sum() + info["gi"].prec.sum() >= 1          # the run did switch groups
+
+
 def test_command_line_rating_cache(tmp_path):
     """-cache 1: the second run loads <train>.mfcache instead of parsing, reports the same data set, prints the same
     "Missing" line and rewrites remove_user.txt; touching the training file invalidates the cache."""
