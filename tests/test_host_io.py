@@ -108,3 +108,12 @@ def test_round_half_away_identity_is_exhaustive(tmp_path):
     subprocess.run(["gcc", "-O2", "-fopenmp", "-ffp-contract=off", "-o", exe, os.path.join(ROOT, "tests", "round_identity_check.c"), "-lm"], check=True)
     r = subprocess.run([exe], capture_output=True, text=True, timeout=600)
     assert r.returncode == 0 and r.stdout.strip() == "0", r.stdout + r.stderr
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py measures one GPU; asked for more it says so and exits without touching a device."""
+    import subprocess
+    import sys
+    res = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=120)
+    assert res.returncode == 2
+    assert "one GPU" in res.stderr and res.stdout == ""
