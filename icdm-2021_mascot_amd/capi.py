@@ -16,11 +16,7 @@ u8, u16, u32, u64, i32, f32, vp = C.c_uint8, C.c_uint16, C.c_uint32, C.c_uint64,
 SIGNATURES = {
     "mf_version": (i32, []),
     "mf_last_error": (C.c_char_p, []),
-    "mf_set_row_coherence": (i32, [i32]),
-    "mf_get_row_coherence": (i32, []),
-    "mf_set_epoch_splits": (i32, [u32]),
-    "mf_get_epoch_splits": (u32, []),
-    "mf_set_hot_row_thinning": (i32, [vp, vp]),
+    "mf_hogwild_inflight": (f32, [u32, i32, u32, u32, u32]),
     "mf_mascot_norm_blocks": (u32, [u32]),
     "mf_update_count": (u32, [u32, u32, u32]),
     "mf_auto_workers": (u32, [u32]),
@@ -30,8 +26,8 @@ SIGNATURES = {
     "mf_window_start": (u32, [u64, u32, u32, u32, u32]),
     "mf_single_sgd_hogwild": (i32, [vp, u32, vp, vp, i32, u32, u32, u32, f32, f32, u64, u32, vp, vp]),
     "mf_mem_quant_sgd_hogwild": (i32, [vp, u32, vp, vp, i32, u32, u32, u32, f32, f32, u64, u32, vp, vp]),
-    "mf_hot_row_table": (i32, [vp, u32, u32, u32, f32, vp]),
-    "mf_row_traffic_probe": (i32, [vp, u32, vp, vp, u32, u32, vp, vp, u64, i32, vp]),
+    "mf_hot_row_table": (i32, [vp, u32, u32, f32, f32, f32, f32, vp, vp, vp, vp]),
+    "mf_row_traffic_probe": (i32, [vp, u32, vp, vp, u32, u32, u64, vp, vp]),
     "mf_synth_baseline_config": (i32, [i32, vp]),
     "mf_generate_ratings": (i32, [vp, u64, u64, u64, vp, vp]),
     "mf_generate_ratings_host": (i32, [vp, u64, u64, u64, vp]),
@@ -57,7 +53,19 @@ SIGNATURES = {
     "mf_init_model": (i32, [vp, vp, u32, u32, u32, u64, i32]),
     "mf_train": (i32, [vp, vp, u32, u32, u32, vp, u32, vp, vp, vp]),
     "mf_group_end_indices": (u32, [vp, u32, u32, vp]),
+    "mf_session_create": (i32, [vp, vp, u32, u32, u32, vp, u32, vp, vp, vp, vp]),
+    "mf_session_epoch": (i32, [vp, vp, vp]),
+    "mf_session_finish": (i32, [vp, vp, vp]),
+    "mf_session_destroy": (None, [vp]),
+    "mf_session_workers": (u32, [vp]),
+    "mf_session_hot_rows": (i32, [vp, vp, vp, vp]),
+    "mf_session_device_state": (i32, [vp, u32, vp, vp]),
+    "mf_replicate_threshold": (f32, [f32, f32]),
+    "mf_replica_sync_dense": (i32, [vp, u32, i32, vp, vp, u32, i32, vp]),
 }
+# the update launches with one more argument, const mf_hogwild_options*
+for _name in ("mf_single_sgd_hogwild", "mf_mem_quant_sgd_hogwild", "mf_mpt_sgd_hogwild", "mf_muppet_sgd_hogwild", "mf_afp_sgd_hogwild", "mf_mascot_sgd_hogwild"):
+    SIGNATURES[_name + "_opt"] = (i32, SIGNATURES[_name][1] + [vp])
 
 
 f64 = C.c_double
@@ -74,7 +82,14 @@ class MfParams(C.Structure):
     _fields_ = [("lambda_", f32), ("learning_rate", f32), ("decay", f32), ("sample_ratio", f32), ("error_threshold", f32),
                 ("interval", u32), ("user_group_num", u32), ("item_group_num", u32), ("k", u32), ("num_workers", u32),
                 ("epoch", u32), ("thread_block_size", u32), ("version", u32), ("is_yahoo", u32), ("seed", u64),
-                ("verbose", u32), ("cached_rows", u32), ("epoch_splits", u32), ("hot_row_inflight", f32), ("hot_row_inflight_early", f32), ("hot_row_early_epochs", u32)]
+                ("verbose", u32), ("cached_rows", u32), ("epoch_splits", u32), ("hot_row_inflight", f32), ("hot_row_inflight_early", f32), ("hot_row_early_epochs", u32),
+                ("hot_rows", u32), ("replicate_inflight", f32), ("replica_merges", u32), ("replica_add_inflight", f32)]
+
+
+class HogwildOptions(C.Structure):
+    """mf_hogwild_options of include/mascot_hip.h."""
+    _fields_ = [("cached_rows", u32), ("launches", u32), ("user_keep", vp), ("item_keep", vp), ("user_slot", vp), ("item_slot", vp),
+                ("user_slot_row", vp), ("item_slot_row", vp), ("user_replicas", vp), ("item_replicas", vp), ("user_slots", u32), ("item_slots", u32)]
 
 
 class MfReport(C.Structure):
@@ -124,7 +139,7 @@ class MascotHip:
     def __getattr__(self, name):
         if name.startswith("mf_"):
             fn = getattr(self.lib, name)
-            if SIGNATURES[name][0] is i32 and name not in ("mf_version", "mf_get_row_coherence"):
+            if SIGNATURES[name][0] is i32 and name != "mf_version":
                 return lambda *a: self.call(name, *a)
             return fn
         raise AttributeError(name)
@@ -178,6 +193,56 @@ class MascotHip:
         out["user_prec"] = out["user_prec"][:rep.user_group_num]
         out["item_prec"] = out["item_prec"][:rep.item_group_num]
         return out
+
+
+class Session:
+    """mf_session_* over numpy arrays: the product's training driver, one epoch per call."""
+
+    def __init__(self, h, prm, R, n_users, n_items, test, p, q):
+        self.h, self.prm = h, prm
+        self.R, self.test, self.p, self.q = np.ascontiguousarray(R), np.ascontiguousarray(test), p, q
+        self.report = MfReport()
+        self.ptr = vp()
+        h.call("mf_session_create", C.byref(prm), self.R.ctypes.data, self.R.size, n_users, n_items, self.test.ctypes.data, self.test.size,
+               p.ctypes.data, q.ctypes.data, C.byref(self.report), C.byref(self.ptr))
+        self.epochs_done = 0
+
+    def epoch(self):
+        """Runs the next epoch; returns (test RMSE, milliseconds of its update launches)."""
+        rmse, ms = C.c_double(0), C.c_float(0)
+        self.h.call("mf_session_epoch", self.ptr, C.byref(rmse), C.byref(ms))
+        self.epochs_done += 1
+        return rmse.value, ms.value
+
+    @property
+    def workers(self):
+        return self.h.lib.mf_session_workers(self.ptr)
+
+    def hot_rows(self):
+        u, v, f = u32(0), u32(0), f32(0)
+        self.h.call("mf_session_hot_rows", self.ptr, C.byref(u), C.byref(v), C.byref(f))
+        return u.value, v.value, f.value
+
+    def device_state(self, epoch):
+        """(device address of the session's ratings, address of the mf_hogwild_options of `epoch`)."""
+        r, o = vp(), vp()
+        self.h.call("mf_session_device_state", self.ptr, epoch, C.byref(r), C.byref(o))
+        return r.value, o.value
+
+    def finish(self):
+        self.h.call("mf_session_finish", self.ptr, self.p.ctypes.data, self.q.ctypes.data)
+        return self.p, self.q
+
+    def close(self):
+        if self.ptr:
+            self.h.lib.mf_session_destroy(self.ptr)
+            self.ptr = vp()
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
 
 
 _handle = None

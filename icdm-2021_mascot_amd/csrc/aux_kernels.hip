@@ -400,7 +400,8 @@ using namespace mf;
 // write policy, the figure the update kernels' epoch time is compared with.
 template <int BYTES, bool COH>       // bytes per lane: a row is 64 * BYTES bytes
 __global__ __launch_bounds__(kBlock) void row_traffic_probe_kernel(const mf_node* R, uint32_t n, uint8_t* P, uint8_t* Q, uint32_t per_worker,
-                                                                  const uint8_t* keep_u, const uint8_t* keep_v, uint64_t key, uint32_t zero)
+                                                                  const uint8_t* keep_u, const uint8_t* keep_v, const uint16_t* slot_u, const uint16_t* slot_v,
+                                                                  uint32_t slots_u, uint32_t slots_v, uint8_t* RP, uint8_t* RQ, uint64_t key, uint32_t zero)
 {
     using T = typename std::conditional<BYTES == 8, uint64_t, typename std::conditional<BYTES == 4, uint32_t, uint16_t>::type>::type;
     constexpr int kDepth = 4;
@@ -408,17 +409,20 @@ __global__ __launch_bounds__(kBlock) void row_traffic_probe_kernel(const mf_node
     const uint32_t worker = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
     const uint64_t begin64 = (uint64_t)worker * per_worker;
     if (begin64 >= n) return;
+    const uint32_t xcd = xcd_id();
     const uint32_t begin = (uint32_t)begin64, end = (uint64_t)begin + per_worker < n ? begin + per_worker : n;
     for (uint32_t base = begin; base < end; base += kWave) {
-        uint32_t mu = 0, mv = 0, keep = 0;
+        uint32_t mu = 0, mv = 0, keep = 0;      // keep: bit0/bit1 write the P/Q row back, bit2/bit3 the row is this XCD's copy of a replicated row
         if (base + (uint32_t)lane < end) {
             const Rating x = load_rating(R, base + (uint32_t)lane);
             mu = x.u; mv = x.v; keep = 3u;
             if (keep_u) {
                 const uint32_t rnd = (uint32_t)(mix64(key ^ (((uint64_t)(base + (uint32_t)lane) << 20) ^ (uint64_t)worker ^ 0x7468696eull)) >> 40);
                 const uint32_t ku = keep_u[mu], kv = keep_v[mv];
-                if (ku != 255u && (((rnd & 0xfffu) * 255u) >> 12) > ku) keep &= ~1u;
-                if (kv != 255u && (((rnd >> 12) * 255u) >> 12) > kv) keep &= ~2u;
+                if (ku == kKeepReplicated || ku == kKeepReplicatedAdded) { keep |= 4u; mu = xcd * slots_u + slot_u[mu]; }
+                else if (ku != 255u && (((rnd & 0xfffu) * 255u) >> 12) > ku) keep &= ~1u;
+                if (kv == kKeepReplicated || kv == kKeepReplicatedAdded) { keep |= 8u; mv = xcd * slots_v + slot_v[mv]; }
+                else if (kv != 255u && (((rnd >> 12) * 255u) >> 12) > kv) keep &= ~2u;
             }
         }
         const int cnt = end - base < (uint32_t)kWave ? (int)(end - base) : kWave;
@@ -428,14 +432,15 @@ __global__ __launch_bounds__(kBlock) void row_traffic_probe_kernel(const mf_node
             for (int d = 0; d < kDepth; ++d) {
                 const int j = j0 + d < cnt ? j0 + d : cnt - 1;
                 kp[d] = j0 + d < cnt ? bcast(keep, j) : 0u;
-                pa[d] = reinterpret_cast<T*>(P + (size_t)bcast(mu, j) * (kWave * BYTES)) + lane;
-                pb[d] = reinterpret_cast<T*>(Q + (size_t)bcast(mv, j) * (kWave * BYTES)) + lane;
+                const uint32_t flags = bcast(keep, j);
+                pa[d] = reinterpret_cast<T*>(((flags & 4u) ? RP : P) + (size_t)bcast(mu, j) * (kWave * BYTES)) + lane;
+                pb[d] = reinterpret_cast<T*>(((flags & 8u) ? RQ : Q) + (size_t)bcast(mv, j) * (kWave * BYTES)) + lane;
                 a[d] = row_load(pa[d]); b[d] = row_load(pb[d]);
             }
 #pragma unroll
             for (int d = 0; d < kDepth; ++d) {
-                if (kp[d] & 1u) row_store<COH>(pa[d], (T)(a[d] + (T)zero));
-                if (kp[d] & 2u) row_store<COH>(pb[d], (T)(b[d] + (T)zero));
+                if (kp[d] & 4u) row_store<false>(pa[d], (T)(a[d] + (T)zero)); else if (kp[d] & 1u) row_store<COH>(pa[d], (T)(a[d] + (T)zero));
+                if (kp[d] & 8u) row_store<false>(pb[d], (T)(b[d] + (T)zero)); else if (kp[d] & 2u) row_store<COH>(pb[d], (T)(b[d] + (T)zero));
             }
         }
     }
@@ -602,19 +607,25 @@ int mf_matrix_reconst_triplet(mf_node* R, const uint32_t* user2sorted_idx, const
 }
 
 int mf_row_traffic_probe(const mf_node* R, uint32_t n, void* p, void* q, uint32_t row_bytes, uint32_t num_workers,
-                         const uint8_t* user_keep, const uint8_t* item_keep, uint64_t seed, int coherent, void* stream)
+                         uint64_t seed, void* stream, const mf_hogwild_options* options)
 {
     if (n == 0) return MF_OK;
     if (!R || !p || !q) return invalid("mf_row_traffic_probe: null pointer");
     if (row_bytes != 128 && row_bytes != 256 && row_bytes != 512) return invalid("mf_row_traffic_probe: row_bytes must be 128, 256 or 512 (got %u)", row_bytes);
     if (num_workers == 0) return invalid("mf_row_traffic_probe: num_workers must be positive");
-    if ((user_keep == nullptr) != (item_keep == nullptr)) return invalid("mf_row_traffic_probe: give both keep tables or neither");
+    mf_hogwild_options o = {};
+    if (options) o = *options;
+    if ((o.user_keep == nullptr) != (o.item_keep == nullptr)) return invalid("mf_row_traffic_probe: give both keep tables or neither");
+    if ((o.user_slots && (!o.user_slot || !o.user_replicas)) || (o.item_slots && (!o.item_slot || !o.item_replicas))) return invalid("mf_row_traffic_probe: replicated rows need slot tables and replica arrays");
     if ((reinterpret_cast<uintptr_t>(p) | reinterpret_cast<uintptr_t>(q)) & 7) return invalid("mf_row_traffic_probe: rows must be 8-byte aligned");
+    const bool coherent = o.cached_rows == 0;
+    const uint8_t* user_keep = o.user_keep; const uint8_t* item_keep = o.item_keep;
     const uint32_t per_worker = (uint32_t)(((uint64_t)n + num_workers - 1) / num_workers);
     const dim3 grid((num_workers + kWavesPerBlock - 1) / kWavesPerBlock), block(kBlock);
     uint8_t* P = static_cast<uint8_t*>(p); uint8_t* Q = static_cast<uint8_t*>(q);
+    uint8_t* RP = static_cast<uint8_t*>(o.user_replicas); uint8_t* RQ = static_cast<uint8_t*>(o.item_replicas);
     const uint64_t key = mix64(seed ^ 0x70726f6265ull);
-#define MF_PROBE(BYTES, COH) hipLaunchKernelGGL((row_traffic_probe_kernel<BYTES, COH>), grid, block, 0, as_stream(stream), R, n, P, Q, per_worker, user_keep, item_keep, key, 0u)
+#define MF_PROBE(BYTES, COH) hipLaunchKernelGGL((row_traffic_probe_kernel<BYTES, COH>), grid, block, 0, as_stream(stream), R, n, P, Q, per_worker, user_keep, item_keep, o.user_slot, o.item_slot, o.user_slots, o.item_slots, RP, RQ, key, 0u)
     if (row_bytes == 128) { if (coherent) MF_PROBE(2, true); else MF_PROBE(2, false); }
     else if (row_bytes == 256) { if (coherent) MF_PROBE(4, true); else MF_PROBE(4, false); }
     else { if (coherent) MF_PROBE(8, true); else MF_PROBE(8, false); }

@@ -123,6 +123,7 @@ void hogwild_kernel(Schedule s, typename Rule::Params prm)
     const uint32_t first_wid = (uint32_t)__builtin_amdgcn_readfirstlane((int)(blockIdx.x * waves_per_block + (threadIdx.x >> 6)));
     Rule rule;
     rule.init(prm, smem, lane, first_wid);              // may synchronise the workgroup
+    const uint32_t xcd = HOT ? xcd_id() : 0u;           // which copy of the replicated rows this wavefront works on
     // a launch normally has one wavefront per worker; a launch with fewer wavefronts (the sampled tail of
     // a MASCOT epoch, which keeps per-workgroup statistics in LDS) lets each wavefront play several workers,
     // and may cut every worker's range into s.pieces parts (on chunk boundaries) to even out the wavefronts' loads
@@ -157,7 +158,7 @@ void hogwild_kernel(Schedule s, typename Rule::Params prm)
             return left < (uint32_t)kWave ? (int)left : kWave;
         };
         auto fetch = [&](uint32_t st, uint32_t cc, int nn) -> Rating {
-            Rating x = {0.f, 0u, 0u, 0u};
+            Rating x = {0.f, 0u, 0u, 0u, 0u, 0u};
             if (lane < nn) {
                 uint32_t off = (cc + (uint32_t)lane) % s.nnz;
                 uint32_t idx = st + off;
@@ -167,8 +168,12 @@ void hogwild_kernel(Schedule s, typename Rule::Params prm)
                     const uint32_t rnd = (uint32_t)(mix64(s.epoch_key ^ (((uint64_t)idx << 20) ^ (uint64_t)wid ^ 0x7468696eull)) >> 40);
                     const uint32_t ku = s.keep_u[x.u], kv = s.keep_v[x.v];
                     // two independent draws, uniform over 0..254
-                    if (ku != 255u) x.thin |= (((rnd & 0xfffu) * 255u) >> 12) > ku ? 5u : 4u;
-                    if (kv != 255u) x.thin |= (((rnd >> 12) * 255u) >> 12) > kv ? 10u : 8u;
+                    if (ku == kKeepReplicated || ku == kKeepReplicatedAdded) {
+                        x.thin |= ku == kKeepReplicated ? 16u : 20u; x.ru = kReplicaRow | (xcd * s.slots_u + s.slot_u[x.u]);
+                    } else if (ku != 255u) x.thin |= (((rnd & 0xfffu) * 255u) >> 12) > ku ? 5u : 4u;
+                    if (kv == kKeepReplicated || kv == kKeepReplicatedAdded) {
+                        x.thin |= kv == kKeepReplicated ? 32u : 40u; x.rv = kReplicaRow | (xcd * s.slots_v + s.slot_v[x.v]);
+                    } else if (kv != 255u) x.thin |= (((rnd >> 12) * 255u) >> 12) > kv ? 10u : 8u;
                 }
             }
             return x;
@@ -182,7 +187,7 @@ void hogwild_kernel(Schedule s, typename Rule::Params prm)
             uint32_t nc = c + (uint32_t)n, nite = ite, nstart = start;
             const bool more = nprocessed < range_end;
             int nn = 0;
-            Rating nmy = {0.f, 0u, 0u, 0u};
+            Rating nmy = {0.f, 0u, 0u, 0u, 0u, 0u};
             if (more) {
                 if (nc >= s.update_vector_size) { nc = 0; ++nite; nstart = window_of(nite); }
                 nn = chunk_len(nc, nprocessed);

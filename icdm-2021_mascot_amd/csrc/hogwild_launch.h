@@ -1,5 +1,5 @@
 // Shared by the launcher translation units (one per rule family, so that they compile in parallel): argument checks,
-// the schedule of a call, and the launch of hogwild_kernel<Rule, HOT> for the four (k, coherence) combinations.
+// the schedule and options of a call, and the launch of hogwild_kernel<Rule, HOT> for the four (k, coherence) combinations.
 #pragma once
 #include "mf_host.h"
 #include "hogwild.h"
@@ -9,30 +9,65 @@
 
 namespace mf {
 
-// process-wide settings, defined in hogwild_launch.hip (mf_set_hot_row_thinning, mf_set_row_coherence, mf_set_epoch_splits)
-extern const uint8_t* g_keep_u;
-extern const uint8_t* g_keep_v;
-extern int g_row_coherence;
-extern uint32_t g_epoch_splits;
+// One side's replicated rows: slot s of replica block x (x = 0..kXcds-1) is at replicas + (x * slots + s) * k * 4 bytes
+// and holds a copy of row slot_row[s] in the precision the row is stored in (a binary16 row fills the first half).
+struct ReplicaSide { RowStorage rows; uint8_t* replicas = nullptr; const uint32_t* slot_row = nullptr; uint32_t slots = 0; };
+// merge = false: every replica := the row.  merge = true: the row and every replica := the mean of the replicas.
+int replica_sync(const ReplicaSide& user, const ReplicaSide& item, int k, bool merge, void* stream);
+
+// A call's schedule (what the kernel gets) and the host-side part of its options.
+struct Call {
+    Schedule s;
+    bool coherent = true;           // agent-scope row stores (mf_hogwild_options::cached_rows == 0)
+    uint32_t launches = 1;          // kernel launches the call is cut into
+    uint8_t* rep_u = nullptr;       // replica arrays (mf_hogwild_options::user_replicas / item_replicas)
+    uint8_t* rep_v = nullptr;
+    const uint32_t* slot_row_u = nullptr;
+    const uint32_t* slot_row_v = nullptr;
+    bool replicated() const { return s.slots_u != 0 || s.slots_v != 0; }
+};
 
 static int check_schedule(const char* who, const void* R, uint32_t nnz, int k, uint32_t num_workers,
-                          uint32_t update_count, uint32_t update_vector_size)
+                          uint32_t update_count, uint32_t update_vector_size, const mf_hogwild_options* o)
 {
     if (k != 64 && k != 128) return invalid("%s: k must be 64 or 128 (got %d)", who, k);
     if (!R || nnz == 0) return invalid("%s: empty rating array", who);
     if (num_workers == 0) return invalid("%s: num_workers must be positive", who);
     if ((uint64_t)update_count * update_vector_size > 0xffffffffull) return invalid("%s: update_count*update_vector_size overflows 32 bits", who);
     if ((uint64_t)nnz + update_vector_size > 0xffffffffull) return invalid("%s: nnz + update_vector_size overflows 32 bits", who);
-    (void)update_count;
+    if (o) {
+        if (o->cached_rows > 1) return invalid("%s: options.cached_rows is 0 (device-coherent row stores) or 1 (cached)", who);
+        if (o->launches > 65536) return invalid("%s: options.launches is at most 65536", who);
+        if ((o->user_keep == nullptr) != (o->item_keep == nullptr)) return invalid("%s: options: pass both hot-row tables or neither", who);
+        const bool rep = o->user_slots || o->item_slots;
+        if (rep && !o->user_keep) return invalid("%s: options: replicated rows are marked in the hot-row tables, which are missing", who);
+        if (o->user_slots && (!o->user_slot || !o->user_slot_row || !o->user_replicas)) return invalid("%s: options: user_slots > 0 needs user_slot, user_slot_row and user_replicas", who);
+        if (o->item_slots && (!o->item_slot || !o->item_slot_row || !o->item_replicas)) return invalid("%s: options: item_slots > 0 needs item_slot, item_slot_row and item_replicas", who);
+        if (o->user_slots > 65535u || o->item_slots > 65535u) return invalid("%s: options: at most 65535 replicated rows per side", who);
+        if (rep && ((reinterpret_cast<uintptr_t>(o->user_replicas) | reinterpret_cast<uintptr_t>(o->item_replicas)) & 255u))
+            return invalid("%s: options: replica arrays must be 256-byte aligned", who);
+    }
     return MF_OK;
 }
-static Schedule make_schedule(const mf_node* R, uint32_t nnz, uint32_t num_workers, uint32_t update_count,
-                              uint32_t update_vector_size, uint64_t seed, uint32_t epoch, const uint32_t* window_start)
+static Call make_call(const mf_node* R, uint32_t nnz, uint32_t num_workers, uint32_t update_count, uint32_t update_vector_size,
+                      uint64_t seed, uint32_t epoch, const uint32_t* window_start, const mf_hogwild_options* o)
 {
-    Schedule s;
+    Call c;
+    Schedule& s = c.s;
     s.R = R; s.nnz = nnz; s.num_workers = num_workers; s.update_count = update_count;
-    s.update_vector_size = update_vector_size; s.pieces = 1; s.range_begin = 0; s.range_end = update_count * update_vector_size; s.epoch_key = window_epoch_key(seed, epoch); s.window_start = window_start; s.keep_u = g_keep_u; s.keep_v = g_keep_v;
-    return s;
+    s.update_vector_size = update_vector_size; s.pieces = 1; s.range_begin = 0; s.range_end = update_count * update_vector_size;
+    s.epoch_key = window_epoch_key(seed, epoch); s.window_start = window_start;
+    s.keep_u = nullptr; s.keep_v = nullptr; s.slot_u = nullptr; s.slot_v = nullptr; s.slots_u = 0; s.slots_v = 0;
+    if (o) {
+        c.coherent = o->cached_rows == 0;
+        c.launches = o->launches ? o->launches : 1;
+        s.keep_u = o->user_keep; s.keep_v = o->item_keep;
+        // a side without replicated rows keeps slots = 0; its keep table then must not hold the replicated mark
+        s.slot_u = o->user_slot; s.slot_v = o->item_slot; s.slots_u = o->user_slots; s.slots_v = o->item_slots;
+        c.rep_u = static_cast<uint8_t*>(o->user_replicas); c.rep_v = static_cast<uint8_t*>(o->item_replicas);
+        c.slot_row_u = o->user_slot_row; c.slot_row_v = o->item_slot_row;
+    }
+    return c;
 }
 static inline uint32_t grid_for(uint32_t num_workers) { return (num_workers + kWavesPerBlock - 1) / kWavesPerBlock; }
 
@@ -48,19 +83,31 @@ template <class P> static auto set_lds_stats(P& p, bool v) -> decltype(p.lds_sta
 static void set_lds_stats(...) {}
 
 template <class Rule, bool HOT>
-static int launch_hot(const char* who, const Schedule& s0, const typename Rule::Params& prm0, size_t lds, void* stream, Range r);
+static int launch_hot(const char* who, const Call& c, const typename Rule::Params& prm0, size_t lds, void* stream, Range r);
 // the kernel comes in two builds: with and without the hot-row code (Schedule::keep_u)
 template <class Rule>
-static int launch(const char* who, const Schedule& s0, const typename Rule::Params& prm0, size_t lds, void* stream, Range r)
+static int launch(const char* who, const Call& c, const typename Rule::Params& prm0, size_t lds, void* stream, Range r)
 {
-    return s0.keep_u ? launch_hot<Rule, true>(who, s0, prm0, lds, stream, r) : launch_hot<Rule, false>(who, s0, prm0, lds, stream, r);
+    return c.s.keep_u ? launch_hot<Rule, true>(who, c, prm0, lds, stream, r) : launch_hot<Rule, false>(who, c, prm0, lds, stream, r);
 }
 template <class Rule, bool HOT>
-static int launch_hot(const char* who, const Schedule& s0, const typename Rule::Params& prm0, size_t lds, void* stream, Range r)
+static int launch_hot(const char* who, const Call& c, const typename Rule::Params& prm0, size_t lds, void* stream, Range r)
 {
+    const Schedule& s0 = c.s;
     if (s0.update_count == 0 || s0.update_vector_size == 0 || r.begin >= r.end) return MF_OK;
     Schedule s = s0;
     typename Rule::Params prm = prm0;
+    prm.rep_p = c.rep_u; prm.rep_q = c.rep_v;
+    // Replicated rows: every XCD's copy starts as the row, and after every kernel the row and the copies become the
+    // mean of the copies (a kernel boundary is where the L2s of the XCDs are written back).
+    ReplicaSide ru, rv;
+    const bool replicated = HOT && c.replicated();
+    if (replicated) {
+        Rule::row_storage(prm, ru.rows, rv.rows);
+        ru.replicas = c.rep_u; ru.slot_row = c.slot_row_u; ru.slots = s0.slots_u;
+        rv.replicas = c.rep_v; rv.slot_row = c.slot_row_v; rv.slots = s0.slots_v;
+        if (int rc = replica_sync(ru, rv, Rule::kK, false, stream)) return rc;
+    }
     if (r.stats_lds) {
         s.range_begin = r.begin; s.range_end = r.end;
         prm.accumulate = r.accumulate;
@@ -79,10 +126,11 @@ static int launch_hot(const char* who, const Schedule& s0, const typename Rule::
                                "hipFuncSetAttribute(MaxDynamicSharedMemorySize)")) return rc;
         set_lds_stats(prm, true);
         hipLaunchKernelGGL((hogwild_kernel<Rule, HOT>), dim3(blocks), dim3(kMaxBlock), r.stats_lds, as_stream(stream), s, prm);
-        return launch_status(who);
+        if (int rc = launch_status(who)) return rc;
+        return replicated ? replica_sync(ru, rv, Rule::kK, true, stream) : MF_OK;
     }
-    // ordinary launches, cut into g_epoch_splits pieces on window boundaries
-    uint32_t splits = Rule::kSplittable ? g_epoch_splits : 1;
+    // ordinary launches, cut into c.launches pieces on window boundaries
+    uint32_t splits = Rule::kSplittable ? c.launches : 1;
     const uint32_t first_window = (r.begin + s0.update_vector_size - 1) / s0.update_vector_size, end_window = r.end / s0.update_vector_size;
     const uint32_t windows = end_window > first_window ? end_window - first_window : 0;
     if (splits > windows) splits = windows ? windows : 1;
@@ -96,6 +144,7 @@ static int launch_hot(const char* who, const Schedule& s0, const typename Rule::
         first = false;
         hipLaunchKernelGGL((hogwild_kernel<Rule, HOT>), dim3(grid_for(s.num_workers)), dim3(kBlock), lds, as_stream(stream), s, prm);
         if (int rc = launch_status(who)) return rc;
+        if (replicated) { if (int rc = replica_sync(ru, rv, Rule::kK, true, stream)) return rc; }
     }
     return MF_OK;
 }
@@ -103,16 +152,38 @@ static int launch_hot(const char* who, const Schedule& s0, const typename Rule::
 // Instantiates Rule<K, COH> for the four (k, coherence) combinations; P is the parameter pack type,
 // identical across instantiations apart from the template arguments.
 template <template <int, bool> class Rule, class MakeParams>
-static int launch_k_coh(const char* who, int k, const Schedule& s, MakeParams make, size_t lds, void* stream, Range r)
+static int launch_k_coh(const char* who, int k, const Call& c, MakeParams make, size_t lds, void* stream, Range r)
 {
-    const bool coh = g_row_coherence != 0;
     if (k == 128) {
-        if (coh) { auto a = make(typename Rule<128, true>::Params{}); return launch<Rule<128, true>>(who, s, a, lds, stream, r); }
-        auto a = make(typename Rule<128, false>::Params{}); return launch<Rule<128, false>>(who, s, a, lds, stream, r);
+        if (c.coherent) { auto a = make(typename Rule<128, true>::Params{}); return launch<Rule<128, true>>(who, c, a, lds, stream, r); }
+        auto a = make(typename Rule<128, false>::Params{}); return launch<Rule<128, false>>(who, c, a, lds, stream, r);
     }
-    if (coh) { auto a = make(typename Rule<64, true>::Params{}); return launch<Rule<64, true>>(who, s, a, lds, stream, r); }
-    auto a = make(typename Rule<64, false>::Params{}); return launch<Rule<64, false>>(who, s, a, lds, stream, r);
+    if (c.coherent) { auto a = make(typename Rule<64, true>::Params{}); return launch<Rule<64, true>>(who, c, a, lds, stream, r); }
+    auto a = make(typename Rule<64, false>::Params{}); return launch<Rule<64, false>>(who, c, a, lds, stream, r);
 }
-static Range whole_epoch(const Schedule& s) { Range r; r.begin = 0; r.end = s.range_end; return r; }
+// Updates in flight during a launch of num_workers workers of Rule at this k (the build with the hot-row code and
+// coherent stores, which is what a run with hot-row tables launches): resident wavefronts x ratings per wavefront.
+template <template <int, bool> class Rule>
+static float inflight_updates(int k, uint32_t num_workers, size_t lds)
+{
+    int blocks = 0, dev = 0, cus = 0;
+    hipError_t e = k == 128 ? hipOccupancyMaxActiveBlocksPerMultiprocessor(&blocks, reinterpret_cast<const void*>(&hogwild_kernel<Rule<128, true>, true>), kBlock, lds)
+                            : hipOccupancyMaxActiveBlocksPerMultiprocessor(&blocks, reinterpret_cast<const void*>(&hogwild_kernel<Rule<64, true>, true>), kBlock, lds);
+    if (e != hipSuccess || hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || blocks <= 0 || cus <= 0) {
+        (void)hipGetLastError();
+        return 0.f;
+    }
+    const double resident = (double)blocks * kWavesPerBlock * cus;
+    const double ahead = k == 128 ? Rule<128, true>::kAhead + 1 : Rule<64, true>::kAhead + 1;
+    return (float)(((double)num_workers < resident ? (double)num_workers : resident) * ahead);
+}
+float inflight_sgd(int k, uint32_t num_workers);          // hogwild_launch.hip
+float inflight_mpt(int k, uint32_t num_workers);
+float inflight_mem_quant(int k, uint32_t num_workers);    // launch_mem_quant.hip
+float inflight_muppet(int k, uint32_t num_workers);       // launch_muppet.hip
+float inflight_afp(int k, uint32_t num_workers);          // launch_afp.hip
+float inflight_mascot(int k, uint32_t num_workers, uint32_t user_groups, uint32_t item_groups);   // launch_mascot_plain.hip
+
+static Range whole_epoch(const Call& c) { Range r; r.begin = 0; r.end = c.s.range_end; return r; }
 
 }  // namespace mf

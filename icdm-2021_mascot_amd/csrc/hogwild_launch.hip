@@ -5,15 +5,6 @@
 
 namespace mf {
 
-// hot-row tables (device pointers, see Schedule::keep_u); null = off
-const uint8_t* g_keep_u = nullptr;
-const uint8_t* g_keep_v = nullptr;
-// 0: ordinary write-back row stores, 1: agent-scope coherent row stores (see row_store in mf_device.h)
-int g_row_coherence = 1;
-// number of consecutive kernel launches one call is cut into (each worker's windows are split evenly);
-// a kernel boundary writes back and invalidates the per-XCD L2s, which is how cached row copies of
-// different XCDs are reconciled during an epoch
-uint32_t g_epoch_splits = 1;
 static thread_local char g_error[512] = "";
 void set_error(const char* fmt, ...)
 {
@@ -23,6 +14,77 @@ void set_error(const char* fmt, ...)
     va_end(ap);
 }
 
+
+// ---- replicated rows: copy out, average back -------------------------------------------------------------------
+// One wavefront per replicated row.  merge = 0: every XCD's copy := the row.  merge = 1: the row and every copy := the
+// mean of the copies that differ from the row (an XCD that did not touch its copy -- no workgroup of the launch ran
+// there, or none of its ratings fell on the row -- has nothing to contribute), summed in binary32 in XCD order and
+// rounded once to the row's precision; if no copy differs the row stays as it is.
+struct SyncSide { RowStorage rows; uint8_t* replicas; const uint32_t* slot_row; uint32_t slots; };
+template <int K>
+__global__ __launch_bounds__(kWave) void replica_sync_kernel(SyncSide user, SyncSide item, int merge)
+{
+    constexpr int E = K / kWave;
+    const bool is_item = blockIdx.x >= user.slots;
+    const SyncSide& side = is_item ? item : user;
+    const uint32_t slot = is_item ? blockIdx.x - user.slots : blockIdx.x;
+    const uint32_t row = side.slot_row[slot];
+    uint8_t* master; bool wide;
+    if (side.rows.dense) {
+        wide = side.rows.elem_bytes == 4;
+        master = static_cast<uint8_t*>(side.rows.dense) + (size_t)row * K * side.rows.elem_bytes;
+    } else {
+        uint32_t lo = 0, hi = side.rows.groups - 1;            // min{g : row <= end[g]}
+        while (lo < hi) { const uint32_t mid = (lo + hi) >> 1; if (row <= side.rows.group_end[mid]) hi = mid; else lo = mid + 1; }
+        const uint32_t local = lo ? row - side.rows.group_end[lo - 1] - 1 : row;
+        wide = side.rows.group_prec[lo] != 0;
+        master = static_cast<uint8_t*>(side.rows.group_ptr[lo]) + (size_t)local * K * (wide ? 4u : 2u);
+    }
+    const size_t slot_bytes = (size_t)K * 4u;
+    auto copy_of = [&](uint32_t x) { return side.replicas + ((size_t)x * side.slots + slot) * slot_bytes; };
+    auto load = [&](const uint8_t* at, int e) { return wide ? reinterpret_cast<const float*>(at)[e] : (float)reinterpret_cast<const half_t*>(at)[e]; };
+    auto store = [&](uint8_t* at, int e, float v) { if (wide) reinterpret_cast<float*>(at)[e] = v; else reinterpret_cast<half_t*>(at)[e] = (half_t)v; };
+    float base[E], out[E];
+#pragma unroll
+    for (int j = 0; j < E; ++j) { base[j] = load(master, (int)threadIdx.x + j * kWave); out[j] = base[j]; }
+    if (merge) {
+        float sum[E];
+#pragma unroll
+        for (int j = 0; j < E; ++j) sum[j] = 0.f;
+        uint32_t changed = 0;
+        for (uint32_t x = 0; x < kXcds; ++x) {
+            float v[E]; bool differs = false;
+#pragma unroll
+            for (int j = 0; j < E; ++j) { v[j] = load(copy_of(x), (int)threadIdx.x + j * kWave); differs |= bits(v[j]) != bits(base[j]); }
+            if (__builtin_amdgcn_ballot_w64(differs) != 0ull) {        // wave-uniform: the whole copy counts or does not
+                ++changed;
+#pragma unroll
+                for (int j = 0; j < E; ++j) sum[j] += v[j];
+            }
+        }
+        if (changed) {
+#pragma unroll
+            for (int j = 0; j < E; ++j) { out[j] = sum[j] / (float)changed; store(master, (int)threadIdx.x + j * kWave, out[j]); }
+        }
+    }
+    for (uint32_t x = 0; x < kXcds; ++x) {
+#pragma unroll
+        for (int j = 0; j < E; ++j) store(copy_of(x), (int)threadIdx.x + j * kWave, out[j]);
+    }
+}
+int replica_sync(const ReplicaSide& user, const ReplicaSide& item, int k, bool merge, void* stream)
+{
+    const uint32_t blocks = user.slots + item.slots;
+    if (blocks == 0) return MF_OK;
+    const SyncSide u{user.rows, user.replicas, user.slot_row, user.slots}, v{item.rows, item.replicas, item.slot_row, item.slots};
+    if (k == 128) hipLaunchKernelGGL(replica_sync_kernel<128>, dim3(blocks), dim3(kWave), 0, as_stream(stream), u, v, merge ? 1 : 0);
+    else hipLaunchKernelGGL(replica_sync_kernel<64>, dim3(blocks), dim3(kWave), 0, as_stream(stream), u, v, merge ? 1 : 0);
+    return launch_status("replica_sync");
+}
+
+float inflight_sgd(int k, uint32_t num_workers) { return inflight_updates<SgdRule>(k, num_workers, 0); }
+float inflight_mpt(int k, uint32_t num_workers) { return inflight_updates<MptRule>(k, num_workers, 0); }
+
 }  // namespace mf
 
 using namespace mf;
@@ -31,27 +93,31 @@ extern "C" {
 
 
 int mf_version(void) { return 1; }
-int mf_set_row_coherence(int coherent)
-{
-    if (coherent != 0 && coherent != 1) return invalid("mf_set_row_coherence: 0 (cached) or 1 (device-coherent)");
-    g_row_coherence = coherent;
-    return MF_OK;
-}
-int mf_get_row_coherence(void) { return g_row_coherence; }
-int mf_set_epoch_splits(uint32_t splits)
-{
-    if (splits == 0 || splits > 65536) return invalid("mf_set_epoch_splits: between 1 and 65536");
-    g_epoch_splits = splits;
-    return MF_OK;
-}
-uint32_t mf_get_epoch_splits(void) { return g_epoch_splits; }
-int mf_set_hot_row_thinning(const uint8_t* user_keep, const uint8_t* item_keep)
-{
-    if ((user_keep == nullptr) != (item_keep == nullptr)) return invalid("mf_set_hot_row_thinning: pass both tables or neither");
-    g_keep_u = user_keep; g_keep_v = item_keep;
-    return MF_OK;
-}
 const char* mf_last_error(void) { return g_error; }
+int mf_replica_sync_dense(void* matrix, uint32_t elem_bytes, int k, void* replicas, const uint32_t* slot_row, uint32_t slots, int merge, void* stream)
+{
+    if (k != 64 && k != 128) return invalid("mf_replica_sync_dense: k must be 64 or 128 (got %d)", k);
+    if (elem_bytes != 2 && elem_bytes != 4) return invalid("mf_replica_sync_dense: elem_bytes is 2 (binary16) or 4 (binary32)");
+    if (slots == 0) return MF_OK;
+    if (!matrix || !replicas || !slot_row) return invalid("mf_replica_sync_dense: null pointer");
+    ReplicaSide side, none;
+    side.rows.dense = matrix; side.rows.elem_bytes = elem_bytes; side.replicas = static_cast<uint8_t*>(replicas); side.slot_row = slot_row; side.slots = slots;
+    return replica_sync(side, none, k, merge != 0, stream);
+}
+float mf_hogwild_inflight(uint32_t version, int k, uint32_t num_workers, uint32_t user_groups, uint32_t item_groups)
+{
+    if (k != 64 && k != 128) return 0.f;
+    switch (version) {
+    case 0: case 5: return inflight_sgd(k, num_workers);
+    case 4: return inflight_mpt(k, num_workers);
+    case 3: return inflight_muppet(k, num_workers);
+    case 2: return inflight_afp(k, num_workers);
+    case 7: return inflight_mem_quant(k, num_workers);
+    case 8: return inflight_mascot(k, num_workers, 1, 1);
+    case 1: case 6: return inflight_mascot(k, num_workers, user_groups ? user_groups : 1, item_groups ? item_groups : 1);
+    default: return 0.f;
+    }
+}
 uint32_t mf_mascot_norm_blocks(uint32_t num_workers) { return grid_for(num_workers); }
 
 uint32_t mf_update_count(uint32_t n, uint32_t num_workers, uint32_t update_vector_size)
@@ -80,28 +146,42 @@ uint32_t mf_window_start(uint64_t seed, uint32_t epoch, uint32_t worker, uint32_
     return window_start_rng(window_epoch_key(seed, epoch), worker, ite, nnz);
 }
 
+int mf_single_sgd_hogwild_opt(const mf_node* R, uint32_t nnz, float* p, float* q, int k,
+                              uint32_t num_workers, uint32_t update_count, uint32_t update_vector_size,
+                              float lrate, float lambda,
+                              uint64_t seed, uint32_t epoch, const uint32_t* window_start, void* stream, const mf_hogwild_options* options)
+{
+    if (int rc = check_schedule("mf_single_sgd_hogwild", R, nnz, k, num_workers, update_count, update_vector_size, options)) return rc;
+    if (!p || !q) return invalid("mf_single_sgd_hogwild: null model pointer");
+    const Call c = make_call(R, nnz, num_workers, update_count, update_vector_size, seed, epoch, window_start, options);
+    return launch_k_coh<SgdRule>("mf_single_sgd_hogwild", k, c, [&](auto a) { a.p = p; a.q = q; a.lrate = lrate; a.lambda = lambda; return a; }, 0, stream, whole_epoch(c));
+}
 int mf_single_sgd_hogwild(const mf_node* R, uint32_t nnz, float* p, float* q, int k,
                           uint32_t num_workers, uint32_t update_count, uint32_t update_vector_size,
                           float lrate, float lambda,
                           uint64_t seed, uint32_t epoch, const uint32_t* window_start, void* stream)
 {
-    if (int rc = check_schedule("mf_single_sgd_hogwild", R, nnz, k, num_workers, update_count, update_vector_size)) return rc;
-    if (!p || !q) return invalid("mf_single_sgd_hogwild: null model pointer");
-    Schedule s = make_schedule(R, nnz, num_workers, update_count, update_vector_size, seed, epoch, window_start);
-    return launch_k_coh<SgdRule>("mf_single_sgd_hogwild", k, s, [&](auto a) { a.p = p; a.q = q; a.lrate = lrate; a.lambda = lambda; return a; }, 0, stream, whole_epoch(s));
+    return mf_single_sgd_hogwild_opt(R, nnz, p, q, k, num_workers, update_count, update_vector_size, lrate, lambda, seed, epoch, window_start, stream, nullptr);
 }
 
+int mf_mpt_sgd_hogwild_opt(const mf_node* R, uint32_t nnz, float* p, float* q, int k,
+                           uint32_t num_workers, uint32_t update_count, uint32_t update_vector_size,
+                           float lrate, uint16_t scaled_lambda_half, float scaling_factor,
+                           uint64_t seed, uint32_t epoch, const uint32_t* window_start, void* stream, const mf_hogwild_options* options)
+{
+    if (int rc = check_schedule("mf_mpt_sgd_hogwild", R, nnz, k, num_workers, update_count, update_vector_size, options)) return rc;
+    if (!p || !q) return invalid("mf_mpt_sgd_hogwild: null model pointer");
+    if (!(scaling_factor > 0)) return invalid("mf_mpt_sgd_hogwild: scaling_factor must be positive");
+    const Call c = make_call(R, nnz, num_workers, update_count, update_vector_size, seed, epoch, window_start, options);
+    return launch_k_coh<MptRule>("mf_mpt_sgd_hogwild", k, c, [&](auto a) {
+        a.p = p; a.q = q; a.lrate = lrate; a.scaled_lambda_half = scaled_lambda_half; a.scaling_factor = scaling_factor; return a; }, 0, stream, whole_epoch(c));
+}
 int mf_mpt_sgd_hogwild(const mf_node* R, uint32_t nnz, float* p, float* q, int k,
                        uint32_t num_workers, uint32_t update_count, uint32_t update_vector_size,
                        float lrate, uint16_t scaled_lambda_half, float scaling_factor,
                        uint64_t seed, uint32_t epoch, const uint32_t* window_start, void* stream)
 {
-    if (int rc = check_schedule("mf_mpt_sgd_hogwild", R, nnz, k, num_workers, update_count, update_vector_size)) return rc;
-    if (!p || !q) return invalid("mf_mpt_sgd_hogwild: null model pointer");
-    if (!(scaling_factor > 0)) return invalid("mf_mpt_sgd_hogwild: scaling_factor must be positive");
-    Schedule s = make_schedule(R, nnz, num_workers, update_count, update_vector_size, seed, epoch, window_start);
-    return launch_k_coh<MptRule>("mf_mpt_sgd_hogwild", k, s, [&](auto a) {
-        a.p = p; a.q = q; a.lrate = lrate; a.scaled_lambda_half = scaled_lambda_half; a.scaling_factor = scaling_factor; return a; }, 0, stream, whole_epoch(s));
+    return mf_mpt_sgd_hogwild_opt(R, nnz, p, q, k, num_workers, update_count, update_vector_size, lrate, scaled_lambda_half, scaling_factor, seed, epoch, window_start, stream, nullptr);
 }
 
 }  // extern "C"

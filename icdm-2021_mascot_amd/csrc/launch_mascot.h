@@ -7,7 +7,7 @@ namespace mf {
 
 // What one mf_mascot_sgd_hogwild call carries to its launches.
 struct MascotCall {
-    const char* who; int k; Schedule s; size_t lds; void* stream;
+    const char* who; int k; Call c; size_t lds; void* stream;
     void* const* p; void* const* q;
     const uint32_t* user_end; const uint32_t* item_end;
     const uint8_t* user_prec; const uint8_t* item_prec;

@@ -5,17 +5,17 @@ using namespace mf;
 
 extern "C" {
 
-int mf_mascot_sgd_hogwild(const mf_node* R, uint32_t nnz, void* const* p, void* const* q, int k,
-                          uint32_t num_workers, uint32_t update_count, uint32_t update_vector_size,
-                          float lrate, float lambda,
-                          const uint32_t* user_group_end_idx, const uint32_t* item_group_end_idx,
-                          const uint8_t* user_group_prec_info, const uint8_t* item_group_prec_info,
-                          float* grad_sum_norm_p, float* grad_sum_norm_q, float* norm_sum_p, float* norm_sum_q,
-                          uint32_t first_sample_rating_idx, uint32_t user_group_num, uint32_t item_group_num,
-                          uint64_t seed, uint32_t epoch, const uint32_t* window_start, void* stream)
+int mf_mascot_sgd_hogwild_opt(const mf_node* R, uint32_t nnz, void* const* p, void* const* q, int k,
+                              uint32_t num_workers, uint32_t update_count, uint32_t update_vector_size,
+                              float lrate, float lambda,
+                              const uint32_t* user_group_end_idx, const uint32_t* item_group_end_idx,
+                              const uint8_t* user_group_prec_info, const uint8_t* item_group_prec_info,
+                              float* grad_sum_norm_p, float* grad_sum_norm_q, float* norm_sum_p, float* norm_sum_q,
+                              uint32_t first_sample_rating_idx, uint32_t user_group_num, uint32_t item_group_num,
+                              uint64_t seed, uint32_t epoch, const uint32_t* window_start, void* stream, const mf_hogwild_options* options)
 {
     const char* who = "mf_mascot_sgd_hogwild";
-    if (int rc = check_schedule(who, R, nnz, k, num_workers, update_count, update_vector_size)) return rc;
+    if (int rc = check_schedule(who, R, nnz, k, num_workers, update_count, update_vector_size, options)) return rc;
     if (!p || !q || !user_group_end_idx || !item_group_end_idx || !user_group_prec_info || !item_group_prec_info)
         return invalid("%s: null group table", who);
     if (!grad_sum_norm_p || !grad_sum_norm_q || !norm_sum_p || !norm_sum_q) return invalid("%s: null statistics buffer", who);
@@ -25,15 +25,14 @@ int mf_mascot_sgd_hogwild(const mf_node* R, uint32_t nnz, void* const* p, void* 
     if (lds > 64 * 1024) return invalid("%s: group tables need %zu bytes of LDS (limit 65536)", who, lds);
     MascotCall c;
     c.who = who; c.k = k; c.lds = lds; c.stream = stream;
-    c.s = make_schedule(R, nnz, num_workers, update_count, update_vector_size, seed, epoch, window_start);
+    c.c = make_call(R, nnz, num_workers, update_count, update_vector_size, seed, epoch, window_start, options);
     c.p = p; c.q = q; c.user_end = user_group_end_idx; c.item_end = item_group_end_idx;
     c.user_prec = user_group_prec_info; c.item_prec = item_group_prec_info;
     c.grad_sum_p = grad_sum_norm_p; c.grad_sum_q = grad_sum_norm_q; c.norm_sum_p = norm_sum_p; c.norm_sum_q = norm_sum_q;
     c.first_sample = first_sample_rating_idx; c.user_groups = user_group_num; c.item_groups = item_group_num;
     c.lrate = lrate; c.lambda = lambda; c.norm_stride = grid_for(num_workers);
-    const Schedule& s = c.s;
-    const uint32_t total = s.range_end;
-    Range body = whole_epoch(s);
+    const uint32_t total = c.c.s.range_end;
+    Range body = whole_epoch(c.c);
     if (first_sample_rating_idx >= total)                     // nothing is sampled: the kernel without the statistics code
         return launch_mascot_plain(c, body);
     // A check epoch.  The sampled ratings [first_sample, total) run as their own launch with the gradient sums in
@@ -46,6 +45,19 @@ int mf_mascot_sgd_hogwild(const mf_node* R, uint32_t nnz, void* const* p, void* 
     Range tail;
     tail.begin = first_sample_rating_idx; tail.end = total; tail.accumulate = body.begin < body.end; tail.stats_lds = need;
     return launch_mascot_sampled(c, tail);
+}
+int mf_mascot_sgd_hogwild(const mf_node* R, uint32_t nnz, void* const* p, void* const* q, int k,
+                          uint32_t num_workers, uint32_t update_count, uint32_t update_vector_size,
+                          float lrate, float lambda,
+                          const uint32_t* user_group_end_idx, const uint32_t* item_group_end_idx,
+                          const uint8_t* user_group_prec_info, const uint8_t* item_group_prec_info,
+                          float* grad_sum_norm_p, float* grad_sum_norm_q, float* norm_sum_p, float* norm_sum_q,
+                          uint32_t first_sample_rating_idx, uint32_t user_group_num, uint32_t item_group_num,
+                          uint64_t seed, uint32_t epoch, const uint32_t* window_start, void* stream)
+{
+    return mf_mascot_sgd_hogwild_opt(R, nnz, p, q, k, num_workers, update_count, update_vector_size, lrate, lambda, user_group_end_idx, item_group_end_idx,
+                                     user_group_prec_info, item_group_prec_info, grad_sum_norm_p, grad_sum_norm_q, norm_sum_p, norm_sum_q,
+                                     first_sample_rating_idx, user_group_num, item_group_num, seed, epoch, window_start, stream, nullptr);
 }
 
 }  // extern "C"

@@ -6,7 +6,7 @@ namespace mf {
 
 int launch_mascot_sampled(const MascotCall& c, Range r)
 {
-    return launch_k_coh<MascotRule>(c.who, c.k, c.s, [&](auto a) { return c.fill(a); }, c.lds, c.stream, r);
+    return launch_k_coh<MascotRule>(c.who, c.k, c.c, [&](auto a) { return c.fill(a); }, c.lds, c.stream, r);
 }
 
 }  // namespace mf

@@ -1,7 +1,10 @@
 // quantized_mf: the reference's command line (main.cu:15-175) over libmascot_hip.
 // Same flags, same stdout lines, same model files.  Additions: `-seed <n>` (the reference seeds from
 // time(0) and clock(), so two of its runs never agree; here the default seed is fixed), `-cached <0|1>`
-// and `-split <n>` (row access policy and kernel launches per epoch, see include/mascot_hip.h), `-synth <c>[,<n>]`
+// and `-split <n>` (row access policy and kernel launches per epoch, see include/mascot_hip.h), `-hot <0|1>`,
+// `-replicate <t>[,<merges>]` and `-thin <cap>[,<early cap>,<epochs>]` (how rows with several updates in flight are
+// treated: mf_params.hot_rows, replicate_inflight, hot_row_inflight; `-hot 0` is the reference's race semantics),
+// `-synth <c>[,<n>]`
 // (no input files: the seeded synthetic stand-in of BASELINE configuration c, optionally with n training ratings
 // and the test set scaled alike, generated on the device; mf_generate_ratings).
 #include <sys/stat.h>
@@ -50,7 +53,17 @@ int main(int argc, const char* argv[])
             if (a == "-seed" && has) prm.seed = std::strtoull(argv[i + 1], nullptr, 10);
             if (a == "-cached" && has) prm.cached_rows = std::atoi(argv[i + 1]);
             if (a == "-split" && has) prm.epoch_splits = std::atoi(argv[i + 1]);
-            if (a == "-hot" && has) {            // <steady cap>[,<early cap>,<early epochs>]
+            if (a == "-hot" && has) {            // 0: no hot rows at all, every row stored as the reference does; 1 (default): hot rows
+                prm.hot_rows = std::atoi(argv[i + 1]) != 0;
+                if (!prm.hot_rows) { prm.replicate_inflight = 0; prm.hot_row_inflight = 0; }
+            }
+            if (a == "-replicate" && has) {      // <updates in flight above which a row gets a copy per XCD; 0 = none>[,<merges per epoch>]
+                float above = 0; unsigned merges = 0;
+                const int got = std::sscanf(argv[i + 1], "%f,%u", &above, &merges);
+                if (got >= 1) prm.replicate_inflight = above;
+                if (got >= 2) prm.replica_merges = merges;
+            }
+            if (a == "-thin" && has) {           // opt-in thinning of hot rows: <steady cap>[,<early cap>,<early epochs>]
                 float steady = 0, early = 0; unsigned ep = 0;
                 const int got = std::sscanf(argv[i + 1], "%f,%f,%u", &steady, &early, &ep);
                 if (got >= 1) prm.hot_row_inflight = steady;
@@ -88,6 +101,16 @@ int main(int argc, const char* argv[])
     std::cout << "Error threshold             : " << prm.error_threshold << std::endl;
     std::cout << "Interval                    : " << prm.interval << std::endl;
     std::cout << "Seed                        : " << prm.seed << std::endl;
+    std::cout << "Hot rows                    : ";
+    if (!prm.hot_rows && !(prm.replicate_inflight != 0) && !(prm.hot_row_inflight > 0)) std::cout << "off (every row stored as the reference does; -hot 0)";
+    else {
+        std::cout << "updates of rows with more than one update in flight are added";
+        if (prm.replicate_inflight < 0) std::cout << "; rows above 0.3 / (learning rate x mean rating) in flight are replicated per XCD";
+        else if (prm.replicate_inflight > 0) std::cout << "; rows above " << prm.replicate_inflight << " in flight are replicated per XCD";
+        if (prm.replicate_inflight != 0) std::cout << ", merged " << prm.replica_merges << " times per epoch";
+        if (prm.hot_row_inflight > 0) std::cout << "; rows above " << prm.hot_row_inflight << " in flight are thinned";
+    }
+    std::cout << std::endl;
 
     Dataset d;
     bool from_cache = false;

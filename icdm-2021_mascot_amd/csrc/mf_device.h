@@ -199,10 +199,41 @@ struct Schedule {
     // the memory side.
     const uint8_t* keep_u;
     const uint8_t* keep_v;
+    // Replicated rows (optional, with the hot-row tables).  A row whose keep value is kKeepReplicated has one copy per
+    // XCD: the wavefronts of XCD x read and write copy x (slot slot_u[row] of replica block x) with ordinary cached
+    // accesses -- the copy lives in that XCD's L2, where the 32 CUs of the XCD race on it as the reference's
+    // workers race on a row, every update carried out -- and the copies are averaged between kernel launches
+    // (replica_sync_kernel).  With kKeepReplicatedAdded (rows with few updates in flight per XCD) the update is added
+    // to the copy instead, so that the XCD's concurrent updates add up; the hottest rows (kKeepReplicated) use neither
+    // atomics nor write-through stores, so nothing of them serialises at the memory side.
+    const uint16_t* slot_u;
+    const uint16_t* slot_v;
+    uint32_t slots_u, slots_v;      // replica rows per XCD and side
+};
+constexpr uint32_t kKeepReplicated = 253u;   // keep-table value of a replicated row whose updates are stored
+constexpr uint32_t kKeepReplicatedAdded = 252u;   // ... whose updates are added to this XCD's copy
+constexpr uint32_t kKeepThinnedMax = 251u;   // largest keep value of a thinned row
+constexpr uint32_t kReplicaRow = 0x80000000u; // Rating::ru / rv: the row is replica row (value & ~kReplicaRow) of the replica array
+constexpr uint32_t kXcds = 8u;                // replica blocks: one per XCD of an MI355X
+
+// Where the rows of one side of the model live, for the kernel that copies them to and from their per-XCD replicas:
+// a dense matrix [rows][k] of elem_bytes-wide elements, or the grouped storage of the MASCOT kernel.
+struct RowStorage {
+    void* dense = nullptr; uint32_t elem_bytes = 4;
+    void* const* group_ptr = nullptr; const uint32_t* group_end = nullptr; const uint8_t* group_prec = nullptr; uint32_t groups = 0;
 };
 
+// Index of the XCD this wavefront runs on (hardware register XCC_ID, bits 3:0).
+__device__ __forceinline__ uint32_t xcd_id()
+{
+    return (uint32_t)__builtin_amdgcn_s_getreg(20 /* HW_REG_XCC_ID */ | (0 << 6) | (3 << 11)) & (kXcds - 1u);
+}
+
 // One lane's rating of a 64-rating chunk; the stream is read once per epoch, so bypass-style loads.
-struct Rating { float r; uint32_t u; uint32_t v; uint32_t thin; };   // thin: bit0/bit1 skip the P/Q update, bit2/bit3 the P/Q row is a hot row (updates are added)
+// thin: bit0/bit1 skip the P/Q update, bit2/bit3 the P/Q row is a hot row (updates are added), bit4/bit5 the P/Q row is
+// a replicated row (the update goes to this XCD's copy: an ordinary cached store, or an add when bit2/bit3 is set as
+// well).  ru, rv: the row to address -- u, v themselves, or kReplicaRow | index of the replica row.
+struct Rating { float r; uint32_t u; uint32_t v; uint32_t thin; uint32_t ru; uint32_t rv; };
 __device__ __forceinline__ Rating load_rating(const mf_node* R, uint32_t idx)
 {
     const uint32_t* w = reinterpret_cast<const uint32_t*>(R + idx);
@@ -211,6 +242,7 @@ __device__ __forceinline__ Rating load_rating(const mf_node* R, uint32_t idx)
     x.u = __builtin_nontemporal_load(w + 1);
     x.v = __builtin_nontemporal_load(w + 2);
     x.thin = 0u;
+    x.ru = x.u; x.rv = x.v;
     return x;
 }
 

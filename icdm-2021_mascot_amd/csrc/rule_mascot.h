@@ -39,7 +39,15 @@ template <int K, bool COH, bool SAMPLED> struct MascotRuleT {
         float lrate; float lambda; bool accumulate;
         uint32_t norm_stride;     // columns per group in norm_sum_* (workgroups of an ordinary launch)
         bool lds_stats;           // sampled gradient sums are kept per workgroup in LDS and flushed once
+        void* rep_p; void* rep_q; // replica rows (Schedule::slot_u): slots of kReplicaSlotBytes, a binary16 row in the first half
     };
+    static constexpr uint32_t kReplicaSlotBytes = K * 4u;
+    static constexpr int kK = K;
+    static void row_storage(const Params& a, RowStorage& u, RowStorage& v)
+    {
+        u.group_ptr = a.p; u.group_end = a.user_end; u.group_prec = a.user_prec; u.groups = a.user_groups;
+        v.group_ptr = a.q; v.group_end = a.item_end; v.group_prec = a.item_prec; v.groups = a.item_groups;
+    }
     static constexpr bool kSplittable = true;
     // raw row registers: binary16 rows use r[0] only
     struct Row { uint32_t p[E], q[E]; };
@@ -58,6 +66,7 @@ template <int K, bool COH, bool SAMPLED> struct MascotRuleT {
     uint32_t* ulock_s; uint32_t* ilock_s; // with them: one lock per group (add_sums_locked)
     uint32_t first_sample, user_groups, item_groups;
     float lrate, lambda;
+    uint64_t rep_p, rep_q;
     int lane;
     // Sampled sums of the most popular group of each side (the last one; with Zipf-like data it takes half of all
     // ratings) stay in registers and reach the shared sums once per wavefront: one contended group lock less.
@@ -88,6 +97,7 @@ template <int K, bool COH, bool SAMPLED> struct MascotRuleT {
         }
         grad_sum_p = a.grad_sum_p; grad_sum_q = a.grad_sum_q;
         first_sample = a.first_sample; lrate = a.lrate; lambda = a.lambda;
+        rep_p = reinterpret_cast<uint64_t>(a.rep_p); rep_q = reinterpret_cast<uint64_t>(a.rep_q);
         for (int e = 0; e < E; ++e) { top_gp[e] = 0.f; top_gq[e] = 0.f; }
         top_np = 0.f; top_nq = 0.f;
         ugrad_s = nullptr; igrad_s = nullptr; ulock_s = nullptr; ilock_s = nullptr;
@@ -124,6 +134,9 @@ template <int K, bool COH, bool SAMPLED> struct MascotRuleT {
             // a rating that is skipped carries null pointers: forward() then matches it with no row
             pr.pptr = ok ? pptr_s[ug] + (uint64_t)urow * (K * (up ? 4u : 2u)) : 0ull;
             pr.qptr = ok ? qptr_s[ig] + (uint64_t)irow * (K * (ip ? 4u : 2u)) : 0ull;
+            // a replicated row: this XCD's copy, in the precision of the row's group
+            if (ok && (my.ru & kReplicaRow)) pr.pptr = rep_p + (uint64_t)(my.ru & ~kReplicaRow) * kReplicaSlotBytes;
+            if (ok && (my.rv & kReplicaRow)) pr.qptr = rep_q + (uint64_t)(my.rv & ~kReplicaRow) * kReplicaSlotBytes;
             pr.flags = up | (ip << 1) | (ok ? 0u : kSkip) | (ug << 3) | (ig << 17);
         }
         return pr;
@@ -176,14 +189,14 @@ template <int K, bool COH, bool SAMPLED> struct MascotRuleT {
 #pragma unroll
         for (int e = 0; e < E; ++e) row_add((reinterpret_cast<float*>(ptr) + lane * E + e), d[e]);
     }
-    static __device__ __forceinline__ void store_side(const uint32_t* r, uint64_t ptr, bool fp32, int lane)
+    template <bool C = COH> static __device__ __forceinline__ void store_side(const uint32_t* r, uint64_t ptr, bool fp32, int lane)
     {
         if (fp32) {
-            if constexpr (E == 2) row_store<COH>((reinterpret_cast<uint64_t*>(ptr) + lane), (uint64_t)r[0] | ((uint64_t)r[1] << 32));
-            else row_store<COH>((reinterpret_cast<uint32_t*>(ptr) + lane), r[0]);
+            if constexpr (E == 2) row_store<C>((reinterpret_cast<uint64_t*>(ptr) + lane), (uint64_t)r[0] | ((uint64_t)r[1] << 32));
+            else row_store<C>((reinterpret_cast<uint32_t*>(ptr) + lane), r[0]);
         } else {
-            if constexpr (E == 2) row_store<COH>((reinterpret_cast<uint32_t*>(ptr) + lane), r[0]);
-            else row_store<COH>((reinterpret_cast<uint16_t*>(ptr) + lane), (uint16_t)r[0]);
+            if constexpr (E == 2) row_store<C>((reinterpret_cast<uint32_t*>(ptr) + lane), r[0]);
+            else row_store<C>((reinterpret_cast<uint16_t*>(ptr) + lane), (uint16_t)r[0]);
         }
     }
     template <int CLS> __device__ __forceinline__ void load(Row& row, const Info& i) const
@@ -329,11 +342,13 @@ template <int K, bool COH, bool SAMPLED> struct MascotRuleT {
             const HV gq = ruv * P - lam_h * Q;
             if (!(i.thin & 1u)) {
                 row.p[0] = bits(HV(__builtin_elementwise_fma(lr_h, gp, P)));
-                if (i.thin & 4u) add_side_half(i.pptr, lr_h * gp, lane); else store_side(row.p, i.pptr, false, lane);
+                if ((i.thin & 20u) == 16u) store_side<false>(row.p, i.pptr, false, lane);
+                else if (i.thin & 4u) add_side_half(i.pptr, lr_h * gp, lane); else store_side(row.p, i.pptr, false, lane);
             }
             if (!(i.thin & 2u)) {
                 row.q[0] = bits(HV(__builtin_elementwise_fma(lr_h, gq, Q)));
-                if (i.thin & 8u) add_side_half(i.qptr, lr_h * gq, lane); else store_side(row.q, i.qptr, false, lane);
+                if ((i.thin & 40u) == 32u) store_side<false>(row.q, i.qptr, false, lane);
+                else if (i.thin & 8u) add_side_half(i.qptr, lr_h * gq, lane); else store_side(row.q, i.qptr, false, lane);
             }
             if (sampled) {
                 float g[E];
@@ -364,7 +379,8 @@ template <int K, bool COH, bool SAMPLED> struct MascotRuleT {
             if (!(i.thin & 1u)) {
                 if (up) { for (int e = 0; e < E; ++e) row.p[e] = bits(np_[e]); }
                 else row.p[0] = bits(narrow(np_));
-                if (i.thin & 4u) {
+                if ((i.thin & 20u) == 16u) store_side<false>(row.p, i.pptr, up, lane);
+                else if (i.thin & 4u) {
                     float d[E];
                     for (int e = 0; e < E; ++e) d[e] = lrate * gp[e];
                     if (up) add_side_float(i.pptr, d, lane); else add_side_half(i.pptr, narrow(d), lane);
@@ -373,7 +389,8 @@ template <int K, bool COH, bool SAMPLED> struct MascotRuleT {
             if (!(i.thin & 2u)) {
                 if (ip) { for (int e = 0; e < E; ++e) row.q[e] = bits(nq_[e]); }
                 else row.q[0] = bits(narrow(nq_));
-                if (i.thin & 8u) {
+                if ((i.thin & 40u) == 32u) store_side<false>(row.q, i.qptr, ip, lane);
+                else if (i.thin & 8u) {
                     float d[E];
                     for (int e = 0; e < E; ++e) d[e] = lrate * gq[e];
                     if (ip) add_side_float(i.qptr, d, lane); else add_side_half(i.qptr, narrow(d), lane);

@@ -140,6 +140,7 @@ template <int K, bool COH> struct MuppetRule : DenseBase<K, COH> {
     struct Params {
         float* p; float* q; float lrate; float lambda; uint32_t first_sample;
         float* sum_updated_val; float* sum_norms; uint32_t num_workers; int fwd; int bwd; bool accumulate;
+        void* rep_p; void* rep_q;
     };
     static constexpr bool kSplittable = false;     // per-worker statistics span the whole launch
     float lrate, lambda; uint32_t first_sample; float* sum_updated_val; int fwd, bwd;
@@ -148,7 +149,8 @@ template <int K, bool COH> struct MuppetRule : DenseBase<K, COH> {
 
     __device__ __forceinline__ void init(const Params& a, uint8_t*, int lane_, uint32_t)
     {
-        this->P = a.p; this->Q = a.q; this->lane = lane_; lrate = a.lrate; lambda = a.lambda;
+        this->P = a.p; this->Q = a.q; this->RP = static_cast<float*>(a.rep_p); this->RQ = static_cast<float*>(a.rep_q);
+        this->lane = lane_; lrate = a.lrate; lambda = a.lambda;
         first_sample = a.first_sample; sum_updated_val = a.sum_updated_val; fwd = a.fwd; bwd = a.bwd;
         sum_norms_reg = 0.f;
 #pragma unroll
@@ -302,7 +304,7 @@ template <int K, bool COH> struct AfpRule : DenseBase<K, COH> {
     static constexpr int kAhead = 1, kRing = 4;    // as for MuPPET: three ratings ahead measured no faster (k = 128) or slower (k = 64)
     static constexpr int kMinWavesPerSimd = 6;     // 24 wavefronts per CU: the 6104 workers of a 100M-rating launch all resident (85 VGPRs otherwise: 5)
     static constexpr bool kSplittable = false;    // the per-worker quantiser state lives for one launch
-    struct Params { float* p; float* q; float lrate; float lambda; int afp_epoch; int init_threshold; bool accumulate; };
+    struct Params { float* p; float* q; float lrate; float lambda; int afp_epoch; int init_threshold; bool accumulate; void* rep_p; void* rep_q; };
     float lrate, lambda; int afp_epoch, init_threshold;
     AfpQ uq, iq, bq;
     int upd_u, upd_i, upd_b, cur_iter;
@@ -311,7 +313,8 @@ template <int K, bool COH> struct AfpRule : DenseBase<K, COH> {
 
     __device__ __forceinline__ void init(const Params& a, uint8_t*, int lane_, uint32_t)
     {
-        this->P = a.p; this->Q = a.q; this->lane = lane_; lrate = a.lrate; lambda = a.lambda;
+        this->P = a.p; this->Q = a.q; this->RP = static_cast<float*>(a.rep_p); this->RQ = static_cast<float*>(a.rep_q);
+        this->lane = lane_; lrate = a.lrate; lambda = a.lambda;
         afp_epoch = a.afp_epoch; init_threshold = a.init_threshold;
         uq = AfpQ{0, 0, 0, 0.f}; iq = uq; bq = uq;
         upd_u = upd_i = upd_b = cur_iter = 0; sp = sq = sb = 0.f; upper = lane_ >= 32;

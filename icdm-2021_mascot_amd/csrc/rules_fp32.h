@@ -24,26 +24,36 @@ template <int K, bool COH> struct DenseBase {
     using Info = DenseInfo;
     using Prep = NoPrep;
     static constexpr int kClasses = 1;
+    static constexpr int kK = K;
+    template <class Params> static void row_storage(const Params& a, RowStorage& u, RowStorage& v) { u.dense = a.p; v.dense = a.q; }
     float* P;
     float* Q;
+    float* RP;      // replica rows (Schedule::slot_u), or null
+    float* RQ;
     int lane;
 
     __device__ __forceinline__ Prep prepare(const Rating&, bool) const { return Prep(); }
     __device__ __forceinline__ int classify(const Prep&, bool) const { return 0; }
     static __device__ __forceinline__ Info no_row() { return Info{0.f, 0xffffffffu, 0xffffffffu, 0u}; }   // matches no rating
+    // u, v: the rows to address (Rating::ru, rv); equal values are the same row, which is all forward() needs
     __device__ __forceinline__ Info info(const Rating& my, const Prep&, int j) const
     {
         Info i;
         i.r = bcast(my.r, j);
-        i.u = bcast(my.u, j);
-        i.v = bcast(my.v, j);
+        i.u = bcast(my.ru, j);
+        i.v = bcast(my.rv, j);
         i.thin = bcast(my.thin, j);
         return i;
     }
+    // first element of a row of the matrix or, for a replicated row, of this XCD's copy (wave-uniform: scalar selects)
+    template <class T> static __device__ __forceinline__ T* row_of(T* matrix, T* replicas, uint32_t row)
+    {
+        return ((row & kReplicaRow) ? replicas : matrix) + (size_t)(row & ~kReplicaRow) * K;
+    }
     template <int CLS> __device__ __forceinline__ void load(Row& row, const Info& i) const
     {
-        const float* pp = P + (size_t)i.u * K + lane;
-        const float* qq = Q + (size_t)i.v * K + lane;
+        const float* pp = row_of(P, RP, i.u) + lane;
+        const float* qq = row_of(Q, RQ, i.v) + lane;
 #pragma unroll
         for (int e = 0; e < E; ++e) { row.p[e] = row_load(pp + 64 * e); row.q[e] = row_load(qq + 64 * e); }
     }
@@ -54,19 +64,32 @@ template <int K, bool COH> struct DenseBase {
     // lose more to the dropped stores than the longer look-ahead gives them, and keep their branches.)
     template <bool HOT> __device__ __forceinline__ void store(const Row& row, const Info& i, const float* dp, const float* dq) const
     {
-        float* pp = P + (size_t)i.u * K + lane;
-        float* qq = Q + (size_t)i.v * K + lane;
+        float* prow = row_of(P, RP, i.u);
+        float* qrow = row_of(Q, RQ, i.v);
+        float* pp = prow + lane;
+        float* qq = qrow + lane;
         if constexpr (!HOT) {
 #pragma unroll
             for (int e = 0; e < E; ++e) { row_store<COH>(pp + 64 * e, row.p[e]); row_store<COH>(qq + 64 * e, row.q[e]); }
         } else {
             const bool add_p = (i.thin & 5u) == 4u, add_q = (i.thin & 10u) == 8u;
-            const row_window_t wp = row_window(reinterpret_cast<uint64_t>(P + (size_t)i.u * K), (i.thin & 5u) ? 0u : K * 4u);
-            const row_window_t wq = row_window(reinterpret_cast<uint64_t>(Q + (size_t)i.v * K), (i.thin & 10u) ? 0u : K * 4u);
+            // a replicated row is stored with an ordinary cached store (it stays in this XCD's L2): a second window per
+            // side with that cache policy, open for replicated rows only
+            const row_window_t wp = row_window(reinterpret_cast<uint64_t>(prow), ((i.thin & 5u) || (COH && (i.thin & 16u))) ? 0u : K * 4u);
+            const row_window_t wq = row_window(reinterpret_cast<uint64_t>(qrow), ((i.thin & 10u) || (COH && (i.thin & 32u))) ? 0u : K * 4u);
 #pragma unroll
             for (int e = 0; e < E; ++e) {
                 window_store<COH>(wp, (uint32_t)(lane + 64 * e) * 4u, bits(row.p[e]));
                 window_store<COH>(wq, (uint32_t)(lane + 64 * e) * 4u, bits(row.q[e]));
+            }
+            if constexpr (COH) {
+                const row_window_t rp = row_window(reinterpret_cast<uint64_t>(prow), (i.thin & 20u) == 16u ? K * 4u : 0u);
+                const row_window_t rq = row_window(reinterpret_cast<uint64_t>(qrow), (i.thin & 40u) == 32u ? K * 4u : 0u);
+#pragma unroll
+                for (int e = 0; e < E; ++e) {
+                    window_store<false>(rp, (uint32_t)(lane + 64 * e) * 4u, bits(row.p[e]));
+                    window_store<false>(rq, (uint32_t)(lane + 64 * e) * 4u, bits(row.q[e]));
+                }
             }
             if (add_p) {
 #pragma unroll
@@ -112,12 +135,13 @@ template <int K, bool COH> struct SgdRule : DenseBase<K, COH> {
     static constexpr int E = Base::E;
     static constexpr int kAhead = 3, kRing = 8;
     static constexpr bool kSplittable = true;
-    struct Params { float* p; float* q; float lrate; float lambda; bool accumulate; };
+    struct Params { float* p; float* q; float lrate; float lambda; bool accumulate; void* rep_p; void* rep_q; };
     float lrate, lambda;
 
     __device__ __forceinline__ void init(const Params& a, uint8_t*, int lane_, uint32_t)
     {
-        this->P = a.p; this->Q = a.q; this->lane = lane_; lrate = a.lrate; lambda = a.lambda;
+        this->P = a.p; this->Q = a.q; this->RP = static_cast<float*>(a.rep_p); this->RQ = static_cast<float*>(a.rep_q);
+        this->lane = lane_; lrate = a.lrate; lambda = a.lambda;
     }
     template <int CLS, bool HOT> __device__ __forceinline__ void update(Row& row, const Info& i, uint32_t) const
     {
@@ -148,13 +172,14 @@ template <int K, bool COH> struct MptRule : DenseBase<K, COH> {
     static constexpr int E = Base::E;
     static constexpr int kAhead = 3, kRing = 8;
     static constexpr bool kSplittable = true;
-    struct Params { float* p; float* q; float lrate; uint16_t scaled_lambda_half; float scaling_factor; bool accumulate; };
+    struct Params { float* p; float* q; float lrate; uint16_t scaled_lambda_half; float scaling_factor; bool accumulate; void* rep_p; void* rep_q; };
     float lrate, scaling_factor_rev;
     half_t lambda_h, scaling_factor_h;
 
     __device__ __forceinline__ void init(const Params& a, uint8_t*, int lane_, uint32_t)
     {
-        this->P = a.p; this->Q = a.q; this->lane = lane_; lrate = a.lrate;
+        this->P = a.p; this->Q = a.q; this->RP = static_cast<float*>(a.rep_p); this->RQ = static_cast<float*>(a.rep_q);
+        this->lane = lane_; lrate = a.lrate;
         scaling_factor_rev = 1 / a.scaling_factor;
         scaling_factor_h = (half_t)a.scaling_factor;
         lambda_h = from_bits<half_t>(a.scaled_lambda_half);
@@ -196,17 +221,27 @@ template <int K, bool COH> struct MemQuantRule {
     static constexpr int kClasses = 1;
     static constexpr int kAhead = 3, kRing = 8;
     static constexpr bool kSplittable = true;
-    struct Params { uint16_t* p; uint16_t* q; float lrate; float lambda; bool accumulate; };
-    uint16_t* P; uint16_t* Q; float lrate, lambda; int lane;
+    struct Params { uint16_t* p; uint16_t* q; float lrate; float lambda; bool accumulate; void* rep_p; void* rep_q; };
+    uint16_t* P; uint16_t* Q; uint16_t* RP; uint16_t* RQ; float lrate, lambda; int lane;
 
-    __device__ __forceinline__ void init(const Params& a, uint8_t*, int lane_, uint32_t) { P = a.p; Q = a.q; lrate = a.lrate; lambda = a.lambda; lane = lane_; }
+    __device__ __forceinline__ void init(const Params& a, uint8_t*, int lane_, uint32_t)
+    {
+        P = a.p; Q = a.q; RP = static_cast<uint16_t*>(a.rep_p); RQ = static_cast<uint16_t*>(a.rep_q); lrate = a.lrate; lambda = a.lambda; lane = lane_;
+    }
+    // a replica slot is k * 4 bytes for every rule; a binary16 row fills its first half
+    static __device__ __forceinline__ uint16_t* row_of(uint16_t* matrix, uint16_t* replicas, uint32_t row)
+    {
+        return (row & kReplicaRow) ? replicas + (size_t)(row & ~kReplicaRow) * (2 * K) : matrix + (size_t)row * K;
+    }
+    static constexpr int kK = K;
+    static void row_storage(const Params& a, RowStorage& u, RowStorage& v) { u.dense = a.p; u.elem_bytes = 2; v.dense = a.q; v.elem_bytes = 2; }
     __device__ __forceinline__ Prep prepare(const Rating&, bool) const { return Prep(); }
     __device__ __forceinline__ int classify(const Prep&, bool) const { return 0; }
     static __device__ __forceinline__ Info no_row() { return Info{0.f, 0xffffffffu, 0xffffffffu, 0u}; }
     __device__ __forceinline__ Info info(const Rating& my, const Prep&, int j) const
     {
         Info i;
-        i.r = bcast(my.r, j); i.u = bcast(my.u, j); i.v = bcast(my.v, j); i.thin = bcast(my.thin, j);
+        i.r = bcast(my.r, j); i.u = bcast(my.ru, j); i.v = bcast(my.rv, j); i.thin = bcast(my.thin, j);
         return i;
     }
     __device__ __forceinline__ uint32_t load_side(const uint16_t* row) const
@@ -216,8 +251,8 @@ template <int K, bool COH> struct MemQuantRule {
     }
     template <int CLS> __device__ __forceinline__ void load(Row& row, const Info& i) const
     {
-        row.p = load_side(P + (size_t)i.u * K);
-        row.q = load_side(Q + (size_t)i.v * K);
+        row.p = load_side(row_of(P, RP, i.u));
+        row.q = load_side(row_of(Q, RQ, i.v));
     }
     __device__ __forceinline__ void forward(Row& nxt, const Info& in, const Row& cur, const Info& ic) const
     {
@@ -235,8 +270,13 @@ template <int K, bool COH> struct MemQuantRule {
         else return bits((half_t)f[0]);
     }
     // store the rounded row, or add the rounded change to a hot row
-    __device__ __forceinline__ void write_side(uint16_t* row, uint32_t now, const float* change, bool hot) const
+    __device__ __forceinline__ void write_side(uint16_t* row, uint32_t now, const float* change, bool hot, bool replicated) const
     {
+        if (replicated && !hot) {      // this XCD's copy: an ordinary cached store
+            if constexpr (E == 2) row_store<false>(reinterpret_cast<uint32_t*>(row) + lane, now);
+            else row_store<false>(row + lane, (uint16_t)now);
+            return;
+        }
         if constexpr (E == 2) {
             uint32_t* at = reinterpret_cast<uint32_t*>(row) + lane;
             if (hot) row_add(reinterpret_cast<half2_t*>(at), from_bits<half2_t>(narrow(change)));
@@ -287,8 +327,8 @@ template <int K, bool COH> struct MemQuantRule {
             nq[e] = qf[e] + dq[e];
         }
         // the register copy is what the row holds afterwards: the sum rounded to binary16
-        if (!(i.thin & 1u)) { row.p = narrow(np); write_side(P + (size_t)i.u * K, row.p, dp, i.thin & 4u); }
-        if (!(i.thin & 2u)) { row.q = narrow(nq); write_side(Q + (size_t)i.v * K, row.q, dq, i.thin & 8u); }
+        if (!(i.thin & 1u)) { row.p = narrow(np); write_side(row_of(P, RP, i.u), row.p, dp, i.thin & 4u, i.thin & 16u); }
+        if (!(i.thin & 2u)) { row.q = narrow(nq); write_side(row_of(Q, RQ, i.v), row.q, dq, i.thin & 8u, i.thin & 32u); }
     }
     __device__ __forceinline__ void finish(const Params&, uint32_t) const {}
 };

@@ -15,6 +15,8 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <functional>
+#include <memory>
 #include <string>
 #include <vector>
 #include "mf_host.h"
@@ -60,8 +62,11 @@ struct Common {
     uint32_t n, n_users, n_items, test_n, k;
     uint32_t update_vector_size = 128;       // hard-coded in every driver (mf_methods.cu:100,858)
     uint32_t update_count;
+    float mean_rating = 0.f;                 // mean |rating| of the training set
     DevBuf d_R, d_test, d_sum_sq;
     std::vector<float> lr;
+    std::vector<double> rmse_hist;           // per epoch, whether or not the caller passed a report
+    std::vector<float> ms_hist;
     mf_report* rep;
 };
 
@@ -95,7 +100,7 @@ void fill_schedule(Common& c)
 {
     const mf_params& p = *c.prm;
     c.update_count = mf_update_count(c.n, p.num_workers, c.update_vector_size);
-    c.lr.resize(p.epoch);
+    c.lr.resize(p.epoch); c.rmse_hist.assign(p.epoch, 0.0); c.ms_hist.assign(p.epoch, 0.f);
     for (uint32_t e = 0; e < p.epoch; ++e) c.lr[e] = mf_lr_schedule(p.learning_rate, p.decay, e);
     if (c.rep) {
         c.rep->update_count = c.update_count;
@@ -105,6 +110,7 @@ void fill_schedule(Common& c)
 
 int report_epoch(Common& c, uint32_t e, double rmse, float sgd_ms)
 {
+    c.rmse_hist[e] = rmse; c.ms_hist[e] = sgd_ms;
     if (c.rep) {
         if (c.rep->rmse_per_epoch) c.rep->rmse_per_epoch[e] = rmse;
         if (c.rep->sgd_ms_per_epoch) c.rep->sgd_ms_per_epoch[e] = sgd_ms;
@@ -132,57 +138,106 @@ int dense_rmse(Common& c, const float* d_p, const float* d_q, double* out)
     return finish_rmse(c, out);
 }
 
-// Hot-row table from rating counts (see mf_set_hot_row_thinning): a row with count c has about F*c/n updates in
-// flight (F = resident workers x ratings a worker keeps in flight).  Rows with more than one are hot rows (their
-// updates are added); of those, rows above inflight_cap are thinned to inflight_cap updates in flight.
-std::vector<uint8_t> keep_table(const uint32_t* cnt, uint32_t rows, uint32_t n, uint32_t num_workers, float inflight_cap)
+// Hot-row table of one side from its rating counts (mf_hogwild_options::user_keep): a row with count c has about
+// inflight * c / n updates in flight.  Rows with more than one are hot rows: above replicate_above they get a copy per
+// XCD (numbered in row order; at most 65535, the most popular ones; updates are stored in the copy, or added to it
+// while the XCD's share of them is within add_within), above thin_above they are thinned to that many updates in
+// flight, the rest have their updates added.
+struct KeepTable { std::vector<uint8_t> keep; std::vector<uint16_t> slot; std::vector<uint32_t> slot_row; };
+KeepTable keep_table(const uint32_t* cnt, uint32_t rows, uint32_t n, double inflight, double replicate_above, double thin_above, double add_within = 0)
 {
-    const double resident = num_workers < 8192u ? num_workers : 8192u;      // 256 CUs x 32 wavefronts
-    const double F = resident * 4.0;                                         // three ratings of look-ahead
-    std::vector<uint8_t> t(rows);
+    KeepTable t;
+    t.keep.resize(rows); t.slot.assign(rows, 0);
+    // the 65535 slots go to the highest counts: raise the bar to the count of the 65536th candidate
+    double min_replicated = replicate_above > 0 ? replicate_above : 1e300;
+    if (replicate_above > 0) {
+        std::vector<uint32_t> cand;
+        for (uint32_t r = 0; r < rows; ++r) if (inflight * (double)cnt[r] / (double)n > replicate_above) cand.push_back(cnt[r]);
+        if (cand.size() > 65535u) {
+            std::nth_element(cand.begin(), cand.begin() + 65535, cand.end(), std::greater<uint32_t>());
+            min_replicated = inflight * (double)cand[65535] / (double)n;      // strictly above this one
+        }
+    }
     for (uint32_t r = 0; r < rows; ++r) {
-        const double inflight = F * (double)cnt[r] / (double)n;
-        if (inflight <= 1.0) { t[r] = 255; continue; }
-        const double keep = inflight > inflight_cap ? inflight_cap / inflight : 1.0;
-        const int v = (int)std::floor(keep * 255.0) - 1;
-        t[r] = (uint8_t)(v < 0 ? 0 : (v > 254 ? 254 : v));
+        const double fly = inflight * (double)cnt[r] / (double)n;
+        if (fly <= 1.0) { t.keep[r] = MF_KEEP_ORDINARY; continue; }
+        if (fly > min_replicated && t.slot_row.size() < 65535u) {
+            // each XCD's copy sees an eighth of the row's updates: a caller may have those added to the copy while they
+            // are few (add_within per XCD); otherwise, and above, they are stored (last writer wins inside the XCD)
+            t.keep[r] = fly <= add_within * MF_XCDS ? MF_KEEP_REPLICATED_ADDED : MF_KEEP_REPLICATED;
+            t.slot[r] = (uint16_t)t.slot_row.size(); t.slot_row.push_back(r);
+            continue;
+        }
+        if (thin_above > 0 && fly > thin_above) {
+            const int v = (int)std::floor(thin_above / fly * 255.0) - 1;
+            t.keep[r] = (uint8_t)(v < 0 ? 0 : (v > 251 ? 251 : v));
+            continue;
+        }
+        t.keep[r] = MF_KEEP_ADDED;
     }
     return t;
 }
 
-// The two pairs of hot-row tables of a run: the early cap for the first epochs, while every row still grows from its
-// small initial value and the popular rows need many updates, and the steady cap afterwards.
+// The launch options of a run (mf_hogwild_options) and the device arrays they name: the hot-row tables of both sides
+// -- two pairs when rows are thinned, an early cap for the first epochs, while every row still grows from its small
+// initial value and the popular rows need many updates, and the steady cap afterwards -- and the replica arrays.
 struct HotRows {
-    DevBuf early_u, early_v, steady_u, steady_v;
-    bool active = false;
+    struct SideTables { DevBuf early, steady, slot, slot_row, replicas; uint32_t slots = 0; };
+    SideTables u, v;
+    mf_hogwild_options opt_early{}, opt_steady{};
     uint32_t early_epochs = 0;
-    ~HotRows() { if (active) (void)mf_set_hot_row_thinning(nullptr, nullptr); }
-    static int upload(DevBuf& d, const std::vector<uint8_t>& t)
+    double inflight = 0, replicate_above = 0;
+    static bool wanted(const mf_params& prm) { return prm.hot_rows || prm.hot_row_inflight > 0 || prm.replicate_inflight > 0; }
+    static int upload(DevBuf& d, const void* src, size_t bytes, const char* what)
     {
-        MF_TRY(d.alloc(t.size(), "hipMalloc(hot-row table)"));
-        HIP_TRY(hipMemcpy(d.p, t.data(), t.size(), hipMemcpyHostToDevice), "H2D hot-row table");
+        MF_TRY(d.alloc(bytes, what));
+        if (bytes) HIP_TRY(hipMemcpy(d.p, src, bytes, hipMemcpyHostToDevice), what);
         return 0;
     }
-    int install(const mf_params& prm, const uint32_t* ucnt, uint32_t n_users, const uint32_t* icnt, uint32_t n_items, uint32_t n)
+    int build_side(SideTables& t, const mf_params& prm, const uint32_t* cnt, uint32_t rows, uint32_t n, bool early)
     {
-        if (!(prm.hot_row_inflight > 0)) return 0;
-        early_epochs = prm.hot_row_inflight_early > prm.hot_row_inflight ? prm.hot_row_early_epochs : 0;
-        MF_TRY(upload(steady_u, keep_table(ucnt, n_users, n, prm.num_workers, prm.hot_row_inflight)));
-        MF_TRY(upload(steady_v, keep_table(icnt, n_items, n, prm.num_workers, prm.hot_row_inflight)));
-        if (early_epochs) {
-            MF_TRY(upload(early_u, keep_table(ucnt, n_users, n, prm.num_workers, prm.hot_row_inflight_early)));
-            MF_TRY(upload(early_v, keep_table(icnt, n_items, n, prm.num_workers, prm.hot_row_inflight_early)));
+        const KeepTable steady = keep_table(cnt, rows, n, inflight, replicate_above, prm.hot_row_inflight, prm.replica_add_inflight);
+        MF_TRY(upload(t.steady, steady.keep.data(), rows, "hot-row table"));
+        if (early) {
+            const KeepTable e = keep_table(cnt, rows, n, inflight, replicate_above, prm.hot_row_inflight_early, prm.replica_add_inflight);
+            MF_TRY(upload(t.early, e.keep.data(), rows, "hot-row table"));
         }
-        active = true;
+        t.slots = (uint32_t)steady.slot_row.size();
+        if (t.slots) {
+            MF_TRY(upload(t.slot, steady.slot.data(), (size_t)rows * 2, "replica slots"));
+            MF_TRY(upload(t.slot_row, steady.slot_row.data(), (size_t)t.slots * 4, "replica rows"));
+            MF_TRY(t.replicas.alloc((size_t)MF_XCDS * t.slots * prm.k * 4, "hipMalloc(row replicas)"));
+        }
         return 0;
     }
-    // tables for the launches of epoch e (a launch takes the pointers with it, so switching between launches is safe)
-    int select(uint32_t e)
+    int install(const mf_params& prm, const uint32_t* ucnt, uint32_t n_users, const uint32_t* icnt, uint32_t n_items, uint32_t n,
+                uint32_t user_groups, uint32_t item_groups, float mean_rating)
     {
-        if (!active) return 0;
-        const bool early = e < early_epochs;
-        return mf_set_hot_row_thinning((early ? early_u : steady_u).as<uint8_t>(), (early ? early_v : steady_v).as<uint8_t>());
+        opt_steady = mf_hogwild_options{};
+        opt_steady.cached_rows = prm.cached_rows ? 1u : 0u;
+        opt_steady.launches = prm.epoch_splits ? prm.epoch_splits : 1u;
+        opt_early = opt_steady;
+        if (!wanted(prm)) return 0;
+        inflight = mf_hogwild_inflight(prm.version, (int)prm.k, prm.num_workers, user_groups, item_groups);
+        if (!(inflight > 0)) return invalid("mf_train: cannot determine the number of updates in flight (%s)", mf_last_error());
+        replicate_above = prm.replicate_inflight > 0 ? prm.replicate_inflight : (prm.replicate_inflight < 0 ? mf_replicate_threshold(prm.learning_rate, mean_rating) : 0.0);
+        const bool early = prm.hot_row_inflight > 0 && prm.hot_row_inflight_early > prm.hot_row_inflight && prm.hot_row_early_epochs > 0;
+        early_epochs = early ? prm.hot_row_early_epochs : 0;
+        MF_TRY(build_side(u, prm, ucnt, n_users, n, early));
+        MF_TRY(build_side(v, prm, icnt, n_items, n, early));
+        mf_hogwild_options& o = opt_steady;
+        o.user_keep = u.steady.as<uint8_t>(); o.item_keep = v.steady.as<uint8_t>();
+        o.user_slot = u.slot.as<uint16_t>(); o.item_slot = v.slot.as<uint16_t>();
+        o.user_slot_row = u.slot_row.as<uint32_t>(); o.item_slot_row = v.slot_row.as<uint32_t>();
+        o.user_replicas = u.replicas.p; o.item_replicas = v.replicas.p;
+        o.user_slots = u.slots; o.item_slots = v.slots;
+        if ((u.slots || v.slots) && prm.epoch_splits == 0) o.launches = prm.replica_merges ? prm.replica_merges : 1u;
+        opt_early = o;
+        if (early) { opt_early.user_keep = u.early.as<uint8_t>(); opt_early.item_keep = v.early.as<uint8_t>(); }
+        return 0;
     }
+    // options of the launches of epoch e
+    const mf_hogwild_options* options(uint32_t e) const { return e < early_epochs ? &opt_early : &opt_steady; }
 };
 
 // Whole-model precision switching (-v 8, training_switching_only, mf_methods.cu:1396-1562): the MASCOT kernel with
@@ -218,96 +273,118 @@ struct WholeModel {
     }
 };
 
-// ---- variants over dense P/Q (versions 2..5, 7, 8) ----------------------------------------------
-int train_dense(Common& c, float* p, float* q)
-{
-    const mf_params& prm = *c.prm;
-    const uint32_t version = prm.version == 0 ? 5 : prm.version;
-    const size_t pn = (size_t)c.n_users * c.k, qn = (size_t)c.n_items * c.k;
-    DevBuf d_p, d_q, d_sum_updated, d_sum_norms;
-    MF_TRY(d_p.alloc(pn * 4, "hipMalloc(P)"));
-    MF_TRY(d_q.alloc(qn * 4, "hipMalloc(Q)"));
-    HIP_TRY(hipMemcpy(d_p.p, p, pn * 4, hipMemcpyHostToDevice), "H2D P");
-    HIP_TRY(hipMemcpy(d_q.p, q, qn * 4, hipMemcpyHostToDevice), "H2D Q");
+// A training run as an object: setup() uploads and prepares, epoch(e) runs epoch e (update launches, error estimate,
+// switching, test RMSE), download() brings the model back.  mf_train runs all epochs; the mf_session_* entry points
+// hand the epochs to the caller one at a time.
+struct Run {
+    Common c;
+    mf_params prm;
+    HotRows hot;
+    uint32_t next_epoch = 0;
+    virtual ~Run() {}
+    virtual int setup(const mf_node* R, const mf_node* test, const float* p, const float* q) = 0;
+    virtual int epoch(uint32_t e) = 0;
+    virtual int download(float* p, float* q) = 0;
+};
 
-    // MPT: loss scale 1000, lambda*1000 rounded to binary16 on the host (mf_methods.cu:764-765)
+// ---- variants over dense P/Q (versions 2..5, 7, 8) ----------------------------------------------
+struct DenseRun : Run {
+    uint32_t version = 5;
+    size_t pn = 0, qn = 0;
+    DevBuf d_p, d_q, d_sum_updated, d_sum_norms, d_hp, d_hq;
+    // MPT: loss scale 1000, lambda*1000 rounded to binary16 (mf_methods.cu:764-765)
     const float scaling_factor = 1000;
     uint16_t scaled_lambda_h = 0;
-    if (version == 4) {
-        DevBuf tmp_f, tmp_h;
-        MF_TRY(tmp_f.alloc(8, "hipMalloc")); MF_TRY(tmp_h.alloc(8, "hipMalloc"));
-        const float v[2] = {prm.lambda * scaling_factor, 0.f};
-        HIP_TRY(hipMemcpy(tmp_f.p, v, 8, hipMemcpyHostToDevice), "H2D");
-        MF_TRY(mf_transform_float2half(tmp_f.as<float>(), tmp_h.as<uint16_t>(), 2, nullptr));
-        uint16_t hb[2];
-        HIP_TRY(hipMemcpy(hb, tmp_h.p, 4, hipMemcpyDeviceToHost), "D2H");
-        scaled_lambda_h = hb[0];
-    }
     // MuPPET ladder state (mf_methods.cu:586-601)
     const unsigned char bit_width_set[5] = {8, 12, 14, 16, 32};
-    int precision_idx = prm.is_yahoo ? 1 : 0, switched_epoch = -1, violation_times = 0;
+    int precision_idx = 0, switched_epoch = -1, violation_times = 0;
     float max_grad_diversity = -1.f;
     const int resolution_size = 3, gamma = 1;
-    std::vector<float> sum_norms_epoch(prm.epoch, 0.f), sum_updated_val_epoch((size_t)prm.epoch * c.k, 0.f), sum_norms(prm.num_workers), sum_updated(c.k);
+    std::vector<float> sum_norms_epoch, sum_updated_val_epoch, sum_norms, sum_updated;
     uint32_t muppet_first_sample = 0;
-    if (version == 3) {
-        MF_TRY(d_sum_updated.alloc(c.k * 4, "hipMalloc(sum_updated_val)"));
-        MF_TRY(d_sum_norms.alloc((size_t)prm.num_workers * 4, "hipMalloc(sum_norms)"));
-        const int sample_ratings_num = (int)((float)(c.update_count * c.update_vector_size) * prm.sample_ratio);   // :563
-        muppet_first_sample = c.update_count * c.update_vector_size - (uint32_t)sample_ratings_num;
-    }
-
-    // -v 7: dense binary16 storage next to the fp32 buffers, which then only serve the RMSE and the result
-    DevBuf d_hp, d_hq;
-    if (version == 7) {
-        MF_TRY(d_hp.alloc(pn * 2, "hipMalloc(binary16 P)"));
-        MF_TRY(d_hq.alloc(qn * 2, "hipMalloc(binary16 Q)"));
-        MF_TRY(mf_transform_float2half(d_p.as<float>(), d_hp.as<uint16_t>(), pn, nullptr));
-        MF_TRY(mf_transform_float2half(d_q.as<float>(), d_hq.as<uint16_t>(), qn, nullptr));
-    }
     WholeModel whole;
-    const uint32_t total = c.update_count * c.update_vector_size;
-    const uint32_t whole_sample_num = (uint32_t)(int)((float)total * prm.sample_ratio);       // mf_methods.cu:1425
-    if (version == 8) MF_TRY(whole.init(c, d_p.as<float>(), d_q.as<float>(), prm.num_workers));
-
-    HotRows hot;
-    if (prm.hot_row_inflight > 0) {
-        DevBuf d_ucnt, d_icnt;
-        MF_TRY(d_ucnt.alloc((size_t)c.n_users * 4, "hipMalloc(user counts)"));
-        MF_TRY(d_icnt.alloc((size_t)c.n_items * 4, "hipMalloc(item counts)"));
-        HIP_TRY(hipMemset(d_ucnt.p, 0, (size_t)c.n_users * 4), "memset");
-        HIP_TRY(hipMemset(d_icnt.p, 0, (size_t)c.n_items * 4), "memset");
-        MF_TRY(mf_user_item_histogram(c.d_R.as<mf_node>(), c.n, d_ucnt.as<uint32_t>(), d_icnt.as<uint32_t>(), nullptr));
-        std::vector<uint32_t> ucnt(c.n_users), icnt(c.n_items);
-        HIP_TRY(hipMemcpy(ucnt.data(), d_ucnt.p, (size_t)c.n_users * 4, hipMemcpyDeviceToHost), "D2H user counts");
-        HIP_TRY(hipMemcpy(icnt.data(), d_icnt.p, (size_t)c.n_items * 4, hipMemcpyDeviceToHost), "D2H item counts");
-        MF_TRY(hot.install(prm, ucnt.data(), c.n_users, icnt.data(), c.n_items, c.n));
-    }
+    uint32_t total = 0, whole_sample_num = 0;
     Timer t;
-    const mf_node* R = c.d_R.as<mf_node>();
-    for (uint32_t e = 0; e < prm.epoch; ++e) {
-        MF_TRY(hot.select(e));
+
+    int setup(const mf_node* R, const mf_node* test, const float* p, const float* q) override
+    {
+        version = prm.version == 0 ? 5 : prm.version;
+        pn = (size_t)c.n_users * c.k; qn = (size_t)c.n_items * c.k;
+        MF_TRY(upload_and_shuffle(c, R, test));
+        MF_TRY(d_p.alloc(pn * 4, "hipMalloc(P)"));
+        MF_TRY(d_q.alloc(qn * 4, "hipMalloc(Q)"));
+        HIP_TRY(hipMemcpy(d_p.p, p, pn * 4, hipMemcpyHostToDevice), "H2D P");
+        HIP_TRY(hipMemcpy(d_q.p, q, qn * 4, hipMemcpyHostToDevice), "H2D Q");
+        if (version == 4) {
+            DevBuf tmp_f, tmp_h;
+            MF_TRY(tmp_f.alloc(8, "hipMalloc")); MF_TRY(tmp_h.alloc(8, "hipMalloc"));
+            const float v[2] = {prm.lambda * scaling_factor, 0.f};
+            HIP_TRY(hipMemcpy(tmp_f.p, v, 8, hipMemcpyHostToDevice), "H2D");
+            MF_TRY(mf_transform_float2half(tmp_f.as<float>(), tmp_h.as<uint16_t>(), 2, nullptr));
+            uint16_t hb[2];
+            HIP_TRY(hipMemcpy(hb, tmp_h.p, 4, hipMemcpyDeviceToHost), "D2H");
+            scaled_lambda_h = hb[0];
+        }
+        precision_idx = prm.is_yahoo ? 1 : 0;
+        sum_norms_epoch.assign(prm.epoch, 0.f); sum_updated_val_epoch.assign((size_t)prm.epoch * c.k, 0.f);
+        sum_norms.resize(prm.num_workers); sum_updated.resize(c.k);
+        if (version == 3) {
+            MF_TRY(d_sum_updated.alloc(c.k * 4, "hipMalloc(sum_updated_val)"));
+            MF_TRY(d_sum_norms.alloc((size_t)prm.num_workers * 4, "hipMalloc(sum_norms)"));
+            const int sample_ratings_num = (int)((float)(c.update_count * c.update_vector_size) * prm.sample_ratio);   // :563
+            muppet_first_sample = c.update_count * c.update_vector_size - (uint32_t)sample_ratings_num;
+        }
+        // -v 7: dense binary16 storage next to the fp32 buffers, which then only serve the RMSE and the result
+        if (version == 7) {
+            MF_TRY(d_hp.alloc(pn * 2, "hipMalloc(binary16 P)"));
+            MF_TRY(d_hq.alloc(qn * 2, "hipMalloc(binary16 Q)"));
+            MF_TRY(mf_transform_float2half(d_p.as<float>(), d_hp.as<uint16_t>(), pn, nullptr));
+            MF_TRY(mf_transform_float2half(d_q.as<float>(), d_hq.as<uint16_t>(), qn, nullptr));
+        }
+        total = c.update_count * c.update_vector_size;
+        whole_sample_num = (uint32_t)(int)((float)total * prm.sample_ratio);       // mf_methods.cu:1425
+        if (version == 8) MF_TRY(whole.init(c, d_p.as<float>(), d_q.as<float>(), prm.num_workers));
+
+        std::vector<uint32_t> ucnt, icnt;
+        if (HotRows::wanted(prm)) {
+            DevBuf d_ucnt, d_icnt;
+            MF_TRY(d_ucnt.alloc((size_t)c.n_users * 4, "hipMalloc(user counts)"));
+            MF_TRY(d_icnt.alloc((size_t)c.n_items * 4, "hipMalloc(item counts)"));
+            HIP_TRY(hipMemset(d_ucnt.p, 0, (size_t)c.n_users * 4), "memset");
+            HIP_TRY(hipMemset(d_icnt.p, 0, (size_t)c.n_items * 4), "memset");
+            MF_TRY(mf_user_item_histogram(c.d_R.as<mf_node>(), c.n, d_ucnt.as<uint32_t>(), d_icnt.as<uint32_t>(), nullptr));
+            ucnt.resize(c.n_users); icnt.resize(c.n_items);
+            HIP_TRY(hipMemcpy(ucnt.data(), d_ucnt.p, (size_t)c.n_users * 4, hipMemcpyDeviceToHost), "D2H user counts");
+            HIP_TRY(hipMemcpy(icnt.data(), d_icnt.p, (size_t)c.n_items * 4, hipMemcpyDeviceToHost), "D2H item counts");
+        }
+        return hot.install(prm, ucnt.data(), c.n_users, icnt.data(), c.n_items, c.n, 1, 1, c.mean_rating);
+    }
+
+    int epoch(uint32_t e) override
+    {
+        const mf_node* R = c.d_R.as<mf_node>();
+        const mf_hogwild_options* opt = hot.options(e);
         bool whole_check = false;
         const double err0 = now_ms();
         if (version == 3) HIP_TRY(hipMemsetAsync(d_sum_updated.p, 0, c.k * 4, nullptr), "memset sum_updated_val");
         double err_ms = now_ms() - err0;
         t.start();
         switch (version) {
-        case 5: MF_TRY(mf_single_sgd_hogwild(R, c.n, d_p.as<float>(), d_q.as<float>(), (int)c.k, prm.num_workers, c.update_count, c.update_vector_size,
-                                             c.lr[e], prm.lambda, prm.seed, e, nullptr, nullptr)); break;
-        case 4: MF_TRY(mf_mpt_sgd_hogwild(R, c.n, d_p.as<float>(), d_q.as<float>(), (int)c.k, prm.num_workers, c.update_count, c.update_vector_size,
-                                          c.lr[e], scaled_lambda_h, scaling_factor, prm.seed, e, nullptr, nullptr)); break;
+        case 5: MF_TRY(mf_single_sgd_hogwild_opt(R, c.n, d_p.as<float>(), d_q.as<float>(), (int)c.k, prm.num_workers, c.update_count, c.update_vector_size,
+                                                 c.lr[e], prm.lambda, prm.seed, e, nullptr, nullptr, opt)); break;
+        case 4: MF_TRY(mf_mpt_sgd_hogwild_opt(R, c.n, d_p.as<float>(), d_q.as<float>(), (int)c.k, prm.num_workers, c.update_count, c.update_vector_size,
+                                              c.lr[e], scaled_lambda_h, scaling_factor, prm.seed, e, nullptr, nullptr, opt)); break;
         case 3: {
             const int idx = precision_idx > 4 ? 4 : precision_idx;      // the reference indexes past the table once at 32 bit (mf_methods.cu:691)
-            MF_TRY(mf_muppet_sgd_hogwild(R, c.n, d_p.as<float>(), d_q.as<float>(), (int)c.k, prm.num_workers, c.update_count, c.update_vector_size,
-                                         c.lr[e], prm.lambda, muppet_first_sample, d_sum_updated.as<float>(), d_sum_norms.as<float>(),
-                                         bit_width_set[idx], bit_width_set[idx], prm.seed, e, nullptr, nullptr));
+            MF_TRY(mf_muppet_sgd_hogwild_opt(R, c.n, d_p.as<float>(), d_q.as<float>(), (int)c.k, prm.num_workers, c.update_count, c.update_vector_size,
+                                             c.lr[e], prm.lambda, muppet_first_sample, d_sum_updated.as<float>(), d_sum_norms.as<float>(),
+                                             bit_width_set[idx], bit_width_set[idx], prm.seed, e, nullptr, nullptr, opt));
             break;
         }
-        case 2: MF_TRY(mf_afp_sgd_hogwild(R, c.n, d_p.as<float>(), d_q.as<float>(), (int)c.k, prm.num_workers, c.update_count, c.update_vector_size,
-                                          c.lr[e], prm.lambda, (int)e, prm.seed, e, nullptr, nullptr)); break;
-        case 7: MF_TRY(mf_mem_quant_sgd_hogwild(R, c.n, d_hp.as<uint16_t>(), d_hq.as<uint16_t>(), (int)c.k, prm.num_workers, c.update_count,
-                                                c.update_vector_size, c.lr[e], prm.lambda, prm.seed, e, nullptr, nullptr)); break;
+        case 2: MF_TRY(mf_afp_sgd_hogwild_opt(R, c.n, d_p.as<float>(), d_q.as<float>(), (int)c.k, prm.num_workers, c.update_count, c.update_vector_size,
+                                              c.lr[e], prm.lambda, (int)e, prm.seed, e, nullptr, nullptr, opt)); break;
+        case 7: MF_TRY(mf_mem_quant_sgd_hogwild_opt(R, c.n, d_hp.as<uint16_t>(), d_hq.as<uint16_t>(), (int)c.k, prm.num_workers, c.update_count,
+                                                    c.update_vector_size, c.lr[e], prm.lambda, prm.seed, e, nullptr, nullptr, opt)); break;
         case 8: {
             // mf_methods.cu:1460-1466: sampled only while the model is binary16
             whole_check = !whole.is_float && prm.interval && e >= 5 && (e % prm.interval == 5 % prm.interval) && prm.epoch - 1 != e;
@@ -318,11 +395,11 @@ int train_dense(Common& c, float* p, float* q)
                 err_ms += now_ms() - e0;
                 t.start();
             }
-            MF_TRY(mf_mascot_sgd_hogwild(R, c.n, whole.ptr_p.as<void*>(), whole.ptr_q.as<void*>(), (int)c.k, prm.num_workers, c.update_count,
-                                         c.update_vector_size, c.lr[e], prm.lambda, whole.end_u.as<uint32_t>(), whole.end_i.as<uint32_t>(),
-                                         whole.prec.as<uint8_t>(), whole.prec.as<uint8_t>(), whole.gsp.as<float>(), whole.gsq.as<float>(),
-                                         whole.nsp.as<float>(), whole.nsq.as<float>(), whole_check ? total - whole_sample_num : total, 1, 1,
-                                         prm.seed, e, nullptr, nullptr));
+            MF_TRY(mf_mascot_sgd_hogwild_opt(R, c.n, whole.ptr_p.as<void*>(), whole.ptr_q.as<void*>(), (int)c.k, prm.num_workers, c.update_count,
+                                             c.update_vector_size, c.lr[e], prm.lambda, whole.end_u.as<uint32_t>(), whole.end_i.as<uint32_t>(),
+                                             whole.prec.as<uint8_t>(), whole.prec.as<uint8_t>(), whole.gsp.as<float>(), whole.gsq.as<float>(),
+                                             whole.nsp.as<float>(), whole.nsq.as<float>(), whole_check ? total - whole_sample_num : total, 1, 1,
+                                             prm.seed, e, nullptr, nullptr, opt));
             break;
         }
         default: return invalid("mf_train: version %u is not a dense variant", version);
@@ -384,13 +461,20 @@ int train_dense(Common& c, float* p, float* q)
             }
             err_ms += now_ms() - e0;
         }
-        if (c.rep) c.rep->error_ms += err_ms;
+        if (c.rep) {
+            c.rep->error_ms += err_ms;
+            c.rep->muppet_final_bits = version == 3 ? bit_width_set[precision_idx > 4 ? 4 : precision_idx] : 0;
+        }
+        return 0;
     }
-    if (c.rep) c.rep->muppet_final_bits = version == 3 ? bit_width_set[precision_idx > 4 ? 4 : precision_idx] : 0;
-    HIP_TRY(hipMemcpy(p, d_p.p, pn * 4, hipMemcpyDeviceToHost), "D2H P");
-    HIP_TRY(hipMemcpy(q, d_q.p, qn * 4, hipMemcpyDeviceToHost), "D2H Q");
-    return 0;
-}
+
+    int download(float* p, float* q) override
+    {
+        HIP_TRY(hipMemcpy(p, d_p.p, pn * 4, hipMemcpyDeviceToHost), "D2H P");
+        HIP_TRY(hipMemcpy(q, d_q.p, qn * 4, hipMemcpyDeviceToHost), "D2H Q");
+        return 0;
+    }
+};
 
 // ---- MASCOT (version 1) --------------------------------------------------------------------------
 struct Side {
@@ -492,65 +576,71 @@ void print_errors(const char* title, const Side& s)
     }
 }
 
-int train_mascot(Common& c, float* p, float* q)
-{
-    const mf_params& prm = *c.prm;
-    const size_t pn = (size_t)c.n_users * c.k, qn = (size_t)c.n_items * c.k;
+struct MascotRun : Run {
+    size_t pn = 0, qn = 0;
     Side U, I;
-    const double pre0 = now_ms();
-    {   // histogram (train only), sort, grouping, re-index of train and test (mf_methods.cu:54-66)
-        DevBuf d_ucnt, d_icnt;
-        MF_TRY(d_ucnt.alloc((size_t)c.n_users * 4, "hipMalloc(user counts)"));
-        MF_TRY(d_icnt.alloc((size_t)c.n_items * 4, "hipMalloc(item counts)"));
-        HIP_TRY(hipMemset(d_ucnt.p, 0, (size_t)c.n_users * 4), "memset");
-        HIP_TRY(hipMemset(d_icnt.p, 0, (size_t)c.n_items * 4), "memset");
-        MF_TRY(mf_user_item_histogram(c.d_R.as<mf_node>(), c.n, d_ucnt.as<uint32_t>(), d_icnt.as<uint32_t>(), nullptr));
-        MF_TRY(build_side(U, d_ucnt, c.n_users, prm.user_group_num, c.k));
-        MF_TRY(build_side(I, d_icnt, c.n_items, prm.item_group_num, c.k));
-    }
-    if (prm.verbose) {      // preprocess_utils.h:192-206
-        std::printf("The number of user groups   : %u\nThe number of item groups   : %u\n", U.groups, I.groups);
-        for (uint32_t g = 0; g < U.groups; ++g) std::printf("%u ", U.end_idx[g]);
-        std::printf("\n\n");
-        for (uint32_t g = 0; g < I.groups; ++g) std::printf("%u ", I.end_idx[g]);
-        std::printf("\n");      // the reference leaves the line open, so its first epoch line lands on it
-        std::fflush(stdout);
-    }
-    DevBuf d_u2s, d_i2s;
-    MF_TRY(d_u2s.alloc((size_t)c.n_users * 4, "hipMalloc(user2sorted)"));
-    MF_TRY(d_i2s.alloc((size_t)c.n_items * 4, "hipMalloc(item2sorted)"));
-    HIP_TRY(hipMemcpy(d_u2s.p, U.id2sorted.data(), (size_t)c.n_users * 4, hipMemcpyHostToDevice), "H2D user2sorted");
-    HIP_TRY(hipMemcpy(d_i2s.p, I.id2sorted.data(), (size_t)c.n_items * 4, hipMemcpyHostToDevice), "H2D item2sorted");
-    MF_TRY(mf_matrix_reconst_triplet(c.d_R.as<mf_node>(), d_u2s.as<uint32_t>(), d_i2s.as<uint32_t>(), c.n, nullptr));
-    MF_TRY(mf_matrix_reconst_triplet(c.d_test.as<mf_node>(), d_u2s.as<uint32_t>(), d_i2s.as<uint32_t>(), c.test_n, nullptr));
-
-    const uint32_t norm_blocks = mf_mascot_norm_blocks(prm.num_workers);
-    MF_TRY(alloc_side_storage(U, norm_blocks));
-    MF_TRY(alloc_side_storage(I, norm_blocks));
-    {   // cpy2grouped_parameters_gpu_for_comparison_indexing, model_init.cu:175-222
-        DevBuf d_dense, d_id2group;
-        MF_TRY(d_dense.alloc(std::max(pn, qn) * 4, "hipMalloc(dense init)"));
-        MF_TRY(d_id2group.alloc((size_t)std::max(c.n_users, c.n_items) * 4, "hipMalloc(id2group)"));
-        HIP_TRY(hipMemcpy(d_dense.p, p, pn * 4, hipMemcpyHostToDevice), "H2D P");
-        HIP_TRY(hipMemcpy(d_id2group.p, U.id2group.data(), (size_t)c.n_users * 4, hipMemcpyHostToDevice), "H2D user2group");
-        MF_TRY(mf_cpyparams2grouped_params(d_dense.as<float>(), U.d_ptr.as<void*>(), U.d_end.as<uint32_t>(), d_id2group.as<uint32_t>(),
-                                           d_u2s.as<uint32_t>(), (int)c.k, c.n_users, U.groups, nullptr));
-        HIP_TRY(hipDeviceSynchronize(), "synchronize");
-        HIP_TRY(hipMemcpy(d_dense.p, q, qn * 4, hipMemcpyHostToDevice), "H2D Q");
-        HIP_TRY(hipMemcpy(d_id2group.p, I.id2group.data(), (size_t)c.n_items * 4, hipMemcpyHostToDevice), "H2D item2group");
-        MF_TRY(mf_cpyparams2grouped_params(d_dense.as<float>(), I.d_ptr.as<void*>(), I.d_end.as<uint32_t>(), d_id2group.as<uint32_t>(),
-                                           d_i2s.as<uint32_t>(), (int)c.k, c.n_items, I.groups, nullptr));
-        HIP_TRY(hipDeviceSynchronize(), "synchronize");
-    }
-    HotRows hot;      // rows are in popularity-sorted order: the sorted counts index them directly
-    MF_TRY(hot.install(prm, U.sorted_cnt.data(), c.n_users, I.sorted_cnt.data(), c.n_items, c.n));
-    if (c.rep) c.rep->preprocess_ms = now_ms() - pre0;
-
+    uint32_t norm_blocks = 0, total = 0;
     const uint32_t start_idx = 5;                                   // mf_methods.cu:110
-    const uint32_t total = c.update_count * c.update_vector_size;
     Timer t;
-    for (uint32_t e = 0; e < prm.epoch; ++e) {
-        MF_TRY(hot.select(e));
+
+    int setup(const mf_node* R, const mf_node* test, const float* p, const float* q) override
+    {
+        pn = (size_t)c.n_users * c.k; qn = (size_t)c.n_items * c.k;
+        MF_TRY(upload_and_shuffle(c, R, test));
+        const double pre0 = now_ms();
+        {   // histogram (train only), sort, grouping, re-index of train and test (mf_methods.cu:54-66)
+            DevBuf d_ucnt, d_icnt;
+            MF_TRY(d_ucnt.alloc((size_t)c.n_users * 4, "hipMalloc(user counts)"));
+            MF_TRY(d_icnt.alloc((size_t)c.n_items * 4, "hipMalloc(item counts)"));
+            HIP_TRY(hipMemset(d_ucnt.p, 0, (size_t)c.n_users * 4), "memset");
+            HIP_TRY(hipMemset(d_icnt.p, 0, (size_t)c.n_items * 4), "memset");
+            MF_TRY(mf_user_item_histogram(c.d_R.as<mf_node>(), c.n, d_ucnt.as<uint32_t>(), d_icnt.as<uint32_t>(), nullptr));
+            MF_TRY(build_side(U, d_ucnt, c.n_users, prm.user_group_num, c.k));
+            MF_TRY(build_side(I, d_icnt, c.n_items, prm.item_group_num, c.k));
+        }
+        if (prm.verbose) {      // preprocess_utils.h:192-206
+            std::printf("The number of user groups   : %u\nThe number of item groups   : %u\n", U.groups, I.groups);
+            for (uint32_t g = 0; g < U.groups; ++g) std::printf("%u ", U.end_idx[g]);
+            std::printf("\n\n");
+            for (uint32_t g = 0; g < I.groups; ++g) std::printf("%u ", I.end_idx[g]);
+            std::printf("\n");      // the reference leaves the line open, so its first epoch line lands on it
+            std::fflush(stdout);
+        }
+        DevBuf d_u2s, d_i2s;
+        MF_TRY(d_u2s.alloc((size_t)c.n_users * 4, "hipMalloc(user2sorted)"));
+        MF_TRY(d_i2s.alloc((size_t)c.n_items * 4, "hipMalloc(item2sorted)"));
+        HIP_TRY(hipMemcpy(d_u2s.p, U.id2sorted.data(), (size_t)c.n_users * 4, hipMemcpyHostToDevice), "H2D user2sorted");
+        HIP_TRY(hipMemcpy(d_i2s.p, I.id2sorted.data(), (size_t)c.n_items * 4, hipMemcpyHostToDevice), "H2D item2sorted");
+        MF_TRY(mf_matrix_reconst_triplet(c.d_R.as<mf_node>(), d_u2s.as<uint32_t>(), d_i2s.as<uint32_t>(), c.n, nullptr));
+        MF_TRY(mf_matrix_reconst_triplet(c.d_test.as<mf_node>(), d_u2s.as<uint32_t>(), d_i2s.as<uint32_t>(), c.test_n, nullptr));
+
+        norm_blocks = mf_mascot_norm_blocks(prm.num_workers);
+        MF_TRY(alloc_side_storage(U, norm_blocks));
+        MF_TRY(alloc_side_storage(I, norm_blocks));
+        {   // cpy2grouped_parameters_gpu_for_comparison_indexing, model_init.cu:175-222
+            DevBuf d_dense, d_id2group;
+            MF_TRY(d_dense.alloc(std::max(pn, qn) * 4, "hipMalloc(dense init)"));
+            MF_TRY(d_id2group.alloc((size_t)std::max(c.n_users, c.n_items) * 4, "hipMalloc(id2group)"));
+            HIP_TRY(hipMemcpy(d_dense.p, p, pn * 4, hipMemcpyHostToDevice), "H2D P");
+            HIP_TRY(hipMemcpy(d_id2group.p, U.id2group.data(), (size_t)c.n_users * 4, hipMemcpyHostToDevice), "H2D user2group");
+            MF_TRY(mf_cpyparams2grouped_params(d_dense.as<float>(), U.d_ptr.as<void*>(), U.d_end.as<uint32_t>(), d_id2group.as<uint32_t>(),
+                                               d_u2s.as<uint32_t>(), (int)c.k, c.n_users, U.groups, nullptr));
+            HIP_TRY(hipDeviceSynchronize(), "synchronize");
+            HIP_TRY(hipMemcpy(d_dense.p, q, qn * 4, hipMemcpyHostToDevice), "H2D Q");
+            HIP_TRY(hipMemcpy(d_id2group.p, I.id2group.data(), (size_t)c.n_items * 4, hipMemcpyHostToDevice), "H2D item2group");
+            MF_TRY(mf_cpyparams2grouped_params(d_dense.as<float>(), I.d_ptr.as<void*>(), I.d_end.as<uint32_t>(), d_id2group.as<uint32_t>(),
+                                               d_i2s.as<uint32_t>(), (int)c.k, c.n_items, I.groups, nullptr));
+            HIP_TRY(hipDeviceSynchronize(), "synchronize");
+        }
+        // rows are in popularity-sorted order: the sorted counts index them directly
+        MF_TRY(hot.install(prm, U.sorted_cnt.data(), c.n_users, I.sorted_cnt.data(), c.n_items, c.n, U.groups, I.groups, c.mean_rating));
+        if (c.rep) c.rep->preprocess_ms = now_ms() - pre0;
+        total = c.update_count * c.update_vector_size;
+        return 0;
+    }
+
+    int epoch(uint32_t e) override
+    {
         const uint32_t first_sample = mf_first_sample_rating_idx(e, prm.interval, prm.epoch, c.update_count, c.update_vector_size, prm.sample_ratio);
         const bool error_check = first_sample < total || (prm.interval && e >= start_idx && (e % prm.interval == start_idx % prm.interval) && prm.epoch - 1 != e);
         double err_ms = 0;
@@ -561,11 +651,11 @@ int train_mascot(Common& c, float* p, float* q)
             err_ms += now_ms() - e0;
         }
         t.start();
-        MF_TRY(mf_mascot_sgd_hogwild(c.d_R.as<mf_node>(), c.n, U.d_ptr.as<void*>(), I.d_ptr.as<void*>(), (int)c.k,
-                                     prm.num_workers, c.update_count, c.update_vector_size, c.lr[e], prm.lambda,
-                                     U.d_end.as<uint32_t>(), I.d_end.as<uint32_t>(), U.d_prec.as<uint8_t>(), I.d_prec.as<uint8_t>(),
-                                     U.d_grad_sum.as<float>(), I.d_grad_sum.as<float>(), U.d_norm_sum.as<float>(), I.d_norm_sum.as<float>(),
-                                     first_sample, U.groups, I.groups, prm.seed, e, nullptr, nullptr));
+        MF_TRY(mf_mascot_sgd_hogwild_opt(c.d_R.as<mf_node>(), c.n, U.d_ptr.as<void*>(), I.d_ptr.as<void*>(), (int)c.k,
+                                         prm.num_workers, c.update_count, c.update_vector_size, c.lr[e], prm.lambda,
+                                         U.d_end.as<uint32_t>(), I.d_end.as<uint32_t>(), U.d_prec.as<uint8_t>(), I.d_prec.as<uint8_t>(),
+                                         U.d_grad_sum.as<float>(), I.d_grad_sum.as<float>(), U.d_norm_sum.as<float>(), I.d_norm_sum.as<float>(),
+                                         first_sample, U.groups, I.groups, prm.seed, e, nullptr, nullptr, hot.options(e)));
         const float sgd_ms = t.stop();
         if (error_check) {          // mf_methods.cu:316-389
             const double e0 = now_ms();
@@ -597,28 +687,57 @@ int train_mascot(Common& c, float* p, float* q)
                                     U.groups, I.groups, c.d_sum_sq.as<double>(), nullptr));
         double rmse = 0;
         MF_TRY(finish_rmse(c, &rmse));
-        MF_TRY(report_epoch(c, e, rmse, sgd_ms));
+        return report_epoch(c, e, rmse, sgd_ms);
     }
 
-    {   // trained model back to the host in sorted row order (what save_trained_model_reconst writes)
-        DevBuf d_dense;
-        MF_TRY(d_dense.alloc(std::max(pn, qn) * 4, "hipMalloc(dense out)"));
-        MF_TRY(mf_grouped_params2dense(U.d_ptr.as<void*>(), U.d_end.as<uint32_t>(), U.d_prec.as<uint8_t>(), d_dense.as<float>(), (int)c.k, c.n_users, U.groups, nullptr));
-        HIP_TRY(hipMemcpy(p, d_dense.p, pn * 4, hipMemcpyDeviceToHost), "D2H P");
-        MF_TRY(mf_grouped_params2dense(I.d_ptr.as<void*>(), I.d_end.as<uint32_t>(), I.d_prec.as<uint8_t>(), d_dense.as<float>(), (int)c.k, c.n_items, I.groups, nullptr));
-        HIP_TRY(hipMemcpy(q, d_dense.p, qn * 4, hipMemcpyDeviceToHost), "D2H Q");
+    int download(float* p, float* q) override
+    {
+        {   // trained model back to the host in sorted row order (what save_trained_model_reconst writes)
+            DevBuf d_dense;
+            MF_TRY(d_dense.alloc(std::max(pn, qn) * 4, "hipMalloc(dense out)"));
+            MF_TRY(mf_grouped_params2dense(U.d_ptr.as<void*>(), U.d_end.as<uint32_t>(), U.d_prec.as<uint8_t>(), d_dense.as<float>(), (int)c.k, c.n_users, U.groups, nullptr));
+            HIP_TRY(hipMemcpy(p, d_dense.p, pn * 4, hipMemcpyDeviceToHost), "D2H P");
+            MF_TRY(mf_grouped_params2dense(I.d_ptr.as<void*>(), I.d_end.as<uint32_t>(), I.d_prec.as<uint8_t>(), d_dense.as<float>(), (int)c.k, c.n_items, I.groups, nullptr));
+            HIP_TRY(hipMemcpy(q, d_dense.p, qn * 4, hipMemcpyDeviceToHost), "D2H Q");
+        }
+        if (c.rep) {
+            mf_report& r = *c.rep;
+            r.user_group_num = U.groups; r.item_group_num = I.groups;
+            if (r.user2sorted_idx) std::copy(U.id2sorted.begin(), U.id2sorted.end(), r.user2sorted_idx);
+            if (r.item2sorted_idx) std::copy(I.id2sorted.begin(), I.id2sorted.end(), r.item2sorted_idx);
+            if (r.user_group_end_idx) std::copy(U.end_idx.begin(), U.end_idx.end(), r.user_group_end_idx);
+            if (r.item_group_end_idx) std::copy(I.end_idx.begin(), I.end_idx.end(), r.item_group_end_idx);
+            if (r.user_group_prec_info) std::copy(U.prec.begin(), U.prec.end(), r.user_group_prec_info);
+            if (r.item_group_prec_info) std::copy(I.prec.begin(), I.prec.end(), r.item_group_prec_info);
+            if (r.test_reconst && c.test_n) HIP_TRY(hipMemcpy(r.test_reconst, c.d_test.p, (size_t)c.test_n * sizeof(mf_node), hipMemcpyDeviceToHost), "D2H test");   // mf_methods.cu:399
+        }
+        return 0;
     }
-    if (c.rep) {
-        mf_report& r = *c.rep;
-        r.user_group_num = U.groups; r.item_group_num = I.groups;
-        if (r.user2sorted_idx) std::copy(U.id2sorted.begin(), U.id2sorted.end(), r.user2sorted_idx);
-        if (r.item2sorted_idx) std::copy(I.id2sorted.begin(), I.id2sorted.end(), r.item2sorted_idx);
-        if (r.user_group_end_idx) std::copy(U.end_idx.begin(), U.end_idx.end(), r.user_group_end_idx);
-        if (r.item_group_end_idx) std::copy(I.end_idx.begin(), I.end_idx.end(), r.item_group_end_idx);
-        if (r.user_group_prec_info) std::copy(U.prec.begin(), U.prec.end(), r.user_group_prec_info);
-        if (r.item_group_prec_info) std::copy(I.prec.begin(), I.prec.end(), r.item_group_prec_info);
-        if (r.test_reconst && c.test_n) HIP_TRY(hipMemcpy(r.test_reconst, c.d_test.p, (size_t)c.test_n * sizeof(mf_node), hipMemcpyDeviceToHost), "D2H test");   // mf_methods.cu:399
-    }
+};
+
+// Checks the arguments of a run and builds its object (nothing touches the device yet).
+int make_run(const mf_params* params, const mf_node* R, uint32_t n, uint32_t n_users, uint32_t n_items,
+             const mf_node* test, uint32_t test_n, const float* p, const float* q, mf_report* report, Run** out)
+{
+    if (!params || !R || !p || !q) return invalid("mf_train: null pointer");
+    if (test_n && !test) return invalid("mf_train: null test set");
+    if (params->k != 64 && params->k != 128) return invalid("mf_train: k must be 64 or 128 (got %u)", params->k);
+    if (n == 0 || n_users == 0 || n_items == 0) return invalid("mf_train: empty problem");
+    const uint32_t version = params->version == 0 ? 5 : params->version;
+    if (version < 1 || version > 8) return invalid("mf_train: version %u does not exist (1 MASCOT, 2 AFP, 3 MuPPET, 4 MPT, 5 fp32 SGD, 6 MASCOT, 7 binary16 storage, 8 whole-model switching)", params->version);
+    // -v 6 (mascot_training_mf_naive, mf_methods.cu:926-1301) is MASCOT with the group search done from global memory
+    // and shifted end-index tables: the same schedule, arithmetic and epoch logic, so it runs the MASCOT path
+    Run* run = (version == 1 || version == 6) ? static_cast<Run*>(new MascotRun) : static_cast<Run*>(new DenseRun);
+    run->prm = *params;
+    if (run->prm.num_workers == 0) run->prm.num_workers = mf_auto_workers(n);
+    Common& c = run->c;
+    c.prm = &run->prm; c.n = n; c.n_users = n_users; c.n_items = n_items; c.test_n = test_n; c.k = params->k; c.rep = report;
+    if (report) { report->preprocess_ms = report->switching_ms = report->error_ms = report->sgd_ms = report->total_ms = 0; report->muppet_final_bits = 0; }
+    double sum = 0;
+    for (uint32_t i = 0; i < n; ++i) sum += std::fabs((double)R[i].r);
+    c.mean_rating = (float)(sum / (double)n);
+    fill_schedule(c);
+    *out = run;
     return 0;
 }
 
@@ -632,7 +751,11 @@ void mf_default_params(mf_params* out)       // main.cu:19-32
     out->lambda = 0.015f; out->learning_rate = 0.01f; out->decay = 0.1f; out->sample_ratio = 0.01f; out->error_threshold = 0.001f;
     out->k = 128; out->epoch = 50; out->num_workers = 2048; out->thread_block_size = 128;
     out->user_group_num = 10; out->item_group_num = 10; out->version = 7; out->interval = 1; out->seed = 1;
-    out->hot_row_inflight = 2.0f; out->hot_row_inflight_early = 8.0f; out->hot_row_early_epochs = 2;   // no reference counterpart: see mf_set_hot_row_thinning
+    // no reference counterpart (mf_hogwild_options): rows with more updates in flight than added updates can safely
+    // sum (mf_replicate_threshold) get a copy per XCD, averaged four times per epoch; rows with more than one have
+    // their updates added; nothing is thinned
+    out->hot_rows = 1; out->replicate_inflight = -1.0f; out->replica_merges = 4;
+    out->hot_row_inflight = 0.0f; out->hot_row_inflight_early = 0.0f; out->hot_row_early_epochs = 0;
 }
 
 uint32_t mf_group_end_indices(const uint32_t* sorted_cnt, uint32_t n, uint32_t requested_groups, uint32_t* end_idx_out)
@@ -699,15 +822,32 @@ int mf_gpu_test_rmse(const mf_node* test, uint32_t test_n, const float* p, const
     return MF_OK;
 }
 
-int mf_hot_row_table(const uint32_t* counts, uint32_t rows, uint32_t n, uint32_t num_workers, float inflight_cap, uint8_t* table)
+int mf_hot_row_table(const uint32_t* counts, uint32_t rows, uint32_t n, float inflight, float replicate_above, float thin_above, float add_within,
+                     uint8_t* table, uint16_t* slot, uint32_t* slot_row, uint32_t* slots)
 {
+    if (slots) *slots = 0;
     if (rows == 0) return MF_OK;
     if (!counts || !table) return invalid("mf_hot_row_table: null pointer");
-    if (n == 0 || num_workers == 0) return invalid("mf_hot_row_table: no ratings or no workers");
-    if (!(inflight_cap > 0)) return invalid("mf_hot_row_table: the cap must be positive");
-    const std::vector<uint8_t> t = keep_table(counts, rows, n, num_workers, inflight_cap);
-    std::memcpy(table, t.data(), rows);
+    if (n == 0 || !(inflight > 0)) return invalid("mf_hot_row_table: no ratings or no updates in flight");
+    if (replicate_above > 0 && (!slot || !slot_row || !slots)) return invalid("mf_hot_row_table: replicated rows need slot, slot_row and slots");
+    const KeepTable t = keep_table(counts, rows, n, inflight, replicate_above, thin_above, add_within);
+    std::memcpy(table, t.keep.data(), rows);
+    if (slot) std::memcpy(slot, t.slot.data(), (size_t)rows * 2);
+    if (slot_row && !t.slot_row.empty()) std::memcpy(slot_row, t.slot_row.data(), t.slot_row.size() * 4);
+    if (slots) *slots = (uint32_t)t.slot_row.size();
     return MF_OK;
+}
+
+float mf_replicate_threshold(float learning_rate, float mean_rating)
+{
+    // C updates of one row in flight add C gradients taken at the same stale row: a step C times as long.  Along the
+    // direction of the other side's mean row the curvature of the objective is about |row|^2, which at convergence is
+    // about the mean rating (row . row' = rating with both factors alike), so the summed step stays a contraction while
+    // C * lr * mean_rating < 2.  A sixth of that bound leaves room for the first epochs, when every row still
+    // moves: 0.3 / (lr * mean_rating), between 2 and 16 (8.3 for lr 0.01 and ratings around 3.6).
+    if (!(learning_rate > 0) || !(mean_rating > 0)) return 8.0f;
+    const float t = 0.3f / (learning_rate * mean_rating);
+    return t < 2.0f ? 2.0f : (t > 16.0f ? 16.0f : t);
 }
 
 uint32_t mf_auto_workers(uint32_t n)
@@ -721,31 +861,68 @@ uint32_t mf_auto_workers(uint32_t n)
 int mf_train(const mf_params* params, const mf_node* R, uint32_t n, uint32_t n_users, uint32_t n_items,
              const mf_node* test, uint32_t test_n, float* p, float* q, mf_report* report)
 {
-    if (!params || !R || !p || !q) return invalid("mf_train: null pointer");
-    if (test_n && !test) return invalid("mf_train: null test set");
-    if (params->k != 64 && params->k != 128) return invalid("mf_train: k must be 64 or 128 (got %u)", params->k);
-    if (n == 0 || n_users == 0 || n_items == 0) return invalid("mf_train: empty problem");
-    mf_params with_workers = *params;
-    if (with_workers.num_workers == 0) with_workers.num_workers = mf_auto_workers(n);
-    params = &with_workers;
-    const uint32_t version = params->version == 0 ? 5 : params->version;
-    if (version < 1 || version > 8) return invalid("mf_train: version %u does not exist (1 MASCOT, 2 AFP, 3 MuPPET, 4 MPT, 5 fp32 SGD, 6 MASCOT, 7 binary16 storage, 8 whole-model switching)", params->version);
-    Common c;
-    c.prm = params; c.n = n; c.n_users = n_users; c.n_items = n_items; c.test_n = test_n; c.k = params->k; c.rep = report;
-    if (report) { report->preprocess_ms = report->switching_ms = report->error_ms = report->sgd_ms = report->total_ms = 0; report->muppet_final_bits = 0; }
     const double t0 = now_ms();
-    const int saved_coherence = mf_get_row_coherence();
-    const uint32_t saved_splits = mf_get_epoch_splits();
-    MF_TRY(mf_set_row_coherence(params->cached_rows ? 0 : 1));
-    MF_TRY(mf_set_epoch_splits(params->epoch_splits ? params->epoch_splits : 1));
-    struct Restore { int c; uint32_t s; ~Restore() { (void)mf_set_row_coherence(c); (void)mf_set_epoch_splits(s); } } restore{saved_coherence, saved_splits};
-    fill_schedule(c);
-    MF_TRY(upload_and_shuffle(c, R, test));
-    // -v 6 (mascot_training_mf_naive, mf_methods.cu:926-1301) is MASCOT with the group search done from global memory
-    // and shifted end-index tables: the same schedule, arithmetic and epoch logic, so it runs the MASCOT path
-    const int rc = (version == 1 || version == 6) ? train_mascot(c, p, q) : train_dense(c, p, q);
-    if (rc == 0 && report) report->total_ms = now_ms() - t0;
-    return rc;
+    Run* raw = nullptr;
+    MF_TRY(make_run(params, R, n, n_users, n_items, test, test_n, p, q, report, &raw));
+    std::unique_ptr<Run> run(raw);
+    MF_TRY(run->setup(R, test, p, q));
+    for (uint32_t e = 0; e < run->prm.epoch; ++e) MF_TRY(run->epoch(e));
+    MF_TRY(run->download(p, q));
+    if (report) report->total_ms = now_ms() - t0;
+    return 0;
 }
+
+struct mf_session { std::unique_ptr<Run> run; };
+
+int mf_session_create(const mf_params* params, const mf_node* R, uint32_t n, uint32_t n_users, uint32_t n_items,
+                      const mf_node* test, uint32_t test_n, const float* p, const float* q, mf_report* report, mf_session** session)
+{
+    if (!session) return invalid("mf_session_create: null session pointer");
+    *session = nullptr;
+    Run* raw = nullptr;
+    MF_TRY(make_run(params, R, n, n_users, n_items, test, test_n, p, q, report, &raw));
+    std::unique_ptr<Run> run(raw);
+    MF_TRY(run->setup(R, test, p, q));
+    *session = new mf_session{std::move(run)};
+    return 0;
+}
+int mf_session_epoch(mf_session* session, double* test_rmse, float* sgd_ms)
+{
+    if (!session || !session->run) return invalid("mf_session_epoch: null session");
+    Run& run = *session->run;
+    if (run.next_epoch >= run.prm.epoch) return invalid("mf_session_epoch: all %u epochs of the run are done", run.prm.epoch);
+    const uint32_t e = run.next_epoch;
+    const int rc = run.epoch(e);
+    const double rmse = rc == 0 ? run.c.rmse_hist[e] : 0.0;
+    const float ms = rc == 0 ? run.c.ms_hist[e] : 0.f;
+    if (rc) return rc;
+    run.next_epoch = e + 1;
+    if (test_rmse) *test_rmse = rmse;
+    if (sgd_ms) *sgd_ms = ms;
+    return 0;
+}
+uint32_t mf_session_workers(const mf_session* session) { return session && session->run ? session->run->prm.num_workers : 0; }
+int mf_session_hot_rows(const mf_session* session, uint32_t* user_replicated, uint32_t* item_replicated, float* inflight)
+{
+    if (!session || !session->run) return invalid("mf_session_hot_rows: null session");
+    if (user_replicated) *user_replicated = session->run->hot.u.slots;
+    if (item_replicated) *item_replicated = session->run->hot.v.slots;
+    if (inflight) *inflight = (float)session->run->hot.inflight;
+    return 0;
+}
+int mf_session_device_state(const mf_session* session, uint32_t epoch, const mf_node** ratings, const mf_hogwild_options** options)
+{
+    if (!session || !session->run) return invalid("mf_session_device_state: null session");
+    if (ratings) *ratings = session->run->c.d_R.as<mf_node>();
+    if (options) *options = session->run->hot.options(epoch);
+    return 0;
+}
+int mf_session_finish(mf_session* session, float* p, float* q)
+{
+    if (!session || !session->run) return invalid("mf_session_finish: null session");
+    if (!p || !q) return invalid("mf_session_finish: null model pointer");
+    return session->run->download(p, q);
+}
+void mf_session_destroy(mf_session* session) { delete session; }
 
 }  // extern "C"

@@ -39,40 +39,83 @@ typedef struct { float r; uint32_t u; uint32_t i; } mf_node;
 
 int mf_version(void);
 const char* mf_last_error(void);
-/* How the update kernels read and write P/Q rows (process-wide, takes effect at the next launch):
- *   1 (default)  device-coherent: every row store writes through the per-XCD L2 to the memory side and drops the
- *                copies other L2s hold (agent-scope relaxed atomic stores; loads stay ordinary cached loads),
- *                so a worker sees the latest row any other worker stored -- the semantics the reference
- *                gets from a GPU with one L2.  All stores to one row serialise at the memory side, which
- *                bounds the epoch when a single row takes percents of all ratings (see
- *                mf_set_hot_row_thinning for what mf_train does about that).
- *   0            cached: ordinary write-back stores; each of the 8 XCDs works on its own L2-resident copy
- *                of a hot row until it is evicted, copies are merged last-writer-wins.
- * No counterpart in the reference (one L2, nothing to choose).  mf_train picks per run, see there. */
-int mf_set_row_coherence(int coherent);
-int mf_get_row_coherence(void);
-/* Cuts every fp32-SGD / MPT / MASCOT update call into `splits` consecutive kernel launches (each worker's
- * windows are divided evenly).  A kernel boundary writes back and invalidates the per-XCD L2s, so with
- * cached row accesses the XCDs' copies of hot rows are reconciled `splits` times per epoch instead of once.
- * Default 1.  No counterpart in the reference. */
-int mf_set_epoch_splits(uint32_t splits);
-uint32_t mf_get_epoch_splits(void);
-/* Hot rows for the update calls (process-wide, both NULL = off, the default).
- * user_keep[row], item_keep[row] are device arrays of bytes indexed like P and Q rows (for MASCOT: sorted row
- * order).  255 marks an ordinary row.  A row with a smaller value is a hot row, meant for rows that have several
- * updates in flight at any time: (1) a rating updates the row with probability (keep+1)/255 and otherwise only
- * reads it for the other side's update; (2) an update that is carried out adds its change to the row in memory
- * (an atomic add per element) instead of storing the new row, so concurrent updates add up where
- * last-writer-wins would keep one of them.  The sum of C stale gradients is a step C times as long, which is why
- * rows with many updates in flight are thinned.  mf_train builds the tables from the rating counts when
- * mf_params.hot_row_inflight > 0.  No counterpart in the reference.  The tables must
- * stay valid while launches that use them are in flight. */
-int mf_set_hot_row_thinning(const uint8_t* user_keep, const uint8_t* item_keep);
+/* ---- options of the Hogwild update launches --------------------------------------------------
+ * Every update entry point below exists in two forms: mf_<rule>_sgd_hogwild(...) with the reference launch's
+ * arguments, and mf_<rule>_sgd_hogwild_opt(..., options) with one more pointer to this structure (NULL = defaults,
+ * which is what the short form passes).  The structure is read during the call and carries no state between calls;
+ * the device arrays it names must stay valid until the launches of the call have finished.  None of it has a
+ * counterpart in the reference, which runs on a GPU with one L2 and a few hundred updates in flight.
+ *
+ * cached_rows   0 (default) device-coherent: every row store writes through the per-XCD L2 to the memory side
+ *               (agent-scope relaxed atomic stores; loads stay ordinary cached loads), so a worker sees the latest
+ *               row any other worker stored -- the semantics the reference gets from a GPU with one L2.  All
+ *               stores to one row serialise at the memory side, which bounds the epoch when a single row takes
+ *               percents of all ratings; that is what the hot-row tables are for.
+ *               1 cached: ordinary write-back stores; each of the 8 XCDs works on its own L2-resident copy of a
+ *               row for as long as it stays cached, copies are merged last-writer-wins.
+ * launches      kernel launches the call is cut into (0 or 1 = one; each worker's windows are divided evenly).
+ *               A kernel boundary writes back and invalidates the per-XCD L2s; replicated rows are averaged there.
+ * user_keep, item_keep   hot-row tables, both or neither: device arrays of bytes indexed like P and Q rows (for
+ *               MASCOT: sorted row order).
+ *                 255  an ordinary row: the new row is stored (the reference's rule, last writer wins);
+ *                 254  a hot row, meant for rows with a few updates in flight at any time: the update adds its
+ *                      change to the row in memory (an atomic add per element), so concurrent updates add up where
+ *                      last-writer-wins would keep one of them;
+ *                 MF_KEEP_REPLICATED (253)  a replicated row, meant for rows with many updates in flight: every XCD
+ *                      works on a copy of its own with ordinary cached loads and stores -- the copy lives in that
+ *                      XCD's L2, where its workers race on it as the reference's warps race on a row, every update
+ *                      carried out -- and after every kernel launch of the call the row and the copies become the
+ *                      mean of the copies that changed (mf_replica_sync_dense).  Nothing of such a row serialises at
+ *                      the memory side;
+ *                 MF_KEEP_REPLICATED_ADDED (252)  a replicated row whose updates are added to the XCD's copy instead of
+ *                      stored, meant for rows with a few updates in flight per XCD: they add up inside the XCD as
+ *                      added updates do on an unreplicated row;
+ *                 0..251  a hot row that is thinned: a rating updates it with probability (value+1)/255 (an added
+ *                      update, as for 254) and otherwise only reads it for the other side's update.
+ * user_slot, item_slot   [rows] uint16: for a replicated row its slot in the replica blocks (read for those rows only)
+ * user_slot_row, item_slot_row   [slots] the row of every slot
+ * user_replicas, item_replicas   caller-owned scratch of MF_XCDS * slots * k * 4 bytes, 256-byte aligned; slot s of
+ *               XCD x is at (x * slots + s) * k * 4 and holds the row in the precision it is stored in.  Filled from
+ *               the rows at the start of every call; nothing is kept in it between calls.
+ * user_slots, item_slots   replicated rows per side (at most 65535; 0 = none) */
+#define MF_KEEP_ORDINARY 255
+#define MF_KEEP_ADDED 254
+#define MF_KEEP_REPLICATED 253
+#define MF_KEEP_REPLICATED_ADDED 252
+#define MF_XCDS 8
+typedef struct {
+    uint32_t cached_rows;
+    uint32_t launches;
+    const uint8_t* user_keep;
+    const uint8_t* item_keep;
+    const uint16_t* user_slot;
+    const uint16_t* item_slot;
+    const uint32_t* user_slot_row;
+    const uint32_t* item_slot_row;
+    void* user_replicas;
+    void* item_replicas;
+    uint32_t user_slots, item_slots;
+} mf_hogwild_options;
+/* What the update calls do with replicated rows before and after every kernel launch, for a dense matrix [rows][k] of
+ * elem_bytes-wide elements (2: binary16, 4: binary32): merge = 0 copies row slot_row[s] into slot s of every XCD's
+ * replica block; merge = 1 sets the row and all its copies to the mean of those copies that differ from the row
+ * (summed in binary32 in XCD order, divided by their number, rounded once); a row none of whose copies differs stays. */
+int mf_replica_sync_dense(void* matrix, uint32_t elem_bytes, int k, void* replicas, const uint32_t* slot_row, uint32_t slots,
+                          int merge, void* stream);
 /* The table mf_train builds for one side (host arrays): counts[row] ratings of `n` fall on the row; with
- * F = min(num_workers, 8192) * 4 updates in flight on the device a row has about F * counts[row] / n of them.
- * Rows with at most one stay ordinary (255); the others become hot rows, kept with probability
- * min(1, inflight_cap / in flight): table value clip(floor(keep * 255) - 1, 0, 254). */
-int mf_hot_row_table(const uint32_t* counts, uint32_t rows, uint32_t n, uint32_t num_workers, float inflight_cap, uint8_t* table);
+ * `inflight` updates in flight on the device (mf_hogwild_inflight) a row has about inflight * counts[row] / n of them.
+ * Rows with at most one stay ordinary (255).  Of the others, rows above replicate_above (> 0) are marked
+ * MF_KEEP_REPLICATED -- MF_KEEP_REPLICATED_ADDED instead up to add_within x MF_XCDS in flight (add_within: updates in
+ * flight per XCD; 0 = never) -- and numbered in row order (slot[row], slot_row[slot]; slot may be NULL
+ * when replicate_above is 0; at most 65535, the rows with the highest counts); rows above thin_above (> 0) are thinned
+ * to that many updates in flight: value clip(floor(thin_above / in flight * 255) - 1, 0, 251); the rest are added (254).
+ * Returns the number of replicated rows in *slots. */
+int mf_hot_row_table(const uint32_t* counts, uint32_t rows, uint32_t n, float inflight, float replicate_above, float thin_above, float add_within,
+                     uint8_t* table, uint16_t* slot, uint32_t* slot_row, uint32_t* slots);
+/* Updates in flight during a launch of `num_workers` workers of the update rule of mf_params.version (1..8) at this k:
+ * min(num_workers, wavefronts the device keeps resident for that kernel) x the ratings a wavefront keeps in flight
+ * (4; 2 for MuPPET and AFP).  Asks the HIP runtime for the kernel's occupancy on the current device. */
+float mf_hogwild_inflight(uint32_t version, int k, uint32_t num_workers, uint32_t user_groups, uint32_t item_groups);
 /* Seeded synthetic ratings (no counterpart in the reference, whose data sets are downloaded): users and items are
  * drawn independently from Zipf(alpha) over a random permutation of the ids; a rating is
  * clamp(round_to_step(U_u . V_i + mean + noise * N(0,1)), lo, hi) with rank-`rank` factors U, V ~ N(0, 0.5^2), or,
@@ -99,13 +142,14 @@ int mf_generate_ratings_host(const mf_synth_config* cfg, uint64_t seed, uint64_t
 /* Measurement aid, no counterpart in the reference: the memory traffic of one epoch of updates without the
  * arithmetic.  Worker w (one wavefront) walks ratings [w*ceil(n/W), (w+1)*ceil(n/W)); per rating it reads row u of p
  * and row i of q (row_bytes = 128, 256 or 512 bytes each: k = 64 binary16, k = 128 binary16 / k = 64 binary32,
- * k = 128 binary32) and writes both back unchanged, with the store policy of mf_set_row_coherence's value
- * `coherent`.  With keep tables (as for mf_set_hot_row_thinning; both or neither) a thinned update only reads its
- * row; an update of a hot row that is kept is a store here as well.  p and q keep their contents (writes of other
- * code that race with the probe may be lost).  The time of this launch is what the memory system sustains for the
- * sequence of addresses and the write policy of an epoch; bench.py reports the update kernel's time beside it. */
+ * k = 128 binary32) and writes both back unchanged, with the store policy, hot-row tables and replicated rows of
+ * `options` (NULL = defaults; `launches` is ignored, replica slots are taken as row_bytes wide): a thinned update
+ * only reads its row, an added update is a store here, a replicated row is read and written in this XCD's copy.
+ * p and q keep their contents (writes of other code that race with the probe may be lost).  The time of this launch is
+ * what the memory system sustains for the sequence of addresses and the write policy of an epoch; bench.py reports the
+ * update kernel's time beside it. */
 int mf_row_traffic_probe(const mf_node* R, uint32_t n, void* p, void* q, uint32_t row_bytes, uint32_t num_workers,
-                         const uint8_t* user_keep, const uint8_t* item_keep, uint64_t seed, int coherent, void* stream);
+                         uint64_t seed, void* stream, const mf_hogwild_options* options);
 /* Number of per-block columns mf_mascot_sgd_hogwild writes into norm_sum_p / norm_sum_q
  * (the reference's `block_num`, mf_methods.cu:109). */
 uint32_t mf_mascot_norm_blocks(uint32_t num_workers);
@@ -129,6 +173,11 @@ int mf_single_sgd_hogwild(const mf_node* R, uint32_t nnz, float* p, float* q, in
                           uint32_t num_workers, uint32_t update_count, uint32_t update_vector_size,
                           float lrate, float lambda,
                           uint64_t seed, uint32_t epoch, const uint32_t* window_start, void* stream);
+int mf_single_sgd_hogwild_opt(const mf_node* R, uint32_t nnz, float* p, float* q, int k,
+                          uint32_t num_workers, uint32_t update_count, uint32_t update_vector_size,
+                          float lrate, float lambda,
+                          uint64_t seed, uint32_t epoch, const uint32_t* window_start, void* stream,
+        const mf_hogwild_options* options);
 
 /* mem_quant_sgd_k128/k64_hogwild_kernel launch (-v 7, the reference's default version), mf_methods.cu:1345-1372:
  * dense binary16 P [users][k], Q [items][k] (bit patterns), binary32 arithmetic, new values rounded to binary16. */
@@ -136,6 +185,11 @@ int mf_mem_quant_sgd_hogwild(const mf_node* R, uint32_t nnz, uint16_t* p, uint16
                              uint32_t num_workers, uint32_t update_count, uint32_t update_vector_size,
                              float lrate, float lambda,
                              uint64_t seed, uint32_t epoch, const uint32_t* window_start, void* stream);
+int mf_mem_quant_sgd_hogwild_opt(const mf_node* R, uint32_t nnz, uint16_t* p, uint16_t* q, int k,
+                             uint32_t num_workers, uint32_t update_count, uint32_t update_vector_size,
+                             float lrate, float lambda,
+                             uint64_t seed, uint32_t epoch, const uint32_t* window_start, void* stream,
+        const mf_hogwild_options* options);
 /* mpt_sgd_k128/k64_hogwild_kernel, mpt/mpt_sgd_kernel.h:1-93, mpt/mpt_sgd_kernel_k64.h;
  * launch site mf_methods.cu:772-799.  scaled_lambda_half = binary16 bits of lambda*scaling_factor
  * (mf_methods.cu:764-765). */
@@ -143,6 +197,11 @@ int mf_mpt_sgd_hogwild(const mf_node* R, uint32_t nnz, float* p, float* q, int k
                        uint32_t num_workers, uint32_t update_count, uint32_t update_vector_size,
                        float lrate, uint16_t scaled_lambda_half, float scaling_factor,
                        uint64_t seed, uint32_t epoch, const uint32_t* window_start, void* stream);
+int mf_mpt_sgd_hogwild_opt(const mf_node* R, uint32_t nnz, float* p, float* q, int k,
+                       uint32_t num_workers, uint32_t update_count, uint32_t update_vector_size,
+                       float lrate, uint16_t scaled_lambda_half, float scaling_factor,
+                       uint64_t seed, uint32_t epoch, const uint32_t* window_start, void* stream,
+        const mf_hogwild_options* options);
 
 /* muppet_sgd_k128/k64_hogwild_kernel, muppet/muppet_sgd_kernel.h:50-292, _k64.h; launch site
  * mf_methods.cu:613-647.  sum_updated_val: [k] (+=, caller zeroes, mf_methods.cu:606-607);
@@ -153,6 +212,13 @@ int mf_muppet_sgd_hogwild(const mf_node* R, uint32_t nnz, float* p, float* q, in
                           float* sum_updated_val, float* sum_norms,
                           uint8_t forward_prop_precision, uint8_t backward_prop_precision,
                           uint64_t seed, uint32_t epoch, const uint32_t* window_start, void* stream);
+int mf_muppet_sgd_hogwild_opt(const mf_node* R, uint32_t nnz, float* p, float* q, int k,
+                          uint32_t num_workers, uint32_t update_count, uint32_t update_vector_size,
+                          float lrate, float lambda, uint32_t first_sample_rating_idx,
+                          float* sum_updated_val, float* sum_norms,
+                          uint8_t forward_prop_precision, uint8_t backward_prop_precision,
+                          uint64_t seed, uint32_t epoch, const uint32_t* window_start, void* stream,
+        const mf_hogwild_options* options);
 
 /* afp_sgd_k128/k64_hogwild_kernel, afp/afp_sgd_kernel.h:127-375, _k64.h; launch site
  * mf_methods.cu:480-507.  `afp_epoch` is the kernel's `epoch` argument (first tenth of
@@ -161,6 +227,11 @@ int mf_afp_sgd_hogwild(const mf_node* R, uint32_t nnz, float* p, float* q, int k
                        uint32_t num_workers, uint32_t update_count, uint32_t update_vector_size,
                        float lrate, float lambda, int afp_epoch,
                        uint64_t seed, uint32_t epoch, const uint32_t* window_start, void* stream);
+int mf_afp_sgd_hogwild_opt(const mf_node* R, uint32_t nnz, float* p, float* q, int k,
+                       uint32_t num_workers, uint32_t update_count, uint32_t update_vector_size,
+                       float lrate, float lambda, int afp_epoch,
+                       uint64_t seed, uint32_t epoch, const uint32_t* window_start, void* stream,
+        const mf_hogwild_options* options);
 
 /* mascot_sgd_k128/k64_hogwild_kernel, mascot/mascot_sgd_kernel.h:1-457, _k64.h:1-397; launch
  * site mf_methods.cu:189-237.
@@ -179,6 +250,15 @@ int mf_mascot_sgd_hogwild(const mf_node* R, uint32_t nnz, void* const* p, void* 
                           float* grad_sum_norm_p, float* grad_sum_norm_q, float* norm_sum_p, float* norm_sum_q,
                           uint32_t first_sample_rating_idx, uint32_t user_group_num, uint32_t item_group_num,
                           uint64_t seed, uint32_t epoch, const uint32_t* window_start, void* stream);
+int mf_mascot_sgd_hogwild_opt(const mf_node* R, uint32_t nnz, void* const* p, void* const* q, int k,
+                          uint32_t num_workers, uint32_t update_count, uint32_t update_vector_size,
+                          float lrate, float lambda,
+                          const uint32_t* user_group_end_idx, const uint32_t* item_group_end_idx,
+                          const uint8_t* user_group_prec_info, const uint8_t* item_group_prec_info,
+                          float* grad_sum_norm_p, float* grad_sum_norm_q, float* norm_sum_p, float* norm_sum_q,
+                          uint32_t first_sample_rating_idx, uint32_t user_group_num, uint32_t item_group_num,
+                          uint64_t seed, uint32_t epoch, const uint32_t* window_start, void* stream,
+        const mf_hogwild_options* options);
 
 /* ---- m-quantization: conversion and grouped storage ---------------------------------- */
 
@@ -262,15 +342,22 @@ typedef struct {
     uint32_t is_yahoo;        /* MuPPET starts at 12 bit (mf_methods.cu:600) */
     uint64_t seed;            /* replaces time(0) / clock() seeding */
     uint32_t verbose;         /* 1: print the reference's stdout lines (mf_methods.cu:396 etc.) */
-    uint32_t cached_rows;     /* 0: device-coherent row stores (default), 1: cached, see mf_set_row_coherence */
-    uint32_t epoch_splits;    /* kernel launches per epoch, 0 or 1 = one, see mf_set_epoch_splits */
-    float hot_row_inflight;   /* > 0: rows expected to have more than one update in flight become hot rows, thinned
-                                 to at most this many updates in flight (see mf_set_hot_row_thinning); 0 = off */
-    float hot_row_inflight_early; /* the cap during the first hot_row_early_epochs epochs, while all rows still grow
-                                 from their small initial values and popular rows need many updates (default 8 for
-                                 2 epochs, then hot_row_inflight = 2; 16 diverges in one run of sixteen at 100M
-                                 ratings) */
+    uint32_t cached_rows;     /* mf_hogwild_options::cached_rows */
+    uint32_t epoch_splits;    /* mf_hogwild_options::launches; 0 = one launch, or replica_merges when rows are replicated */
+    float hot_row_inflight;   /* > 0: hot rows that are not replicated and have more than this many updates in flight are
+                                 thinned to it (mf_hogwild_options, keep values 0..251); 0 (default) = nothing is thinned */
+    float hot_row_inflight_early; /* with thinning: the cap during the first hot_row_early_epochs epochs */
     uint32_t hot_row_early_epochs;
+    uint32_t hot_rows;        /* 1 (default): rows expected to have more than one update in flight become hot rows (updates
+                                 added in memory, MF_KEEP_ADDED); 0 with replicate_inflight = hot_row_inflight = 0: no tables
+                                 at all, every row is stored as the reference does (last writer wins) */
+    float replicate_inflight; /* rows expected to have more than this many updates in flight get a copy per XCD
+                                 (MF_KEEP_REPLICATED); the expectation is mf_hogwild_inflight() x the row's share of the
+                                 ratings.  < 0 (default): mf_replicate_threshold(learning_rate, mean rating); 0 = no replicas */
+    uint32_t replica_merges;  /* launches per epoch when rows are replicated (default 4): their copies are averaged after each */
+    float replica_add_inflight; /* > 0: replicated rows with at most this many updates in flight per XCD have their updates
+                                 added to the XCD's copy (MF_KEEP_REPLICATED_ADDED) instead of stored.  Default 0: at
+                                 100M ratings the extra atomic adds cost 9 ms per epoch and gain 0.0007 test RMSE */
 } mf_params;
 
 /* What a run reports back; every pointer is optional host memory owned by the caller. */
@@ -304,6 +391,30 @@ int mf_init_model(float* p, float* q, uint32_t n_users, uint32_t n_items, uint32
  *                  rows come back in popularity-sorted order (as save_trained_model_reconst expects). */
 int mf_train(const mf_params* params, const mf_node* R, uint32_t n, uint32_t n_users, uint32_t n_items,
              const mf_node* test, uint32_t test_n, float* p, float* q, mf_report* report);
+/* The same run with the epochs handed to the caller one at a time (no counterpart in the reference, whose drivers
+ * run to the end): mf_session_create does what mf_train does before its first epoch (checks, upload, shuffle,
+ * pre-processing, hot-row tables), every mf_session_epoch runs the next epoch exactly as mf_train would -- update
+ * launches, error estimate, precision switching, test RMSE -- and returns that epoch's test RMSE and the hipEvent time
+ * of its update launches, mf_session_finish copies the model to p, q (and fills the MASCOT tables of the report).
+ * `report` is optional, must outlive the session and is filled as in mf_train.  One host thread per session. */
+typedef struct mf_session mf_session;
+int mf_session_create(const mf_params* params, const mf_node* R, uint32_t n, uint32_t n_users, uint32_t n_items,
+                      const mf_node* test, uint32_t test_n, const float* p, const float* q, mf_report* report, mf_session** session);
+int mf_session_epoch(mf_session* session, double* test_rmse, float* sgd_ms);
+int mf_session_finish(mf_session* session, float* p, float* q);
+void mf_session_destroy(mf_session* session);
+/* The worker count the session runs (mf_params.num_workers, or mf_auto_workers), and its hot rows: rows replicated per
+ * side and the updates in flight the tables were built for (0 when the run has no tables). */
+uint32_t mf_session_workers(const mf_session* session);
+int mf_session_hot_rows(const mf_session* session, uint32_t* user_replicated, uint32_t* item_replicated, float* inflight);
+/* The session's training ratings on the device (shuffled; for MASCOT re-indexed to sorted rows) and the launch options
+ * its update calls of `epoch` use; both stay owned by the session and valid until mf_session_destroy.  For
+ * measurements that replay the session's memory traffic (mf_row_traffic_probe). */
+int mf_session_device_state(const mf_session* session, uint32_t epoch, const mf_node** ratings, const mf_hogwild_options** options);
+/* Above how many updates in flight mf_train replicates a row when mf_params.replicate_inflight < 0 (the default):
+ * 0.3 / (learning_rate * mean |rating|), between 2 and 16.  Added updates of one row that are in flight together sum
+ * gradients taken at the same stale row; the sum stays a contraction while their number x lr x mean rating < 2. */
+float mf_replicate_threshold(float learning_rate, float mean_rating);
 /* Host grouping, split_group_based_equal_size_not_strict_ret_end_idx, preprocess_utils.h:101-190:
  * sorted_cnt ascending rating counts; writes inclusive end indices (capacity n) and returns their number. */
 uint32_t mf_group_end_indices(const uint32_t* sorted_cnt, uint32_t n, uint32_t requested_groups, uint32_t* end_idx_out);

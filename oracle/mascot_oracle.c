@@ -948,8 +948,30 @@ void orc_muppet_epoch(int k, const orc_node* R, uint32_t nnz, float* P, float* Q
                       float* sum_updated_val, float* sum_norms, int forward_bits, int backward_bits,
                       uint64_t seed, uint32_t epoch, const uint32_t* window_start, int threads)
 {
-    (void)threads;
     for (uint32_t w = 0; w < num_workers; w++) sum_norms[w] = 0;     /* sum_norms_reg = 0, muppet_sgd_kernel.h:75,288 */
+    if (threads > 1) {
+        /* Hogwild over host threads: workers race on the rows; a worker's norm sum is its own, the sampled gradient
+         * sums are kept per thread and folded at the end (the kernel adds them with atomics, in any order) */
+        #pragma omp parallel num_threads(threads)
+        {
+            float* mine = (float*)calloc((size_t)k, sizeof(float));
+            #pragma omp for schedule(dynamic, 1)
+            for (uint32_t wid = 0; wid < num_workers; wid++)
+                for (uint32_t ite = 0; ite < update_count; ite++) {
+                    uint32_t start = win_start(window_start, seed, epoch, num_workers, wid, ite, nnz);
+                    for (uint32_t i = 0; i < update_vector_size; i++) {
+                        const orc_node* nd = &R[(uint32_t)(((uint64_t)start + i) % nnz)];
+                        int sample = ite * update_vector_size + i >= first_sample_rating_idx;
+                        orc_muppet_update(k, P + (size_t)nd->u * k, Q + (size_t)nd->i * k, nd->r, lr, lambda, forward_bits, backward_bits,
+                                          sample ? mine : NULL, sample ? &sum_norms[wid] : NULL);
+                    }
+                }
+            #pragma omp critical
+            for (int e = 0; e < k; e++) sum_updated_val[e] += mine[e];
+            free(mine);
+        }
+        return;
+    }
     FOR_EACH_UPDATE_SEQ(
         int sample = processed_cnt >= first_sample_rating_idx;
         orc_muppet_update(k, P + (size_t)nd->u * k, Q + (size_t)nd->i * k, nd->r, lr, lambda, forward_bits, backward_bits,
@@ -962,10 +984,16 @@ void orc_afp_epoch(int k, const orc_node* R, uint32_t nnz, float* P, float* Q,
                    float lr, float lambda, int epoch_arg,
                    uint64_t seed, uint32_t epoch, const uint32_t* window_start, int threads)
 {
-    (void)threads;
     orc_afp_state* st = (orc_afp_state*)malloc(sizeof(orc_afp_state) * num_workers);
     for (uint32_t w = 0; w < num_workers; w++) orc_afp_state_init(&st[w]);
     int init_thr = f2i_sat((float)(update_count * update_vector_size) / 10.0f);     /* afp_sgd_kernel.h:145 */
+    if (threads > 1) {      /* Hogwild over host threads: the quantiser state belongs to the worker, the rows are raced on */
+        FOR_EACH_UPDATE_PAR(
+            orc_afp_update(k, &st[wid], P + (size_t)nd->u * k, Q + (size_t)nd->i * k, nd->r, lr, lambda, epoch_arg, init_thr);
+        )
+        free(st);
+        return;
+    }
     FOR_EACH_UPDATE_SEQ(
         orc_afp_update(k, &st[wid], P + (size_t)nd->u * k, Q + (size_t)nd->i * k, nd->r, lr, lambda, epoch_arg, init_thr);
     )
@@ -1005,6 +1033,49 @@ void orc_mascot_epoch(int k, const orc_node* R, uint32_t nnz, void** user_group_
     if (sampling) {
         gsp = (double*)calloc((size_t)user_groups * k, sizeof(double)); gsq = (double*)calloc((size_t)item_groups * k, sizeof(double));
         nsp = (double*)calloc(user_groups, sizeof(double)); nsq = (double*)calloc(item_groups, sizeof(double));
+    }
+    if (threads > 1) {
+        /* a check epoch as a Hogwild loop: the workers race on the rows as in the plain epochs; the sampled sums are
+         * kept per thread in binary64 and folded at the end, so they do not depend on the interleaving beyond the
+         * rows the gradients were computed from */
+        #pragma omp parallel num_threads(threads)
+        {
+            double* tgsp = (double*)calloc((size_t)user_groups * k, sizeof(double)); double* tgsq = (double*)calloc((size_t)item_groups * k, sizeof(double));
+            double* tnsp = (double*)calloc(user_groups, sizeof(double)); double* tnsq = (double*)calloc(item_groups, sizeof(double));
+            float tgp[128], tgq[128];
+            #pragma omp for schedule(dynamic, 1)
+            for (uint32_t wid = 0; wid < num_workers; wid++)
+                for (uint32_t ite = 0; ite < update_count; ite++) {
+                    uint32_t start = win_start(window_start, seed, epoch, num_workers, wid, ite, nnz);
+                    for (uint32_t i = 0; i < update_vector_size; i++) {
+                        const orc_node* nd = &R[(uint32_t)(((uint64_t)start + i) % nnz)];
+                        uint32_t processed_cnt = ite * update_vector_size + i;
+                        uint32_t ug; uint32_t ig; int up; int ip; float np = 0; float nq = 0;
+                        void* prow = group_row(user_group_ptr, user_end_idx, user_prec, user_groups, nd->u, k, &ug, &up);
+                        void* qrow = group_row(item_group_ptr, item_end_idx, item_prec, item_groups, nd->i, k, &ig, &ip);
+                        int sample = processed_cnt >= first_sample_rating_idx;
+                        orc_mascot_update(k, prow, up, qrow, ip, nd->r, lr, lambda, sample ? tgp : NULL, sample ? tgq : NULL, &np, &nq);
+                        if (sample) {
+                            if (!up) { tnsp[ug] += np; for (int e = 0; e < k; e++) tgsp[(size_t)ug * k + e] += tgp[e]; }
+                            if (!ip) { tnsq[ig] += nq; for (int e = 0; e < k; e++) tgsq[(size_t)ig * k + e] += tgq[e]; }
+                        }
+                    }
+                }
+            #pragma omp critical
+            {
+                for (size_t i = 0; i < (size_t)user_groups * k; i++) gsp[i] += tgsp[i];
+                for (size_t i = 0; i < (size_t)item_groups * k; i++) gsq[i] += tgsq[i];
+                for (uint32_t g = 0; g < user_groups; g++) nsp[g] += tnsp[g];
+                for (uint32_t g = 0; g < item_groups; g++) nsq[g] += tnsq[g];
+            }
+            free(tgsp); free(tgsq); free(tnsp); free(tnsq);
+        }
+        for (size_t i = 0; i < (size_t)user_groups * k; i++) grad_sum_norm_p[i] += (float)gsp[i];
+        for (size_t i = 0; i < (size_t)item_groups * k; i++) grad_sum_norm_q[i] += (float)gsq[i];
+        for (uint32_t g = 0; g < user_groups; g++) norm_sum_p[g] += (float)nsp[g];
+        for (uint32_t g = 0; g < item_groups; g++) norm_sum_q[g] += (float)nsq[g];
+        free(gsp); free(gsq); free(nsp); free(nsq);
+        return;
     }
     float gp[128], gq[128];
     FOR_EACH_UPDATE_SEQ(

@@ -85,6 +85,40 @@ def stream_ptr():
     return torch.cuda.current_stream().cuda_stream
 
 
+class HogwildOptions:
+    """mf_hogwild_options over numpy keep tables (device copies are kept alive by the object).  Rows whose keep value
+    is 253 or 252 (MF_KEEP_REPLICATED, MF_KEEP_REPLICATED_ADDED) get replica slots in row order."""
+
+    def __init__(self, k, keep_u=None, keep_v=None, cached_rows=0, launches=1):
+        import torch
+        capi = importlib.import_module("icdm-2021_mascot_amd.capi")
+        self.o = o = capi.HogwildOptions()
+        o.cached_rows, o.launches = cached_rows, launches
+        self.keep = []
+        self.replicas = [None, None]
+        self.slot_rows = [np.zeros(0, np.uint32), np.zeros(0, np.uint32)]
+        for side, keep in enumerate((keep_u, keep_v)):
+            if keep is None:
+                continue
+            keep = np.ascontiguousarray(keep, np.uint8)
+            rows = np.nonzero((keep == 253) | (keep == 252))[0].astype(np.uint32)
+            slot = np.zeros(keep.size, np.uint16)
+            slot[rows] = np.arange(rows.size, dtype=np.uint16)
+            dk, ds, dr = to_dev(keep), to_dev(slot), to_dev(rows if rows.size else np.zeros(1, np.uint32))
+            rep = torch.zeros(max(256, 8 * rows.size * k * 4), dtype=torch.uint8, device="cuda")
+            assert rep.data_ptr() % 256 == 0
+            self.keep += [dk, ds, dr, rep]
+            self.replicas[side], self.slot_rows[side] = rep, rows
+            if side == 0:
+                o.user_keep, o.user_slot, o.user_slot_row, o.user_replicas, o.user_slots = dk.data_ptr(), ds.data_ptr(), dr.data_ptr(), rep.data_ptr(), rows.size
+            else:
+                o.item_keep, o.item_slot, o.item_slot_row, o.item_replicas, o.item_slots = dk.data_ptr(), ds.data_ptr(), dr.data_ptr(), rep.data_ptr(), rows.size
+
+    @property
+    def ptr(self):
+        return C.addressof(self.o)
+
+
 def equal_end_idx(n, groups):
     """Inclusive end indices splitting n sorted rows into `groups` nearly equal groups."""
     bounds = np.linspace(0, n, groups + 1).astype(np.int64)[1:]
@@ -142,9 +176,10 @@ def test_set_order(test):
     return np.ascontiguousarray(t[last])
 
 
-def oracle_train_dense(orc, version, R, test, P, Q, k, W, epochs, lr, lam, decay, seed, threads=8, sample_ratio=0.01):
+def oracle_train_dense(orc, version, R, test, P, Q, k, W, epochs, lr, lam, decay, seed, threads=8, sample_ratio=0.01, sequential_threads=1):
     """training_single_mf / mixed_precision_training_mf / muppet_training_mf / adaptive_fixed_point_training_mf
-    (mf_methods.cu:820-924, 713-818, 529-711, 436-527) on the CPU; returns per-epoch test RMSE."""
+    (mf_methods.cu:820-924, 713-818, 529-711, 436-527) on the CPU; returns per-epoch test RMSE.  MuPPET and AFP run one
+    worker after another (what the bit-exact single-worker tests need) unless sequential_threads > 1 lets host threads race."""
     Rs = orc.shuffle(seed, R)
     uc = orc.lib.orc_update_count(Rs.size, W, 128)
     rmse = []
@@ -165,13 +200,13 @@ def oracle_train_dense(orc, version, R, test, P, Q, k, W, epochs, lr, lam, decay
             nrm = np.zeros(W, np.float32)
             b = bits_ladder[min(pidx_c.value, 4)]
             orc.lib.orc_muppet_epoch(k, Rs.ctypes.data, Rs.size, P.ctypes.data, Q.ctypes.data, W, uc, 128, lre, lam, first_sample,
-                                     s.ctypes.data, nrm.ctypes.data, b, b, seed, e, None, 1)
+                                     s.ctypes.data, nrm.ctypes.data, b, b, seed, e, None, sequential_threads)
             norms_hist[e] = np.float32(nrm.sum(dtype=np.float32))
             upd_hist[e] = s
             orc.lib.orc_muppet_ladder_step(k, e, C.byref(switched), C.byref(pidx_c), C.byref(maxdiv), C.byref(viol),
                                            norms_hist.ctypes.data, upd_hist.ctypes.data)
         elif version == 2:
-            orc.lib.orc_afp_epoch(k, Rs.ctypes.data, Rs.size, P.ctypes.data, Q.ctypes.data, W, uc, 128, lre, lam, e, seed, e, None, 1)
+            orc.lib.orc_afp_epoch(k, Rs.ctypes.data, Rs.size, P.ctypes.data, Q.ctypes.data, W, uc, 128, lre, lam, e, seed, e, None, sequential_threads)
         rmse.append(orc.rmse(k, test, P, Q))
     return np.array(rmse), dict(final_bits=bits_ladder[min(pidx_c.value, 4)])
 
@@ -232,7 +267,7 @@ def oracle_train_switching_only(orc, R, test, P, Q, k, W, epochs, lr, lam, decay
     return np.array(rmse), switched, errors
 
 
-def oracle_train_mascot(orc, R, test, P, Q, k, W, epochs, lr, lam, decay, seed, ug, ig, sample_ratio, interval, threshold, threads=8):
+def oracle_train_mascot(orc, R, test, P, Q, k, W, epochs, lr, lam, decay, seed, ug, ig, sample_ratio, interval, threshold, threads=8, progress=None):
     """mascot_training_mf, mf_methods.cu:36-434, on the CPU: shuffle, histogram, sort, grouping, re-index,
     scatter into binary16 groups, epochs with sampled error estimation and precision switching."""
     n_users, n_items = P.shape[0], Q.shape[0]
@@ -278,4 +313,129 @@ def oracle_train_mascot(orc, R, test, P, Q, k, W, epochs, lr, lam, decay, seed, 
             switches.append((e, eu.copy(), ei.copy()))
         rmse.append(orc.lib.orc_rmse_grouped(k, test.ctypes.data, test.size, gu.ptrs, gi.ptrs, gu.end_idx.ctypes.data, gi.end_idx.ctypes.data,
                                              gu.prec.ctypes.data, gi.prec.ctypes.data, gu.groups, gi.groups))
+        if progress is not None:
+            progress(e, rmse[-1])
     return np.array(rmse), dict(gu=gu, gi=gi, uend=uend, iend=iend, u2s=u2s, i2s=i2s, test=test, errors=switches)
+
+
+# ---- device-resident MASCOT state built with the library's own pre-processing kernels ------------------------------
+class MascotProblem:
+    """Device-resident MASCOT training state built with the library's own pre-processing kernels."""
+
+    def __init__(self, torch, h, R, n_users, n_items, k, ug, ig, seed, test=None):
+        self.torch, self.h, self.k = torch, h, k
+        dev = R.device
+        st = torch.cuda.current_stream().cuda_stream
+        n = R.shape[0]
+        self.n, self.n_users, self.n_items = n, n_users, n_items
+        # seeded shuffle (mf_methods.cu:38-39)
+        self.R = torch.empty_like(R)
+        h.mf_shuffle_ratings(R.data_ptr(), self.R.data_ptr(), n, seed, st)
+        # histogram -> sort -> grouping -> re-index (preprocess_utils.h:54-255)
+        ucnt = torch.zeros(n_users, dtype=torch.int32, device=dev)
+        icnt = torch.zeros(n_items, dtype=torch.int32, device=dev)
+        h.mf_user_item_histogram(self.R.data_ptr(), n, ucnt.data_ptr(), icnt.data_ptr(), st)
+        self.sides = []
+        for cnt, num, req in ((ucnt, n_users, ug), (icnt, n_items, ig)):
+            idx = torch.empty(num, dtype=torch.int32, device=dev)
+            h.mf_init_idx_arr(idx.data_ptr(), num, st)
+            h.mf_sort_by_count(cnt.data_ptr(), idx.data_ptr(), num, st)
+            sorted_cnt = cnt.cpu().numpy().view(np.uint32)
+            sorted_id = idx.cpu().numpy().view(np.uint32)
+            end = np.zeros(num, np.uint32)
+            g = h.mf_group_end_indices(sorted_cnt.ctypes.data, num, req, end.ctypes.data)
+            end = end[:g].copy()
+            id2sorted = np.empty(num, np.uint32)
+            id2sorted[sorted_id] = np.arange(num, dtype=np.uint32)
+            id2group = np.searchsorted(end, id2sorted).astype(np.uint32)
+            self.sides.append(dict(end=end, id2sorted=id2sorted, id2group=id2group, groups=g, num=num, sorted_cnt=sorted_cnt.copy()))
+        du2s = torch.from_numpy(self.sides[0]["id2sorted"].view(np.int32)).to(dev)
+        di2s = torch.from_numpy(self.sides[1]["id2sorted"].view(np.int32)).to(dev)
+        h.mf_matrix_reconst_triplet(self.R.data_ptr(), du2s.data_ptr(), di2s.data_ptr(), n, st)
+        self.test = None
+        if test is not None:
+            self.test = test.clone()
+            h.mf_matrix_reconst_triplet(self.test.data_ptr(), du2s.data_ptr(), di2s.data_ptr(), self.test.shape[0], st)
+        # model init (model_init.cu:114-173) and scatter into binary16 groups (model_init.cu:175-222)
+        for side, (s, d_id2sorted) in enumerate(zip(self.sides, (du2s, di2s))):
+            num, g, end = s["num"], s["groups"], s["end"]
+            dense = torch.empty(num * k, dtype=torch.float32, device=dev)
+            h.mf_init_rand_feature(dense.data_ptr(), num * k, seed, side, st)
+            sizes = np.diff(np.concatenate([[-1], end.astype(np.int64)]))
+            offs = np.concatenate([[0], np.cumsum((sizes * k * 2 + 255) // 256 * 256)[:-1]])
+            arena = torch.zeros(int((sizes * k * 2 + 255).sum() // 1 + 256 * g), dtype=torch.uint8, device=dev)
+            ptrs = torch.tensor([arena.data_ptr() + int(o) for o in offs], dtype=torch.int64, device=dev)
+            d_end = torch.from_numpy(end.view(np.int32)).to(dev)
+            d_prec = torch.zeros(g, dtype=torch.uint8, device=dev)
+            d_id2group = torch.from_numpy(s["id2group"].view(np.int32)).to(dev)
+            h.mf_cpyparams2grouped_params(dense.data_ptr(), ptrs.data_ptr(), d_end.data_ptr(), d_id2group.data_ptr(),
+                                          d_id2sorted.data_ptr(), k, num, g, st)
+            s.update(arena=arena, ptrs=ptrs, d_end=d_end, d_prec=d_prec, sizes=sizes, offs=offs)
+            torch.cuda.synchronize()
+            s["initial"] = arena.clone()
+        self.stats = None
+        self.opt = None
+        self.opt_keep = []
+
+    def reset(self):
+        for s in self.sides:
+            s["arena"].copy_(s["initial"])
+
+    def make_options(self, W, replicate=0.0, thin=0.0, launches=1, add_within=0.0):
+        """mf_hogwild_options as mf_train builds them: hot-row tables from the rating counts (rows are in popularity-sorted
+        order), replica arrays for rows above `replicate` updates in flight.  Returns the number of replicated rows per side."""
+        import torch
+        capi = importlib.import_module("icdm-2021_mascot_amd.capi")
+        h, dev = self.h, self.R.device
+        o = capi.HogwildOptions()
+        o.launches = launches
+        F = h.mf_hogwild_inflight(1, self.k, W, self.sides[0]["groups"], self.sides[1]["groups"])
+        self.opt_keep, slots = [], []
+        for side, s in enumerate(self.sides):
+            cnt = np.ascontiguousarray(s["sorted_cnt"], np.uint32)
+            t = np.empty(cnt.size, np.uint8); slot = np.zeros(cnt.size, np.uint16); slot_row = np.zeros(65536, np.uint32)
+            ns = C.c_uint32(0)
+            h.mf_hot_row_table(cnt.ctypes.data, cnt.size, self.n, F, replicate, thin, add_within, t.ctypes.data, slot.ctypes.data, slot_row.ctypes.data, C.addressof(ns))
+            ns = ns.value
+            dt, dslot, dsr = to_dev(t), to_dev(slot), to_dev(slot_row[:max(ns, 1)])
+            rep = torch.zeros(max(256, 8 * ns * self.k * 4), dtype=torch.uint8, device=dev)
+            self.opt_keep += [dt, dslot, dsr, rep]
+            slots.append(ns)
+            if side == 0:
+                o.user_keep, o.user_slot, o.user_slot_row, o.user_replicas, o.user_slots = dt.data_ptr(), dslot.data_ptr(), dsr.data_ptr(), rep.data_ptr(), ns
+            else:
+                o.item_keep, o.item_slot, o.item_slot_row, o.item_replicas, o.item_slots = dt.data_ptr(), dslot.data_ptr(), dsr.data_ptr(), rep.data_ptr(), ns
+        self.opt = o
+        return slots
+
+    def alloc_stats(self, W):
+        torch, h, k = self.torch, self.h, self.k
+        nb = h.mf_mascot_norm_blocks(W)
+        U, I = self.sides
+        dev = self.R.device
+        self.stats = dict(W=W, nb=nb,
+                          gsp=torch.zeros(U["groups"] * k, device=dev), gsq=torch.zeros(I["groups"] * k, device=dev),
+                          nsp=torch.zeros(U["groups"] * nb, device=dev), nsq=torch.zeros(I["groups"] * nb, device=dev))
+
+    def epoch(self, e, W, epochs, lr0, decay, lam, sample_ratio, interval, seed):
+        h, U, I, s = self.h, self.sides[0], self.sides[1], self.stats
+        st = self.torch.cuda.current_stream().cuda_stream
+        uc = h.mf_update_count(self.n, W, 128)
+        first = h.mf_first_sample_rating_idx(e, interval, epochs, uc, 128, sample_ratio)
+        if first < uc * 128:
+            s["gsp"].zero_()
+            s["gsq"].zero_()
+        h.mf_mascot_sgd_hogwild_opt(self.R.data_ptr(), self.n, U["ptrs"].data_ptr(), I["ptrs"].data_ptr(), self.k, W, uc, 128,
+                                    h.mf_lr_schedule(lr0, decay, e), lam, U["d_end"].data_ptr(), I["d_end"].data_ptr(),
+                                    U["d_prec"].data_ptr(), I["d_prec"].data_ptr(), s["gsp"].data_ptr(), s["gsq"].data_ptr(),
+                                    s["nsp"].data_ptr(), s["nsq"].data_ptr(), first, U["groups"], I["groups"], seed, e, None, st,
+                                    C.addressof(self.opt) if self.opt is not None else None)
+        return uc
+
+    def rmse(self):
+        torch, h, U, I = self.torch, self.h, self.sides[0], self.sides[1]
+        acc = torch.zeros(1, dtype=torch.float64, device=self.R.device)
+        h.mf_test_rmse_grouped(self.test.data_ptr(), self.test.shape[0], U["ptrs"].data_ptr(), I["ptrs"].data_ptr(), self.k,
+                               U["d_end"].data_ptr(), I["d_end"].data_ptr(), U["d_prec"].data_ptr(), I["d_prec"].data_ptr(),
+                               U["groups"], I["groups"], acc.data_ptr(), torch.cuda.current_stream().cuda_stream)
+        return float(np.sqrt(acc.item() / self.test.shape[0]))

@@ -249,21 +249,26 @@ def test_row_traffic_probe_leaves_rows_unchanged(row_bytes, coherent):
     R["u"] = rng.integers(0, n_users, n); R["i"] = rng.integers(0, n_items, n); R["r"] = 1.0
     P = rng.integers(0, 256, n_users * row_bytes, dtype=np.uint8)
     Q = rng.integers(0, 256, n_items * row_bytes, dtype=np.uint8)
-    ku = rng.choice(np.array([0, 100, 254, 255], np.uint8), n_users)
-    kv = rng.choice(np.array([0, 100, 254, 255], np.uint8), n_items)
-    dR, dP, dQ, dku, dkv = to_dev(R), to_dev(P), to_dev(Q), to_dev(ku), to_dev(kv)
-    for tables in ((None, None), (dku.data_ptr(), dkv.data_ptr())):
+    ku = rng.choice(np.array([0, 100, 252, 253, 254, 255], np.uint8), n_users)
+    kv = rng.choice(np.array([0, 100, 252, 253, 254, 255], np.uint8), n_items)
+    dR, dP, dQ = to_dev(R), to_dev(P), to_dev(Q)
+    k = row_bytes // 2
+    plain = mfutil.HogwildOptions(k if k <= 128 else 128, cached_rows=1 - coherent)
+    tables = mfutil.HogwildOptions(k if k <= 128 else 128, ku, kv, cached_rows=1 - coherent)
+    for opt in (plain, tables):
         for workers in (1, 7, 4096):
-            h.mf_row_traffic_probe(dR.data_ptr(), n, dP.data_ptr(), dQ.data_ptr(), row_bytes, workers, tables[0], tables[1], 5, coherent, mfutil.stream_ptr())
+            h.mf_row_traffic_probe(dR.data_ptr(), n, dP.data_ptr(), dQ.data_ptr(), row_bytes, workers, 5, mfutil.stream_ptr(), opt.ptr)
+    h.mf_row_traffic_probe(dR.data_ptr(), n, dP.data_ptr(), dQ.data_ptr(), row_bytes, 64, 5, mfutil.stream_ptr(), None)
     torch.cuda.synchronize()
     assert np.array_equal(from_dev(dP, np.uint8), P) and np.array_equal(from_dev(dQ, np.uint8), Q)
     from importlib import import_module
     MfError = import_module("icdm-2021_mascot_amd.capi").MfError
     with pytest.raises(MfError, match="row_bytes must be"):
-        h.mf_row_traffic_probe(dR.data_ptr(), n, dP.data_ptr(), dQ.data_ptr(), 64, 4, None, None, 5, coherent, mfutil.stream_ptr())
+        h.mf_row_traffic_probe(dR.data_ptr(), n, dP.data_ptr(), dQ.data_ptr(), 64, 4, 5, mfutil.stream_ptr(), None)
+    tables.o.item_keep = None
     with pytest.raises(MfError, match="both keep tables"):
-        h.mf_row_traffic_probe(dR.data_ptr(), n, dP.data_ptr(), dQ.data_ptr(), row_bytes, 4, dku.data_ptr(), None, 5, coherent, mfutil.stream_ptr())
-    h.mf_row_traffic_probe(None, 0, None, None, row_bytes, 4, None, None, 5, coherent, mfutil.stream_ptr())      # nothing to do
+        h.mf_row_traffic_probe(dR.data_ptr(), n, dP.data_ptr(), dQ.data_ptr(), row_bytes, 4, 5, mfutil.stream_ptr(), tables.ptr)
+    h.mf_row_traffic_probe(None, 0, None, None, row_bytes, 4, 5, mfutil.stream_ptr(), None)      # nothing to do
 
 
 @pytest.mark.parametrize("config", [1, 4, 5])

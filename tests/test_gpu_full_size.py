@@ -1,7 +1,8 @@
-"""The hot path at BASELINE.json's full size (configuration 4: 480,000 x 17,800, 100M training ratings), checked through
-properties that do not need a CPU run of that size: range independence of the generator, exact integer invariants of
-the pre-processing kernels, and an epoch with learning rate 0, which must leave every value of the model as it was
-(every row address of 100M updates stays inside its row) before a real epoch lowers the test RMSE."""
+"""The hot path at BASELINE.json's full sizes (configuration 4: 480,000 x 17,800, 100M training ratings; configuration
+5: 1,000,000 x 625,000, 250M training ratings), checked through properties that do not need a CPU run of that size:
+range independence of the generator, exact integer invariants of the pre-processing kernels, and an epoch with
+learning rate 0, which must leave every value of the model as it was (every row address of 100M / 250M updates stays
+inside its row, replicated rows included) before real epochs lower the test RMSE."""
 import ctypes as C
 import os
 import sys
@@ -15,17 +16,21 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 pytestmark = pytest.mark.gpu
 
 
-@pytest.fixture(scope="module")
-def full():
+def _generate(config):
     import torch
-    sys.path.insert(0, ROOT)
-    import bench
     h = mfutil.hip()
-    c = h.synth_config(4)
+    c = h.synth_config(config)
     n, nt = int(c.n_train), int(c.n_test)
     R = torch.empty((n + nt, 3), dtype=torch.int32, device="cuda")
     h.mf_generate_ratings(C.addressof(c), 2021, 0, n + nt, R.data_ptr(), mfutil.stream_ptr())
-    return dict(torch=torch, bench=bench, h=h, c=c, n=n, nt=nt, R=R)
+    return dict(torch=torch, h=h, c=c, n=n, nt=nt, R=R)
+
+
+@pytest.fixture(scope="module")
+def full():
+    d = _generate(4)
+    yield d
+    d.clear()
 
 
 def test_generator_ranges_and_marginals(full):
@@ -76,17 +81,19 @@ def test_preprocessing_invariants(full):
     del S, ka, kb
 
 
-def test_epoch_with_zero_learning_rate_changes_nothing_then_training_learns(full):
-    torch, bench, h, n = full["torch"], full["bench"], full["h"], full["n"]
-    R = full["R"]
-    prob = bench.MascotProblem(torch, h, R[:n].contiguous(), 480_000, 17_800, 128, 100, 100, 2021, test=R[n:].contiguous())
+def _zero_rate_then_learning(d, n_users, n_items, learns_by):
+    """A plain epoch and a check epoch (sampled launch) with learning rate 0 -- with the default hot-row treatment, rows
+    added to and rows replicated per XCD -- leave the model value for value as it was; two real epochs lower the test RMSE."""
+    torch, h, n, R = d["torch"], d["h"], d["n"], d["R"]
+    prob = mfutil.MascotProblem(torch, h, R[:n].contiguous(), n_users, n_items, 128, 100, 100, 2021, test=R[n:].contiguous())
     W = h.mf_auto_workers(n)
     prob.alloc_stats(W)
     before = [s["arena"].clone() for s in prob.sides]
     rmse0 = prob.rmse()
-    prob.set_hot_rows(W, 2.0, 8.0, 2)
-    for e in (0, 5):                      # an early plain epoch (cap 8) and a check epoch (sampled launch, cap 2)
-        prob.select_hot_rows(e)
+    mean_rating = float(R[:1_000_000, 0].view(torch.float32).abs().mean())
+    slots = prob.make_options(W, replicate=h.mf_replicate_threshold(0.01, mean_rating), launches=4)
+    assert slots[1] > 0                   # the popular items are replicated at these sizes
+    for e in (0, 5):
         prob.epoch(e, W, 50, 0.0, 0.1, 0.015, 0.05, 2, 2021)
     torch.cuda.synchronize()
     for s, b in zip(prob.sides, before):
@@ -98,10 +105,41 @@ def test_epoch_with_zero_learning_rate_changes_nothing_then_training_learns(full
     assert abs(prob.rmse() - rmse0) < 1e-9                     # partial sums meet in a different order
     # the sampled sums of the check epoch are finite and non-zero for binary16 groups
     assert bool(torch.isfinite(prob.stats["gsp"]).all()) and float(prob.stats["nsp"].sum()) > 0
-    # two real epochs: the test RMSE falls
     for e in (0, 1):
-        prob.select_hot_rows(e)
         prob.epoch(e, W, 50, 0.01, 0.1, 0.015, 0.05, 2, 2021)
     r2 = prob.rmse()
-    prob.set_hot_rows(W, 0.0)
-    assert np.isfinite(r2) and r2 < rmse0 - 0.5
+    assert np.isfinite(r2) and r2 < rmse0 - learns_by, (rmse0, r2)
+    for s in prob.sides:
+        even = s["arena"].numel() // 2 * 2
+        assert bool(torch.isfinite(s["arena"][:even].view(torch.float16).float()).all())
+
+
+def test_epoch_with_zero_learning_rate_changes_nothing_then_training_learns(full):
+    _zero_rate_then_learning(full, 480_000, 17_800, 0.5)
+
+
+def test_config5_full_size():
+    """BASELINE configuration 5 (1M x 625k, 250M training and 4M test ratings, Zipf(1.2) on both sides, bimodal 0..100
+    ratings mapped to r/25 + 1 as the reference maps its 0..100 data set, io_utils.h:75): the generator's ranges, grid and
+    modes, then the zero-rate and learning properties of the MASCOT epoch at that size (model rows far beyond L2 and MALL)."""
+    d = _generate(5)
+    torch, h, c, n, R = d["torch"], d["h"], d["c"], d["n"], d["R"]
+    assert n == 250_000_000 and d["nt"] == 4_000_000
+    half = torch.empty((n // 4, 3), dtype=torch.int32, device="cuda")
+    h.mf_generate_ratings(C.addressof(c), 2021, n // 2, n // 4, half.data_ptr(), mfutil.stream_ptr())
+    assert torch.equal(half, R[n // 2:n // 2 + n // 4])
+    del half
+    u, i, r = R[:n, 1], R[:n, 2], R[:n, 0].view(torch.float32)
+    assert int(u.max()) < c.n_users and int(i.max()) < c.n_items and int(u.min()) >= 0 and int(i.min()) >= 0
+    raw = torch.round((r[:50_000_000].double() - 1.0) / 0.04)                       # back to 0..100
+    assert float(raw.min()) >= 0 and float(raw.max()) <= 100
+    assert bool(((raw * 0.04 + 1.0).float() == r[:50_000_000]).all())              # exactly the r/25 + 1 grid
+    low = raw[raw < 50]
+    assert abs(low.numel() / raw.numel() - 0.5) < 0.001 and abs(float(low.mean()) - 20.5) < 0.2
+    for ids, count in ((u, c.n_users), (i, c.n_items)):                               # the Zipf(1.2) head
+        share = 1.0 / float((torch.arange(1, count + 1, dtype=torch.float64) ** -1.2).sum())
+        top = int(torch.bincount(ids).max())
+        assert abs(top - n * share) < 6 * np.sqrt(n * share)
+    del raw, low, u, i, r
+    # nothing to learn beyond the mean (the ratings are noise around two modes): the RMSE falls from |r| to the spread
+    _zero_rate_then_learning(d, 1_000_000, 625_000, 0.5)

@@ -398,7 +398,7 @@ def test_argument_errors_launch_nothing():
 @pytest.mark.parametrize("k", [64, 128])
 @pytest.mark.parametrize("variant", ["single", "mascot", "mascot_ff", "mascot_hf"])
 def test_hot_row_thinning_drops_whole_row_updates(orc, k, variant):
-    """mf_set_hot_row_thinning: 255 = ordinary row, nothing changes; 254 = hot row, every update carried out (added
+    """mf_hogwild_options keep tables: 255 = ordinary row, nothing changes; 254 = hot row, every update carried out (added
     in memory: with one update per row the sum equals the stored row, up to the extra rounding of the binary16
     change); 63 carries out a quarter of a row's updates, a skipped row is left untouched while the other side of
     the rating is updated exactly as without thinning."""
@@ -426,28 +426,22 @@ def test_hot_row_thinning_drops_whole_row_updates(orc, k, variant):
 
     def run(keep_u, keep_v):
         dR, dS = to_dev(R), to_dev(starts)
-        ku = torch.full((n,), keep_u, dtype=torch.uint8, device="cuda")
-        kv = torch.full((n,), keep_v, dtype=torch.uint8, device="cuda")
-        h.mf_set_hot_row_thinning(ku.data_ptr(), kv.data_ptr())
-        try:
-            if variant == "single":
-                dP, dQ = to_dev(P0), to_dev(Q0)
-                h.mf_single_sgd_hogwild(dR.data_ptr(), n, dP.data_ptr(), dQ.data_ptr(), k, 1, uc, 128, LR, LAM, 5, 0, dS.data_ptr(), mfutil.stream_ptr())
-                torch.cuda.synchronize()
-                return from_dev(dP, np.float32, P0.shape), from_dev(dQ, np.float32, Q0.shape)
-            gp = mfutil.host_grouped(orc, k, P0, end, uprec)
-            gq = mfutil.host_grouped(orc, k, Q0, end, iprec)
-            dp, dq = mfutil.DeviceGrouped(gp), mfutil.DeviceGrouped(gq)
-            z = torch.zeros(4 * k + 16, dtype=torch.float32, device="cuda")
-            h.mf_mascot_sgd_hogwild(dR.data_ptr(), n, dp.ptrs.data_ptr(), dq.ptrs.data_ptr(), k, 1, uc, 128, LR, LAM,
+        opt = mfutil.HogwildOptions(k, np.full(n, keep_u, np.uint8), np.full(n, keep_v, np.uint8))
+        if variant == "single":
+            dP, dQ = to_dev(P0), to_dev(Q0)
+            h.mf_single_sgd_hogwild_opt(dR.data_ptr(), n, dP.data_ptr(), dQ.data_ptr(), k, 1, uc, 128, LR, LAM, 5, 0, dS.data_ptr(), mfutil.stream_ptr(), opt.ptr)
+            torch.cuda.synchronize()
+            return from_dev(dP, np.float32, P0.shape), from_dev(dQ, np.float32, Q0.shape)
+        gp = mfutil.host_grouped(orc, k, P0, end, uprec)
+        gq = mfutil.host_grouped(orc, k, Q0, end, iprec)
+        dp, dq = mfutil.DeviceGrouped(gp), mfutil.DeviceGrouped(gq)
+        z = torch.zeros(4 * k + 16, dtype=torch.float32, device="cuda")
+        h.mf_mascot_sgd_hogwild_opt(dR.data_ptr(), n, dp.ptrs.data_ptr(), dq.ptrs.data_ptr(), k, 1, uc, 128, LR, LAM,
                                     dp.end.data_ptr(), dq.end.data_ptr(), dp.prec.data_ptr(), dq.prec.data_ptr(),
                                     z.data_ptr(), z[k:].data_ptr(), z[2 * k:].data_ptr(), z[3 * k:].data_ptr(),
-                                    uc * 128, 1, 1, 5, 0, dS.data_ptr(), mfutil.stream_ptr())
-            torch.cuda.synchronize()
-            return rows(dp.download()[0]), rows(dq.download()[0])
-        finally:
-            torch.cuda.synchronize()
-            h.mf_set_hot_row_thinning(None, None)
+                                    uc * 128, 1, 1, 5, 0, dS.data_ptr(), mfutil.stream_ptr(), opt.ptr)
+        torch.cuda.synchronize()
+        return rows(dp.download()[0]), rows(dq.download()[0])
 
     # the checker's result with every update carried out
     if variant == "single":
@@ -485,6 +479,15 @@ def test_hot_row_thinning_drops_whole_row_updates(orc, k, variant):
     P3, Q3 = run(255, 0)
     assert np.array_equal(P3, Pw)
     assert np.any(Q3 != Q0, axis=1).mean() < 0.02                   # (0+1)/255
+    # 253 = replicated rows: the one worker runs on one XCD, whose copies are the only ones that change, so the rows come
+    # back as that XCD left them -- the reference rule's result, bit for bit (every update carried out, stored, not added)
+    for sides in ((253, 255), (255, 253), (253, 253)):
+        P5, Q5 = run(*sides)
+        assert np.array_equal(P5, Pw) and np.array_equal(Q5, Qw), sides
+    # 252 = replicated rows whose updates are added to the copy: as 254, through the copy and the merge
+    P6, Q6 = run(252, 252)
+    assert same(P6, Pw, P0, uprec[0]) and same(Q6, Qw, Q0, iprec[0])
+    assert np.all(np.any(P6 != P0, axis=1)) and np.all(np.any(Q6 != Q0, axis=1))
 
 
 @pytest.mark.parametrize("k", [64, 128])
@@ -507,40 +510,154 @@ def test_hot_row_updates_add_up(orc, k, variant):
     want = np.zeros(k, np.float32)
     want[R["u"]] = lr * R["r"] * 0.5
     dR, dS = to_dev(R), to_dev(starts)
-    ku = torch.full((n,), 255, dtype=torch.uint8, device="cuda")
-    kv = torch.full((1,), 254, dtype=torch.uint8, device="cuda")
-    h.mf_set_hot_row_thinning(ku.data_ptr(), kv.data_ptr())
-    try:
+    opt = mfutil.HogwildOptions(k, np.full(n, 255, np.uint8), np.full(1, 254, np.uint8))
+    if True:
         if variant == "mascot":
             end_u, end_i = np.array([n - 1], np.uint32), np.array([0], np.uint32)
             gp = mfutil.host_grouped(orc, k, P0, end_u, np.zeros(1, np.uint8))
             gq = mfutil.host_grouped(orc, k, Q0, end_i, np.zeros(1, np.uint8))
             dp, dq = mfutil.DeviceGrouped(gp), mfutil.DeviceGrouped(gq)
             z = torch.zeros(4 * k + 4 * n, dtype=torch.float32, device="cuda")
-            h.mf_mascot_sgd_hogwild(dR.data_ptr(), n, dp.ptrs.data_ptr(), dq.ptrs.data_ptr(), k, n, 1, 1, lr, 0.0,
-                                    dp.end.data_ptr(), dq.end.data_ptr(), dp.prec.data_ptr(), dq.prec.data_ptr(),
-                                    z.data_ptr(), z[k:].data_ptr(), z[2 * k:].data_ptr(), z[2 * k + n:].data_ptr(),
-                                    1, 1, 1, 5, 0, dS.data_ptr(), mfutil.stream_ptr())
+            h.mf_mascot_sgd_hogwild_opt(dR.data_ptr(), n, dp.ptrs.data_ptr(), dq.ptrs.data_ptr(), k, n, 1, 1, lr, 0.0,
+                                        dp.end.data_ptr(), dq.end.data_ptr(), dp.prec.data_ptr(), dq.prec.data_ptr(),
+                                        z.data_ptr(), z[k:].data_ptr(), z[2 * k:].data_ptr(), z[2 * k + n:].data_ptr(),
+                                        1, 1, 1, 5, 0, dS.data_ptr(), mfutil.stream_ptr(), opt.ptr)
             torch.cuda.synchronize()
             got = orc.h2f(dq.download()[0]).reshape(k)
         else:
             dP, dQ = to_dev(P0), to_dev(Q0)
             if variant == "single":
-                h.mf_single_sgd_hogwild(dR.data_ptr(), n, dP.data_ptr(), dQ.data_ptr(), k, n, 1, 1, lr, 0.0, 5, 0, dS.data_ptr(), mfutil.stream_ptr())
+                h.mf_single_sgd_hogwild_opt(dR.data_ptr(), n, dP.data_ptr(), dQ.data_ptr(), k, n, 1, 1, lr, 0.0, 5, 0, dS.data_ptr(), mfutil.stream_ptr(), opt.ptr)
             elif variant == "muppet":       # 32 bit forward and backward: the plain binary32 gradient
                 sm, sn = torch.zeros(k, dtype=torch.float32, device="cuda"), torch.zeros(n, dtype=torch.float32, device="cuda")
-                h.mf_muppet_sgd_hogwild(dR.data_ptr(), n, dP.data_ptr(), dQ.data_ptr(), k, n, 1, 1, lr, 0.0, 1, sm.data_ptr(), sn.data_ptr(),
-                                        32, 32, 5, 0, dS.data_ptr(), mfutil.stream_ptr())
+                h.mf_muppet_sgd_hogwild_opt(dR.data_ptr(), n, dP.data_ptr(), dQ.data_ptr(), k, n, 1, 1, lr, 0.0, 1, sm.data_ptr(), sn.data_ptr(),
+                                            32, 32, 5, 0, dS.data_ptr(), mfutil.stream_ptr(), opt.ptr)
             elif variant == "afp":          # quantised on a power-of-two grid that holds 0.5 and the ratings 1..5
-                h.mf_afp_sgd_hogwild(dR.data_ptr(), n, dP.data_ptr(), dQ.data_ptr(), k, n, 1, 1, lr, 0.0, 0, 5, 0, dS.data_ptr(), mfutil.stream_ptr())
+                h.mf_afp_sgd_hogwild_opt(dR.data_ptr(), n, dP.data_ptr(), dQ.data_ptr(), k, n, 1, 1, lr, 0.0, 0, 5, 0, dS.data_ptr(), mfutil.stream_ptr(), opt.ptr)
             else:
-                h.mf_mpt_sgd_hogwild(dR.data_ptr(), n, dP.data_ptr(), dQ.data_ptr(), k, n, 1, 1, lr, 0, 1024.0, 5, 0, dS.data_ptr(), mfutil.stream_ptr())
+                h.mf_mpt_sgd_hogwild_opt(dR.data_ptr(), n, dP.data_ptr(), dQ.data_ptr(), k, n, 1, 1, lr, 0, 1024.0, 5, 0, dS.data_ptr(), mfutil.stream_ptr(), opt.ptr)
             torch.cuda.synchronize()
             got = from_dev(dQ, np.float32, Q0.shape).reshape(k)
-    finally:
-        torch.cuda.synchronize()
-        h.mf_set_hot_row_thinning(None, None)
     if variant == "afp":        # quantised arithmetic and a small non-zero dot product: every update landed, to 2 %
         assert np.all(np.isfinite(got)) and np.all(np.abs(got - Q0.reshape(k) - want) < 0.02 * want)
     else:
         assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("k", [64, 128])
+@pytest.mark.parametrize("elem", [2, 4])
+def test_replica_sync_copies_out_and_averages_changed_copies(orc, k, elem):
+    """mf_replica_sync_dense, the step the update calls run around every kernel launch for replicated rows: merge = 0
+    fills all eight copies of every slot with its row; merge = 1 sets the row and its copies to the mean of the copies
+    that differ from the row (binary32 sum in XCD order, one division, one rounding), and leaves a row alone when none does."""
+    import torch
+    h = mfutil.hip()
+    rng = np.random.default_rng(k + elem)
+    rows, slots = 40, 6
+    dt = np.float32 if elem == 4 else np.float16
+    M = (rng.standard_normal((rows, k)) * 0.3).astype(dt)
+    slot_row = np.array([3, 39, 0, 17, 18, 5], np.uint32)
+    dM, dS = to_dev(M), to_dev(slot_row)
+    rep = torch.full((8 * slots * k * 4,), 0xAB, dtype=torch.uint8, device="cuda")
+    h.mf_replica_sync_dense(dM.data_ptr(), elem, k, rep.data_ptr(), dS.data_ptr(), slots, 0, mfutil.stream_ptr())
+    torch.cuda.synchronize()
+    R = rep.cpu().numpy().reshape(8, slots, k * 4)
+    for x in range(8):
+        for sl in range(slots):
+            assert np.array_equal(R[x, sl, :k * elem].view(dt), M[slot_row[sl]])
+    assert np.array_equal(from_dev(dM, dt, M.shape), M)
+    # change some copies: slot 0 in XCDs 1, 4, 6; slot 1 in all eight; slot 2 in XCD 7 only; slot 3 in none; slots 4, 5 in two
+    touched = {0: [1, 4, 6], 1: list(range(8)), 2: [7], 3: [], 4: [0, 1], 5: [2, 3]}
+    for sl, xs in touched.items():
+        for x in xs:
+            R[x, sl, :k * elem] = (rng.standard_normal(k) * 0.3).astype(dt).view(np.uint8)
+    rep.copy_(torch.from_numpy(R.reshape(-1)))
+    h.mf_replica_sync_dense(dM.data_ptr(), elem, k, rep.data_ptr(), dS.data_ptr(), slots, 1, mfutil.stream_ptr())
+    torch.cuda.synchronize()
+    got, R2 = from_dev(dM, dt, M.shape), rep.cpu().numpy().reshape(8, slots, k * 4)
+    want = M.copy()
+    for sl, xs in touched.items():
+        if xs:
+            acc = np.zeros(k, np.float32)
+            for x in xs:
+                acc = acc + R[x, sl, :k * elem].view(dt).astype(np.float32)
+            want[slot_row[sl]] = (acc / np.float32(len(xs))).astype(dt)
+    assert np.array_equal(got.view(np.uint8), want.view(np.uint8))
+    for x in range(8):
+        for sl in range(slots):
+            assert np.array_equal(R2[x, sl, :k * elem].view(dt).view(np.uint8), want[slot_row[sl]].view(np.uint8))
+
+
+@pytest.mark.parametrize("variant", ["single", "mem_quant", "mascot"])
+def test_replicated_rows_under_many_workers(orc, variant):
+    """2048 workers on every XCD race on a few replicated rows (each XCD on its own copies) while the other rows are
+    ordinary: the ordinary side of a conflict-free schedule must come out as the checker computes it when the
+    replicated side is not updated at all (learning rate 0 on it is not available, so the check is structural): every
+    value finite, every replicated row moved, the copies of a row equal the row after the call, and a second call
+    with the same inputs starts from the rows, not from stale copies."""
+    import torch
+    h = mfutil.hip()
+    k, n_users, n_items, n = 128, 4096, 8, 2048 * 128
+    rng = np.random.default_rng(99)
+    R = np.zeros(n, mfutil.NODE)
+    R["u"], R["i"], R["r"] = rng.integers(0, n_users, n), rng.integers(0, n_items, n), rng.integers(1, 6, n)
+    P0 = (rng.standard_normal((n_users, k)) * 0.1).astype(np.float32)
+    Q0 = (rng.standard_normal((n_items, k)) * 0.1).astype(np.float32)
+    keep_u, keep_v = np.full(n_users, 255, np.uint8), np.full(n_items, 253, np.uint8)
+    keep_u[:5] = 253
+    opt = mfutil.HogwildOptions(k, keep_u, keep_v, launches=2)
+    dR = to_dev(R)
+    W, uc = 2048, 1
+
+    def call(dP, dQ, epoch):
+        if variant == "single":
+            h.mf_single_sgd_hogwild_opt(dR.data_ptr(), n, dP.data_ptr(), dQ.data_ptr(), k, W, uc, 128, 0.01, 0.02, 5, epoch, None, mfutil.stream_ptr(), opt.ptr)
+        elif variant == "mem_quant":
+            h.mf_mem_quant_sgd_hogwild_opt(dR.data_ptr(), n, dP.data_ptr(), dQ.data_ptr(), k, W, uc, 128, 0.01, 0.02, 5, epoch, None, mfutil.stream_ptr(), opt.ptr)
+        torch.cuda.synchronize()
+
+    if variant == "mascot":
+        end_u, end_i = mfutil.equal_end_idx(n_users, 3), np.array([n_items - 1], np.uint32)
+        uprec = np.array([0, 1, 0], np.uint8)
+        gp = mfutil.host_grouped(orc, k, P0, end_u, uprec)
+        gq = mfutil.host_grouped(orc, k, Q0, end_i, np.zeros(1, np.uint8))
+        dp, dq = mfutil.DeviceGrouped(gp), mfutil.DeviceGrouped(gq)
+        nb = h.mf_mascot_norm_blocks(W)
+        z = torch.zeros(4 * k + 4 * nb, dtype=torch.float32, device="cuda")
+        for epoch in range(2):
+            h.mf_mascot_sgd_hogwild_opt(dR.data_ptr(), n, dp.ptrs.data_ptr(), dq.ptrs.data_ptr(), k, W, uc, 128, 0.01, 0.02,
+                                        dp.end.data_ptr(), dq.end.data_ptr(), dp.prec.data_ptr(), dq.prec.data_ptr(),
+                                        z.data_ptr(), z[3 * k:].data_ptr(), z[4 * k:].data_ptr(), z[4 * k + 3 * nb:].data_ptr(),
+                                        uc * 128, 3, 1, 5, epoch, None, mfutil.stream_ptr(), opt.ptr)
+            torch.cuda.synchronize()
+        Qg = orc.h2f(dq.download()[0]).reshape(n_items, k)
+        Pg = np.concatenate([(a if a.dtype == np.float32 else orc.h2f(a)).reshape(-1, k) for a in dp.download()])
+        P0 = np.concatenate([(a if a.dtype == np.float32 else orc.h2f(a)).reshape(-1, k) for a in gp.arrays])
+        Q0 = orc.h2f(gq.arrays[0]).reshape(n_items, k)
+        elem_q = 2
+    else:
+        if variant == "mem_quant":
+            dP, dQ = to_dev(orc.f2h(P0)), to_dev(orc.f2h(Q0))
+            P0, Q0 = orc.h2f(orc.f2h(P0)).reshape(P0.shape), orc.h2f(orc.f2h(Q0)).reshape(Q0.shape)
+        else:
+            dP, dQ = to_dev(P0), to_dev(Q0)
+        call(dP, dQ, 0)
+        call(dP, dQ, 1)
+        if variant == "mem_quant":
+            Pg, Qg = orc.h2f(from_dev(dP, np.uint16)).reshape(P0.shape), orc.h2f(from_dev(dQ, np.uint16)).reshape(Q0.shape)
+            elem_q = 2
+        else:
+            Pg, Qg = from_dev(dP, np.float32, P0.shape), from_dev(dQ, np.float32, Q0.shape)
+            elem_q = 4
+    assert np.all(np.isfinite(Pg)) and np.all(np.isfinite(Qg))
+    assert np.all(np.any(Qg != Q0, axis=1)) and np.all(np.any(Pg[:5] != P0[:5], axis=1))
+    # two epochs of lr 0.01 on ratings 1..5 from rows of size 0.1: the rows grow, nothing explodes
+    assert np.abs(Qg).max() < 5 and np.abs(Pg).max() < 5
+    touched = np.bincount(R["u"], minlength=n_users) > 0
+    assert np.all(np.any(Pg[touched] != P0[touched], axis=1))
+    # the copies of every item row equal the row after the call (the last merge wrote them)
+    rep = opt.replicas[1].cpu().numpy().reshape(8, n_items, k * 4)
+    dtq = np.float32 if elem_q == 4 else np.float16
+    for x in range(8):
+        for sl in range(n_items):
+            assert np.array_equal(rep[x, sl, :k * elem_q].view(dtq).astype(np.float32), Qg[sl])

@@ -460,7 +460,27 @@ def test_argument_checks_need_no_gpu(lib):
         node = np.zeros(1, NODE); node["u"] = 5
         p = np.zeros(128, np.float32); out = C.c_double(0)
         lib.call("mf_gpu_test_rmse", node.ctypes.data, 1, p.ctypes.data, p.ctypes.data, 1, 1, 128, C.byref(out))
-    assert lib.mf_set_row_coherence(1) == 0 and lib.mf_get_row_coherence() == 1
+    # launch options are checked before anything touches a device
+    o = capi.HogwildOptions()
+    o.cached_rows = 2
+    with pytest.raises(capi.MfError, match="cached_rows is 0"):
+        lib.mf_single_sgd_hogwild_opt(1, 1, 1, 1, 64, 1, 1, 1, 0.01, 0.05, 0, 0, None, None, C.addressof(o))
+    o.cached_rows, o.user_keep = 0, 1
+    with pytest.raises(capi.MfError, match="both hot-row tables or neither"):
+        lib.mf_mpt_sgd_hogwild_opt(1, 1, 1, 1, 64, 1, 1, 1, 0.01, 0, 1000.0, 0, 0, None, None, C.addressof(o))
+    o.item_keep, o.item_slots = 1, 3
+    with pytest.raises(capi.MfError, match="item_slots > 0 needs"):
+        lib.mf_afp_sgd_hogwild_opt(1, 1, 1, 1, 64, 1, 1, 1, 0.01, 0.05, 0, 0, 0, None, None, C.addressof(o))
+    o.item_slot, o.item_slot_row, o.item_replicas = 1, 1, 100
+    with pytest.raises(capi.MfError, match="256-byte aligned"):
+        lib.mf_mem_quant_sgd_hogwild_opt(1, 1, 1, 1, 64, 1, 1, 1, 0.01, 0.05, 0, 0, None, None, C.addressof(o))
+    o.item_replicas, o.item_slots = 256, 70000
+    with pytest.raises(capi.MfError, match="at most 65535 replicated rows"):
+        lib.mf_single_sgd_hogwild_opt(1, 1, 1, 1, 64, 1, 1, 1, 0.01, 0.05, 0, 0, None, None, C.addressof(o))
+    prm = lib.default_params()
+    assert prm.hot_rows == 1 and prm.replicate_inflight < 0 and prm.hot_row_inflight == 0      # replicas by default, thinning is opt-in
+    assert abs(lib.mf_replicate_threshold(0.01, 3.6) - 0.3 / 0.036) < 1e-4
+    assert lib.mf_replicate_threshold(0.01, 100.0) == 2.0 and lib.mf_replicate_threshold(0.0001, 1.0) == 16.0
 
 
 # ---- seeded synthetic ratings (the generator behind `quantized_mf -synth`) ------------------------------------------
@@ -527,29 +547,59 @@ def test_synth_baseline_configs():
 
 
 def test_hot_row_table_closed_form():
-    """mf_hot_row_table: rows with at most one update in flight stay ordinary (255); the others are kept with probability
-    min(1, cap / in flight), stored as floor(keep * 255) - 1 in 0..254."""
+    """mf_hot_row_table: rows with at most one update in flight stay ordinary (255); above replicate_above they are
+    replicated (numbered in row order; 252 = updates added to the copies up to 8 x replicate_above in flight, 253 = stored
+    above); above thin_above they are thinned to that many in flight, stored as floor(keep * 255) - 1 in 0..251; the rest
+    are added (254)."""
     capi = importlib.import_module("icdm-2021_mascot_amd.capi")
     h = capi.load()
-    n, W, cap = 1_000_000, 1000, 2.0
-    F = min(W, 8192) * 4.0                                        # 4000 updates in flight: one per 250 ratings of a row
+    n, F = 1_000_000, 4000.0                                      # 4000 updates in flight: one per 250 ratings of a row
     cnt = np.array([0, 1, 249, 250, 251, 400, 500, 501, 1000, 5000, 250_000, 1_000_000], np.uint32)
-    t = np.empty(cnt.size, np.uint8)
-    h.mf_hot_row_table(cnt.ctypes.data, cnt.size, n, W, cap, t.ctypes.data)
-    want = []
-    for c in cnt.tolist():
-        inflight = F * c / n
-        if inflight <= 1.0:
-            want.append(255)
-        else:
-            keep = min(1.0, cap / inflight)
-            want.append(int(min(254, max(0, math.floor(keep * 255.0) - 1))))
-    assert t.tolist() == want
-    assert t.tolist()[:4] == [255, 255, 255, 255] and t[4] == 254 and t[6] == 254 and t[7] < 254 and t[-1] == 0
-    # more workers than can be resident count as 8192
-    a, b = np.empty(cnt.size, np.uint8), np.empty(cnt.size, np.uint8)
-    h.mf_hot_row_table(cnt.ctypes.data, cnt.size, n, 8192, cap, a.ctypes.data)
-    h.mf_hot_row_table(cnt.ctypes.data, cnt.size, n, 100_000, cap, b.ctypes.data)
-    assert np.array_equal(a, b)
-    with pytest.raises(capi.MfError, match="cap must be positive"):
-        h.mf_hot_row_table(cnt.ctypes.data, cnt.size, n, W, 0.0, t.ctypes.data)
+
+    def table(replicate, thin, add_within=0.0):
+        t = np.empty(cnt.size, np.uint8); slot = np.full(cnt.size, 0xffff, np.uint16); slot_row = np.zeros(cnt.size, np.uint32)
+        ns = C.c_uint32(99)
+        h.mf_hot_row_table(cnt.ctypes.data, cnt.size, n, F, replicate, thin, add_within, t.ctypes.data, slot.ctypes.data, slot_row.ctypes.data, C.addressof(ns))
+        return t, slot, slot_row[:ns.value]
+
+    def want(replicate, thin, add_within=0.0):
+        out = []
+        for c in cnt.tolist():
+            fly = F * c / n
+            if fly <= 1.0:
+                out.append(255)
+            elif replicate > 0 and fly > replicate:
+                out.append(252 if fly <= 8 * add_within else 253)
+            elif thin > 0 and fly > thin:
+                out.append(int(min(251, max(0, math.floor(thin / fly * 255.0) - 1))))
+            else:
+                out.append(254)
+        return out
+
+    # thinning only (the opt-in mode): as before, except that the replicated mark is never produced
+    t, _, rows = table(0.0, 2.0)
+    assert t.tolist() == want(0.0, 2.0) and rows.size == 0
+    assert t.tolist()[:4] == [255, 255, 255, 255] and t[4] == 254 and t[6] == 254 and t[7] < 252 and t[-1] == 0
+    # replicas above 4 in flight (count > 1000), nothing thinned: the default mode
+    t, slot, rows = table(4.0, 0.0)
+    assert t.tolist() == want(4.0, 0.0)
+    assert t.tolist() == [255, 255, 255, 255, 254, 254, 254, 254, 254, 253, 253, 253]
+    t2, _, _ = table(4.0, 0.0, 4.0)                                  # copies with at most 4 in flight per XCD (32 in all) are added to
+    assert t2.tolist() == want(4.0, 0.0, 4.0) == [255, 255, 255, 255, 254, 254, 254, 254, 254, 252, 253, 253]      # 20, 1000, 4000 in flight
+    assert rows.tolist() == [9, 10, 11] and slot[9:].tolist() == [0, 1, 2]
+    # both: replicated above 100 in flight, thinned above 2
+    t, _, rows = table(100.0, 2.0)
+    assert t.tolist() == want(100.0, 2.0) and rows.tolist() == [10, 11]
+    # neither: every hot row is added
+    t, _, rows = table(0.0, 0.0)
+    assert t.tolist() == want(0.0, 0.0) and set(t.tolist()) == {254, 255}
+    with pytest.raises(capi.MfError, match="no updates in flight"):
+        h.mf_hot_row_table(cnt.ctypes.data, cnt.size, n, 0.0, 4.0, 0.0, 0.0, t.ctypes.data, None, None, None)
+    with pytest.raises(capi.MfError, match="need slot"):
+        h.mf_hot_row_table(cnt.ctypes.data, cnt.size, n, F, 4.0, 0.0, 0.0, t.ctypes.data, None, None, None)
+    # at most 65535 replicated rows: the most popular ones
+    many = np.arange(1, 80_001, dtype=np.uint32) * 100
+    t = np.empty(many.size, np.uint8); slot = np.zeros(many.size, np.uint16); slot_row = np.zeros(65535, np.uint32)
+    ns = C.c_uint32(0)
+    h.mf_hot_row_table(many.ctypes.data, many.size, int(many.sum()), 1e9, 4.0, 0.0, 0.0, t.ctypes.data, slot.ctypes.data, slot_row.ctypes.data, C.addressof(ns))
+    assert ns.value == 65535 and np.all(t[-65535:] == 253) and np.all(t[:-65535] == 254)
