@@ -99,7 +99,7 @@ class MfReport(C.Structure):
                 ("user_group_prec_info", vp), ("item_group_prec_info", vp),
                 ("user_group_num", u32), ("item_group_num", u32), ("test_reconst", vp),
                 ("preprocess_ms", f64), ("switching_ms", f64), ("error_ms", f64), ("sgd_ms", f64), ("total_ms", f64),
-                ("update_count", u32), ("muppet_final_bits", u32)]
+                ("update_count", u32), ("muppet_final_bits", u32), ("muppet_bits_per_epoch", vp)]
 
 
 class MfError(RuntimeError):
@@ -171,7 +171,7 @@ class MascotHip:
                    user2sorted=np.zeros(n_users, np.uint32), item2sorted=np.zeros(n_items, np.uint32),
                    user_end=np.zeros(max(prm.user_group_num, 1), np.uint32), item_end=np.zeros(max(prm.item_group_num, 1), np.uint32),
                    user_prec=np.zeros(max(prm.user_group_num, 1), np.uint8), item_prec=np.zeros(max(prm.item_group_num, 1), np.uint8),
-                   test_reconst=np.zeros(test.size, NODE))
+                   test_reconst=np.zeros(test.size, NODE), muppet_bits=np.zeros(E, np.uint8))
         rep = MfReport()
         rep.rmse_per_epoch = out["rmse"].ctypes.data
         rep.lr_per_epoch = out["lr"].ctypes.data
@@ -183,6 +183,7 @@ class MascotHip:
         rep.user_group_prec_info = out["user_prec"].ctypes.data
         rep.item_group_prec_info = out["item_prec"].ctypes.data
         rep.test_reconst = out["test_reconst"].ctypes.data
+        rep.muppet_bits_per_epoch = out["muppet_bits"].ctypes.data
         R = np.ascontiguousarray(R)
         test = np.ascontiguousarray(test)
         self.call("mf_train", C.byref(prm), R.ctypes.data, R.size, n_users, n_items, test.ctypes.data, test.size,

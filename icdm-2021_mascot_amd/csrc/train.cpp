@@ -376,6 +376,7 @@ struct DenseRun : Run {
                                               c.lr[e], scaled_lambda_h, scaling_factor, prm.seed, e, nullptr, nullptr, opt)); break;
         case 3: {
             const int idx = precision_idx > 4 ? 4 : precision_idx;      // the reference indexes past the table once at 32 bit (mf_methods.cu:691)
+            if (c.rep && c.rep->muppet_bits_per_epoch) c.rep->muppet_bits_per_epoch[e] = bit_width_set[idx];
             MF_TRY(mf_muppet_sgd_hogwild_opt(R, c.n, d_p.as<float>(), d_q.as<float>(), (int)c.k, prm.num_workers, c.update_count, c.update_vector_size,
                                              c.lr[e], prm.lambda, muppet_first_sample, d_sum_updated.as<float>(), d_sum_norms.as<float>(),
                                              bit_width_set[idx], bit_width_set[idx], prm.seed, e, nullptr, nullptr, opt));

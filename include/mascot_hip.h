@@ -377,6 +377,7 @@ typedef struct {
     double preprocess_ms, switching_ms, error_ms, sgd_ms, total_ms;   /* mf_methods.cu:401-418 */
     uint32_t update_count;
     uint32_t muppet_final_bits;
+    uint8_t* muppet_bits_per_epoch; /* [epoch] MuPPET only: the bit width every epoch ran at (mf_methods.cu:596-601,691) */
 } mf_report;
 
 void mf_default_params(mf_params* out);

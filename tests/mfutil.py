@@ -184,6 +184,7 @@ def oracle_train_dense(orc, version, R, test, P, Q, k, W, epochs, lr, lam, decay
     uc = orc.lib.orc_update_count(Rs.size, W, 128)
     rmse = []
     bits_ladder = [8, 12, 14, 16, 32]
+    bits_hist = []
     pidx, switched, viol, maxdiv = 0, C.c_int(-1), C.c_int(0), C.c_float(-1.0)
     pidx_c = C.c_int(0)
     norms_hist = np.zeros(epochs, np.float32)
@@ -199,6 +200,7 @@ def oracle_train_dense(orc, version, R, test, P, Q, k, W, epochs, lr, lam, decay
             s = np.zeros(k, np.float32)
             nrm = np.zeros(W, np.float32)
             b = bits_ladder[min(pidx_c.value, 4)]
+            bits_hist.append(b)
             orc.lib.orc_muppet_epoch(k, Rs.ctypes.data, Rs.size, P.ctypes.data, Q.ctypes.data, W, uc, 128, lre, lam, first_sample,
                                      s.ctypes.data, nrm.ctypes.data, b, b, seed, e, None, sequential_threads)
             norms_hist[e] = np.float32(nrm.sum(dtype=np.float32))
@@ -208,7 +210,7 @@ def oracle_train_dense(orc, version, R, test, P, Q, k, W, epochs, lr, lam, decay
         elif version == 2:
             orc.lib.orc_afp_epoch(k, Rs.ctypes.data, Rs.size, P.ctypes.data, Q.ctypes.data, W, uc, 128, lre, lam, e, seed, e, None, sequential_threads)
         rmse.append(orc.rmse(k, test, P, Q))
-    return np.array(rmse), dict(final_bits=bits_ladder[min(pidx_c.value, 4)])
+    return np.array(rmse), dict(final_bits=bits_ladder[min(pidx_c.value, 4)], bits=np.array(bits_hist, np.uint8))
 
 
 def oracle_train_mem_quant(orc, R, test, P, Q, k, W, epochs, lr, lam, decay, seed, threads=8):

@@ -133,7 +133,7 @@ def test_config5_full_size():
     assert int(u.max()) < c.n_users and int(i.max()) < c.n_items and int(u.min()) >= 0 and int(i.min()) >= 0
     raw = torch.round((r[:50_000_000].double() - 1.0) / 0.04)                       # back to 0..100
     assert float(raw.min()) >= 0 and float(raw.max()) <= 100
-    assert bool(((raw * 0.04 + 1.0).float() == r[:50_000_000]).all())              # exactly the r/25 + 1 grid
+    assert bool(((raw.float() * 0.04 + 1.0) == r[:50_000_000]).all())              # exactly the r * 0.04 + 1 grid, in binary32 as the generator computes it
     low = raw[raw < 50]
     assert abs(low.numel() / raw.numel() - 0.5) < 0.001 and abs(float(low.mean()) - 20.5) < 0.2
     for ids, count in ((u, c.n_users), (i, c.n_items)):                               # the Zipf(1.2) head
