@@ -61,6 +61,13 @@ SIGNATURES = {
     "mf_session_hot_rows": (i32, [vp, vp, vp, vp]),
     "mf_session_device_state": (i32, [vp, u32, vp, vp]),
     "mf_replicate_threshold": (f32, [f32, f32]),
+    "mf_sort_by_count_workspace_bytes": (C.c_size_t, [u32]),
+    "mf_sort_by_count_ws": (i32, [vp, vp, u32, vp, C.c_size_t, vp]),
+    "mf_shuffle_ratings_workspace_bytes": (C.c_size_t, [u32]),
+    "mf_shuffle_ratings_ws": (i32, [vp, vp, u32, u64, vp, C.c_size_t, vp]),
+    "mf_synth_tables_bytes": (C.c_size_t, [vp]),
+    "mf_synth_build_tables": (i32, [vp, u64, vp, C.c_size_t, vp]),
+    "mf_generate_ratings_ws": (i32, [vp, u64, vp, u64, u64, vp, vp]),
     "mf_replica_sync_dense": (i32, [vp, u32, i32, vp, vp, u32, i32, vp]),
 }
 # the update launches with one more argument, const mf_hogwild_options*

@@ -464,25 +464,6 @@ std::vector<uint32_t> seeded_permutation(uint32_t count, uint64_t base)
     for (uint32_t i = count; i-- > 1;) { const uint32_t j = (uint32_t)(mix64(base ^ (uint64_t)i) % ((uint64_t)i + 1)); std::swap(p[i], p[j]); }
     return p;
 }
-struct DeviceTables {      // frees what it allocated when it goes out of scope
-    std::vector<void*> owned;
-    ~DeviceTables() { for (void* p : owned) (void)hipFree(p); }
-    template <class T> int upload(const std::vector<T>& h, const T** d, hipStream_t st)
-    {
-        void* p = nullptr;
-        if (int rc = check_hip(hipMalloc(&p, h.size() * sizeof(T) + 16), "hipMalloc(synthetic tables)")) return rc;
-        owned.push_back(p);
-        if (int rc = check_hip(hipMemcpyAsync(p, h.data(), h.size() * sizeof(T), hipMemcpyHostToDevice, st), "hipMemcpyAsync(synthetic tables)")) return rc;
-        *d = static_cast<const T*>(p);
-        return MF_OK;
-    }
-    int alloc(size_t bytes, void** d)
-    {
-        if (int rc = check_hip(hipMalloc(d, bytes + 16), "hipMalloc(synthetic factors)")) return rc;
-        owned.push_back(*d);
-        return MF_OK;
-    }
-};
 }  // namespace
 
 extern "C" {
@@ -649,37 +630,91 @@ int mf_synth_baseline_config(int config, mf_synth_config* out)
     return MF_OK;
 }
 
-int mf_generate_ratings(const mf_synth_config* cfg, uint64_t seed, uint64_t first, uint64_t count, mf_node* out, void* stream)
+static int check_synth(const char* who, const mf_synth_config* cfg)
 {
-    if (!cfg) return invalid("mf_generate_ratings: null configuration");
-    if (count == 0) return MF_OK;
-    if (!out) return invalid("mf_generate_ratings: null output");
-    const mf_synth_config c = *cfg;
-    if (c.n_users == 0 || c.n_items == 0) return invalid("mf_generate_ratings: no users or no items");
-    if (!c.bimodal && (c.rank == 0 || c.rank > 1024u)) return invalid("mf_generate_ratings: rank must be 1..1024 (got %u)", c.rank);
-    if (!(c.step > 0.0f) || !(c.lo <= c.hi)) return invalid("mf_generate_ratings: step must be positive and lo <= hi");
-    hipStream_t st = as_stream(stream);
-    const uint64_t key = mix64(seed ^ 0x53594E5448455449ull);
-    DeviceTables dev;
+    if (!cfg) return invalid("%s: null configuration", who);
+    if (cfg->n_users == 0 || cfg->n_items == 0) return invalid("%s: no users or no items", who);
+    if (!cfg->bimodal && (cfg->rank == 0 || cfg->rank > 1024u)) return invalid("%s: rank must be 1..1024 (got %u)", who, cfg->rank);
+    if (!(cfg->step > 0.0f) || !(cfg->lo <= cfg->hi)) return invalid("%s: step must be positive and lo <= hi", who);
+    return MF_OK;
+}
+// Workspace layout of the generator's tables: user CDF, item CDF (binary64), user permutation, item permutation
+// (uint32), and unless bimodal the factors U [users][rank], V [items][rank] (binary32); every part 256-byte aligned.
+struct SynthLayout { size_t ucdf, icdf, uperm, iperm, U, V, total; };
+static SynthLayout synth_layout(const mf_synth_config& c)
+{
+    auto al = [](size_t b) { return (b + 255) / 256 * 256; };
+    SynthLayout l;
+    l.ucdf = 0; l.icdf = l.ucdf + al((size_t)c.n_users * 8); l.uperm = l.icdf + al((size_t)c.n_items * 8);
+    l.iperm = l.uperm + al((size_t)c.n_users * 4); l.U = l.iperm + al((size_t)c.n_items * 4);
+    const size_t fu = c.bimodal ? 0 : al((size_t)c.n_users * c.rank * 4), fv = c.bimodal ? 0 : al((size_t)c.n_items * c.rank * 4);
+    l.V = l.U + fu; l.total = l.V + fv;
+    return l;
+}
+static SynthTables synth_tables(const mf_synth_config& c, const void* workspace)
+{
+    const SynthLayout l = synth_layout(c);
+    const uint8_t* ws = static_cast<const uint8_t*>(workspace);
     SynthTables t = {};
+    t.user_cdf = reinterpret_cast<const double*>(ws + l.ucdf); t.item_cdf = reinterpret_cast<const double*>(ws + l.icdf);
+    t.user_perm = reinterpret_cast<const uint32_t*>(ws + l.uperm); t.item_perm = reinterpret_cast<const uint32_t*>(ws + l.iperm);
+    if (!c.bimodal) { t.U = reinterpret_cast<const float*>(ws + l.U); t.V = reinterpret_cast<const float*>(ws + l.V); }
+    return t;
+}
+static uint64_t synth_key(uint64_t seed) { return mix64(seed ^ 0x53594E5448455449ull); }
+
+size_t mf_synth_tables_bytes(const mf_synth_config* cfg)
+{
+    if (check_synth("mf_synth_tables_bytes", cfg)) return 0;
+    return synth_layout(*cfg).total;
+}
+int mf_synth_build_tables(const mf_synth_config* cfg, uint64_t seed, void* workspace, size_t workspace_bytes, void* stream)
+{
+    if (int rc = check_synth("mf_synth_build_tables", cfg)) return rc;
+    const mf_synth_config c = *cfg;
+    const SynthLayout l = synth_layout(c);
+    if (!workspace || reinterpret_cast<uintptr_t>(workspace) % 256) return invalid("mf_synth_build_tables: the workspace must be non-null and 256-byte aligned");
+    if (workspace_bytes < l.total) return invalid("mf_synth_build_tables: the workspace holds %zu bytes, the tables need %zu (mf_synth_tables_bytes)", workspace_bytes, l.total);
+    hipStream_t st = as_stream(stream);
+    uint8_t* ws = static_cast<uint8_t*>(workspace);
+    const uint64_t key = synth_key(seed);
     const std::vector<double> ucdf = zipf_cdf(c.n_users, c.user_alpha), icdf = zipf_cdf(c.n_items, c.item_alpha);
     const std::vector<uint32_t> uperm = seeded_permutation(c.n_users, mix64(key + 1)), iperm = seeded_permutation(c.n_items, mix64(key + 2));
-    if (int rc = dev.upload(ucdf, &t.user_cdf, st)) return rc;
-    if (int rc = dev.upload(icdf, &t.item_cdf, st)) return rc;
-    if (int rc = dev.upload(uperm, &t.user_perm, st)) return rc;
-    if (int rc = dev.upload(iperm, &t.item_perm, st)) return rc;
+    if (int rc = check_hip(hipMemcpyAsync(ws + l.ucdf, ucdf.data(), ucdf.size() * 8, hipMemcpyHostToDevice, st), "hipMemcpyAsync(synthetic tables)")) return rc;
+    if (int rc = check_hip(hipMemcpyAsync(ws + l.icdf, icdf.data(), icdf.size() * 8, hipMemcpyHostToDevice, st), "hipMemcpyAsync(synthetic tables)")) return rc;
+    if (int rc = check_hip(hipMemcpyAsync(ws + l.uperm, uperm.data(), uperm.size() * 4, hipMemcpyHostToDevice, st), "hipMemcpyAsync(synthetic tables)")) return rc;
+    if (int rc = check_hip(hipMemcpyAsync(ws + l.iperm, iperm.data(), iperm.size() * 4, hipMemcpyHostToDevice, st), "hipMemcpyAsync(synthetic tables)")) return rc;
     if (!c.bimodal) {
-        void *U = nullptr, *V = nullptr;
         const uint64_t nu = (uint64_t)c.n_users * c.rank, nv = (uint64_t)c.n_items * c.rank;
-        if (int rc = dev.alloc(nu * sizeof(float), &U)) return rc;
-        if (int rc = dev.alloc(nv * sizeof(float), &V)) return rc;
-        hipLaunchKernelGGL(init_normal_kernel, dim3(stream_grid(nu)), dim3(kStreamBlock), 0, st, static_cast<float*>(U), nu, mix64(key + 3), 0.5);
-        hipLaunchKernelGGL(init_normal_kernel, dim3(stream_grid(nv)), dim3(kStreamBlock), 0, st, static_cast<float*>(V), nv, mix64(key + 4), 0.5);
-        t.U = static_cast<const float*>(U); t.V = static_cast<const float*>(V);
+        hipLaunchKernelGGL(init_normal_kernel, dim3(stream_grid(nu)), dim3(kStreamBlock), 0, st, reinterpret_cast<float*>(ws + l.U), nu, mix64(key + 3), 0.5);
+        hipLaunchKernelGGL(init_normal_kernel, dim3(stream_grid(nv)), dim3(kStreamBlock), 0, st, reinterpret_cast<float*>(ws + l.V), nv, mix64(key + 4), 0.5);
+        if (int rc = launch_status("mf_synth_build_tables")) return rc;
     }
-    hipLaunchKernelGGL(generate_ratings_kernel, dim3(stream_grid(count)), dim3(kStreamBlock), 0, st, c, t, key, first, count, 1.0f / c.step, out);
-    if (int rc = launch_status("mf_generate_ratings")) return rc;
-    return check_hip(hipStreamSynchronize(st), "mf_generate_ratings: hipStreamSynchronize");       // the tables are freed on return
+    // the host-side tables above go out of scope on return: wait for their copies (the one synchronisation of the generator)
+    return check_hip(hipStreamSynchronize(st), "mf_synth_build_tables: hipStreamSynchronize");
+}
+int mf_generate_ratings_ws(const mf_synth_config* cfg, uint64_t seed, const void* tables, uint64_t first, uint64_t count, mf_node* out, void* stream)
+{
+    if (int rc = check_synth("mf_generate_ratings_ws", cfg)) return rc;
+    if (count == 0) return MF_OK;
+    if (!out || !tables) return invalid("mf_generate_ratings_ws: null output or tables");
+    const mf_synth_config c = *cfg;
+    hipLaunchKernelGGL(generate_ratings_kernel, dim3(stream_grid(count)), dim3(kStreamBlock), 0, as_stream(stream), c, synth_tables(c, tables), synth_key(seed), first, count, 1.0f / c.step, out);
+    return launch_status("mf_generate_ratings_ws");
+}
+int mf_generate_ratings(const mf_synth_config* cfg, uint64_t seed, uint64_t first, uint64_t count, mf_node* out, void* stream)
+{
+    if (int rc = check_synth("mf_generate_ratings", cfg)) return rc;
+    if (count == 0) return MF_OK;
+    if (!out) return invalid("mf_generate_ratings: null output");
+    const size_t bytes = synth_layout(*cfg).total;
+    void* ws = nullptr;
+    if (int rc = check_hip(hipMalloc(&ws, bytes), "mf_generate_ratings: hipMalloc(tables)")) return rc;
+    int rc = mf_synth_build_tables(cfg, seed, ws, bytes, stream);
+    if (rc == MF_OK) rc = mf_generate_ratings_ws(cfg, seed, ws, first, count, out, stream);
+    if (rc == MF_OK) rc = check_hip(hipStreamSynchronize(as_stream(stream)), "mf_generate_ratings: hipStreamSynchronize");       // the tables are freed on return
+    (void)hipFree(ws);
+    return rc;
 }
 
 int mf_generate_ratings_host(const mf_synth_config* cfg, uint64_t seed, uint64_t first, uint64_t count, mf_node* host_out)

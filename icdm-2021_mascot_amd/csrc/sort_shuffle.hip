@@ -28,57 +28,113 @@ struct DeviceBuffers {
     ~DeviceBuffers() { for (void* p : ptr) if (p) (void)hipFree(p); }
 };
 
+constexpr size_t kAlign = 256;
+static inline size_t aligned(size_t bytes) { return (bytes + kAlign - 1) / kAlign * kAlign; }
+
+// Workspace layout of the count sort: sorted counts, sorted ids (the radix sort's output buffers), rocPRIM's own
+// temporary storage.  The size query only computes sizes; it needs a current device (rocPRIM picks its kernel
+// configuration by architecture).
+static int sort_layout(uint32_t n, size_t* tmp_bytes, size_t* total)
+{
+    size_t tmp = 0;
+    uint32_t* none = nullptr;
+    if (int rc = check_hip(rocprim::radix_sort_pairs(nullptr, tmp, none, none, none, none, (size_t)n, 0, 32, nullptr), "radix_sort_pairs(size)")) return rc;
+    *tmp_bytes = tmp;
+    *total = 2 * aligned((size_t)n * 4) + aligned(tmp ? tmp : 4);
+    return MF_OK;
+}
+static int sort_in(uint32_t* cnt, uint32_t* idx, uint32_t n, uint8_t* ws, size_t tmp_bytes, hipStream_t s)
+{
+    uint32_t* cnt_out = reinterpret_cast<uint32_t*>(ws);
+    uint32_t* idx_out = reinterpret_cast<uint32_t*>(ws + aligned((size_t)n * 4));
+    void* tmp = ws + 2 * aligned((size_t)n * 4);
+    if (int rc = check_hip(rocprim::radix_sort_pairs(tmp, tmp_bytes, cnt, cnt_out, idx, idx_out, (size_t)n, 0, 32, s), "mf_sort_by_count: radix_sort_pairs")) return rc;
+    if (int rc = check_hip(hipMemcpyAsync(cnt, cnt_out, (size_t)n * 4, hipMemcpyDeviceToDevice, s), "mf_sort_by_count: copy")) return rc;
+    return check_hip(hipMemcpyAsync(idx, idx_out, (size_t)n * 4, hipMemcpyDeviceToDevice, s), "mf_sort_by_count: copy");
+}
+// The shuffle: 64-bit keys in and out, ids in, permutation out, rocPRIM's temporary storage.
+static int shuffle_layout(uint32_t n, size_t* tmp_bytes, size_t* total)
+{
+    size_t tmp = 0;
+    uint64_t* nk = nullptr; uint32_t* nv = nullptr;
+    if (int rc = check_hip(rocprim::radix_sort_pairs(nullptr, tmp, nk, nk, nv, nv, (size_t)n, 0, 64, nullptr), "radix_sort_pairs(size)")) return rc;
+    *tmp_bytes = tmp;
+    *total = 2 * aligned((size_t)n * 8) + 2 * aligned((size_t)n * 4) + aligned(tmp ? tmp : 4);
+    return MF_OK;
+}
+
 }  // namespace mf
 
 using namespace mf;
 
 extern "C" {
 
+size_t mf_sort_by_count_workspace_bytes(uint32_t n)
+{
+    if (n == 0) return 0;
+    size_t tmp = 0, total = 0;
+    return sort_layout(n, &tmp, &total) == MF_OK ? total : 0;
+}
+int mf_sort_by_count_ws(uint32_t* cnt, uint32_t* idx, uint32_t n, void* workspace, size_t workspace_bytes, void* stream)
+{
+    if (n == 0) return MF_OK;
+    if (!cnt || !idx || !workspace) return invalid("mf_sort_by_count_ws: null pointer");
+    if (reinterpret_cast<uintptr_t>(workspace) % kAlign) return invalid("mf_sort_by_count_ws: the workspace must be 256-byte aligned");
+    size_t tmp = 0, total = 0;
+    if (int rc = sort_layout(n, &tmp, &total)) return rc;
+    if (workspace_bytes < total) return invalid("mf_sort_by_count_ws: the workspace holds %zu bytes, %u counts need %zu (mf_sort_by_count_workspace_bytes)", workspace_bytes, n, total);
+    return sort_in(cnt, idx, n, static_cast<uint8_t*>(workspace), tmp, as_stream(stream));
+}
 int mf_sort_by_count(uint32_t* cnt, uint32_t* idx, uint32_t n, void* stream)
 {
     if (n == 0) return MF_OK;
     if (!cnt || !idx) return invalid("mf_sort_by_count: null pointer");
-    hipStream_t s = as_stream(stream);
+    size_t tmp = 0, total = 0;
+    if (int rc = sort_layout(n, &tmp, &total)) return rc;
     DeviceBuffers b;
-    size_t tmp_bytes = 0;
-    if (int rc = check_hip(hipMalloc(&b.ptr[0], (size_t)n * 4), "mf_sort_by_count: hipMalloc")) return rc;
-    if (int rc = check_hip(hipMalloc(&b.ptr[1], (size_t)n * 4), "mf_sort_by_count: hipMalloc")) return rc;
-    uint32_t* cnt_out = static_cast<uint32_t*>(b.ptr[0]);
-    uint32_t* idx_out = static_cast<uint32_t*>(b.ptr[1]);
-    if (int rc = check_hip(rocprim::radix_sort_pairs(nullptr, tmp_bytes, cnt, cnt_out, idx, idx_out, (size_t)n, 0, 32, s), "mf_sort_by_count: radix_sort_pairs(size)")) return rc;
-    if (int rc = check_hip(hipMalloc(&b.ptr[2], tmp_bytes ? tmp_bytes : 4), "mf_sort_by_count: hipMalloc")) return rc;
-    if (int rc = check_hip(rocprim::radix_sort_pairs(b.ptr[2], tmp_bytes, cnt, cnt_out, idx, idx_out, (size_t)n, 0, 32, s), "mf_sort_by_count: radix_sort_pairs")) return rc;
-    if (int rc = check_hip(hipMemcpyAsync(cnt, cnt_out, (size_t)n * 4, hipMemcpyDeviceToDevice, s), "mf_sort_by_count: copy")) return rc;
-    if (int rc = check_hip(hipMemcpyAsync(idx, idx_out, (size_t)n * 4, hipMemcpyDeviceToDevice, s), "mf_sort_by_count: copy")) return rc;
-    return check_hip(hipStreamSynchronize(s), "mf_sort_by_count: synchronize");
+    if (int rc = check_hip(hipMalloc(&b.ptr[0], total), "mf_sort_by_count: hipMalloc")) return rc;
+    if (int rc = sort_in(cnt, idx, n, static_cast<uint8_t*>(b.ptr[0]), tmp, as_stream(stream))) return rc;
+    return check_hip(hipStreamSynchronize(as_stream(stream)), "mf_sort_by_count: synchronize");      // the workspace is freed on return
 }
-
-int mf_shuffle_ratings(const mf_node* in, mf_node* out, uint32_t n, uint64_t seed, void* stream)
+size_t mf_shuffle_ratings_workspace_bytes(uint32_t n)
+{
+    if (n == 0) return 0;
+    size_t tmp = 0, total = 0;
+    return shuffle_layout(n, &tmp, &total) == MF_OK ? total : 0;
+}
+int mf_shuffle_ratings_ws(const mf_node* in, mf_node* out, uint32_t n, uint64_t seed, void* workspace, size_t workspace_bytes, void* stream)
 {
     if (n == 0) return MF_OK;
     if (!in || !out || in == out) return invalid("mf_shuffle_ratings: null or aliased buffers");
+    if (!workspace || reinterpret_cast<uintptr_t>(workspace) % kAlign) return invalid("mf_shuffle_ratings_ws: the workspace must be non-null and 256-byte aligned");
+    size_t tmp_bytes = 0, total = 0;
+    if (int rc = shuffle_layout(n, &tmp_bytes, &total)) return rc;
+    if (workspace_bytes < total) return invalid("mf_shuffle_ratings_ws: the workspace holds %zu bytes, %u ratings need %zu (mf_shuffle_ratings_workspace_bytes)", workspace_bytes, n, total);
     hipStream_t s = as_stream(stream);
-    DeviceBuffers b;
-    DeviceBuffers b2;
-    if (int rc = check_hip(hipMalloc(&b.ptr[0], (size_t)n * 8), "mf_shuffle_ratings: hipMalloc")) return rc;
-    if (int rc = check_hip(hipMalloc(&b.ptr[1], (size_t)n * 8), "mf_shuffle_ratings: hipMalloc")) return rc;
-    if (int rc = check_hip(hipMalloc(&b.ptr[2], (size_t)n * 4), "mf_shuffle_ratings: hipMalloc")) return rc;
-    if (int rc = check_hip(hipMalloc(&b.ptr[3], (size_t)n * 4), "mf_shuffle_ratings: hipMalloc")) return rc;
-    uint64_t* keys = static_cast<uint64_t*>(b.ptr[0]);
-    uint64_t* keys_out = static_cast<uint64_t*>(b.ptr[1]);
-    uint32_t* idx = static_cast<uint32_t*>(b.ptr[2]);
-    uint32_t* perm = static_cast<uint32_t*>(b.ptr[3]);
+    uint8_t* ws = static_cast<uint8_t*>(workspace);
+    uint64_t* keys = reinterpret_cast<uint64_t*>(ws);
+    uint64_t* keys_out = reinterpret_cast<uint64_t*>(ws + aligned((size_t)n * 8));
+    uint32_t* idx = reinterpret_cast<uint32_t*>(ws + 2 * aligned((size_t)n * 8));
+    uint32_t* perm = reinterpret_cast<uint32_t*>(ws + 2 * aligned((size_t)n * 8) + aligned((size_t)n * 4));
+    void* tmp = ws + 2 * aligned((size_t)n * 8) + 2 * aligned((size_t)n * 4);
     const uint64_t base = mix64(seed ^ 0x53485546464C4521ull);
     uint32_t grid = (n + 255) / 256; if (grid > 8192) grid = 8192;
     hipLaunchKernelGGL(shuffle_keys_kernel, dim3(grid), dim3(256), 0, s, keys, idx, n, base);
     if (int rc = launch_status("mf_shuffle_ratings: keys")) return rc;
-    size_t tmp_bytes = 0;
-    if (int rc = check_hip(rocprim::radix_sort_pairs(nullptr, tmp_bytes, keys, keys_out, idx, perm, (size_t)n, 0, 64, s), "mf_shuffle_ratings: radix_sort_pairs(size)")) return rc;
-    if (int rc = check_hip(hipMalloc(&b2.ptr[0], tmp_bytes ? tmp_bytes : 4), "mf_shuffle_ratings: hipMalloc")) return rc;
-    if (int rc = check_hip(rocprim::radix_sort_pairs(b2.ptr[0], tmp_bytes, keys, keys_out, idx, perm, (size_t)n, 0, 64, s), "mf_shuffle_ratings: radix_sort_pairs")) return rc;
+    if (int rc = check_hip(rocprim::radix_sort_pairs(tmp, tmp_bytes, keys, keys_out, idx, perm, (size_t)n, 0, 64, s), "mf_shuffle_ratings: radix_sort_pairs")) return rc;
     hipLaunchKernelGGL(gather_nodes_kernel, dim3(grid), dim3(256), 0, s, in, out, perm, n);
-    if (int rc = launch_status("mf_shuffle_ratings: gather")) return rc;
-    return check_hip(hipStreamSynchronize(s), "mf_shuffle_ratings: synchronize");
+    return launch_status("mf_shuffle_ratings: gather");
+}
+int mf_shuffle_ratings(const mf_node* in, mf_node* out, uint32_t n, uint64_t seed, void* stream)
+{
+    if (n == 0) return MF_OK;
+    if (!in || !out || in == out) return invalid("mf_shuffle_ratings: null or aliased buffers");
+    size_t tmp = 0, total = 0;
+    if (int rc = shuffle_layout(n, &tmp, &total)) return rc;
+    DeviceBuffers b;
+    if (int rc = check_hip(hipMalloc(&b.ptr[0], total), "mf_shuffle_ratings: hipMalloc")) return rc;
+    if (int rc = mf_shuffle_ratings_ws(in, out, n, seed, b.ptr[0], total, stream)) return rc;
+    return check_hip(hipStreamSynchronize(as_stream(stream)), "mf_shuffle_ratings: synchronize");      // the workspace is freed on return
 }
 
 }  // extern "C"

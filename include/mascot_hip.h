@@ -134,9 +134,17 @@ typedef struct {
 /* The synthetic stand-ins of BASELINE.json's configurations 1..5; MF_EINVAL for any other number. */
 int mf_synth_baseline_config(int config, mf_synth_config* out);
 /* Writes ratings [first, first + count) of the stream to the device array `out` (ids are dense, 0-based).
- * Builds its tables (two CDFs, two permutations, the factors) on every call and frees them before returning, so it
+ * Convenience form: allocates the tables (mf_synth_tables_bytes), builds them, generates and frees them again, so it
  * synchronises the stream. */
 int mf_generate_ratings(const mf_synth_config* cfg, uint64_t seed, uint64_t first, uint64_t count, mf_node* out, void* stream);
+/* The same in two steps with caller-owned device memory: mf_synth_build_tables fills `workspace` (256-byte aligned, at
+ * least mf_synth_tables_bytes(cfg) bytes) with the two CDFs, the two permutations and the factors of (cfg, seed) -- its
+ * host-side tables are copied from pageable memory, so this step waits for the stream once -- and
+ * mf_generate_ratings_ws then writes any range of the stream from those tables: one kernel launch, nothing allocated,
+ * nothing synchronised. */
+size_t mf_synth_tables_bytes(const mf_synth_config* cfg);
+int mf_synth_build_tables(const mf_synth_config* cfg, uint64_t seed, void* workspace, size_t workspace_bytes, void* stream);
+int mf_generate_ratings_ws(const mf_synth_config* cfg, uint64_t seed, const void* tables, uint64_t first, uint64_t count, mf_node* out, void* stream);
 /* The same into a host array (allocates, generates on the default stream, copies back, frees). */
 int mf_generate_ratings_host(const mf_synth_config* cfg, uint64_t seed, uint64_t first, uint64_t count, mf_node* host_out);
 /* Measurement aid, no counterpart in the reference: the memory traffic of one epoch of updates without the
@@ -309,14 +317,24 @@ int mf_init_idx_arr(uint32_t* arr, uint32_t n, void* stream);
 /* user_item_histogram, preprocess_utils.h:13-19 (caller zeroes the bins). */
 int mf_user_item_histogram(const mf_node* R, uint32_t n, uint32_t* user_bin, uint32_t* item_bin, void* stream);
 /* thrust::sort_by_key(cnt, idx), preprocess_utils.h:87-88: ascending stable sort of the counts carrying
- * the ids, in place.  Allocates its temporary storage with hipMalloc and synchronises the stream. */
+ * the ids, in place.  Convenience form: allocates its workspace with hipMalloc, frees it and therefore
+ * synchronises the stream. */
 int mf_sort_by_count(uint32_t* cnt, uint32_t* idx, uint32_t n, void* stream);
+/* The same with a caller-owned workspace (256-byte aligned device memory of at least
+ * mf_sort_by_count_workspace_bytes(n) bytes: the sort's output buffers and rocPRIM's temporary storage): asynchronous
+ * on `stream`, allocates nothing, synchronises nothing.  The size query needs a current device (0 on failure). */
+size_t mf_sort_by_count_workspace_bytes(uint32_t n);
+int mf_sort_by_count_ws(uint32_t* cnt, uint32_t* idx, uint32_t n, void* workspace, size_t workspace_bytes, void* stream);
 /* matrix_reconst_gpu_triplet, preprocess_utils.h:28-36 (in place). */
 int mf_matrix_reconst_triplet(mf_node* R, const uint32_t* user2sorted_idx, const uint32_t* item2sorted_idx,
                               uint32_t n, void* stream);
 /* Seeded replacement for srand(time(0)); std::random_shuffle(R, R+n) (mf_methods.cu:38-39): out = in
- * permuted by ascending 64-bit key(seed, i).  Allocates temporaries with hipMalloc, synchronises. */
+ * permuted by ascending 64-bit key(seed, i).  Convenience form: allocates its workspace, frees it, synchronises. */
 int mf_shuffle_ratings(const mf_node* in, mf_node* out, uint32_t n, uint64_t seed, void* stream);
+/* The same with a caller-owned workspace (256-byte aligned, mf_shuffle_ratings_workspace_bytes(n) bytes: keys, ids,
+ * the permutation and rocPRIM's temporary storage): asynchronous, allocates nothing, synchronises nothing. */
+size_t mf_shuffle_ratings_workspace_bytes(uint32_t n);
+int mf_shuffle_ratings_ws(const mf_node* in, mf_node* out, uint32_t n, uint64_t seed, void* workspace, size_t workspace_bytes, void* stream);
 
 /* ---- host training drivers (the reference's mf_methods.h:4-11 surface) -------------------
  * These take HOST pointers, allocate and free their own device memory with hipMalloc, run on

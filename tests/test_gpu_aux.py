@@ -294,3 +294,63 @@ def test_generated_ratings_match_the_checker(orc, config):
     host = np.empty(500, mfutil.NODE)
     h.mf_generate_ratings_host(C.addressof(c), 11, 10, 500, host.ctypes.data)
     assert np.array_equal(host.view(np.uint8), want[10:510].view(np.uint8))
+
+
+def test_workspace_forms_equal_the_allocating_forms(orc):
+    """mf_sort_by_count_ws, mf_shuffle_ratings_ws and mf_generate_ratings_ws with caller-owned workspaces of exactly the
+    size their queries return give what the forms that allocate for themselves give; a workspace that is too small or
+    misaligned is refused before anything is launched."""
+    import ctypes as C
+    import torch
+    from importlib import import_module
+    MfError = import_module("icdm-2021_mascot_amd.capi").MfError
+    h = mfutil.hip()
+    st = mfutil.stream_ptr()
+    rng = np.random.default_rng(5)
+    for n in (1, 777, 300_001):
+        cnt = rng.integers(0, 50, n).astype(np.uint32)
+        a_cnt, b_cnt = to_dev(cnt), to_dev(cnt)
+        a_idx, b_idx = torch.arange(n, dtype=torch.int32, device="cuda"), torch.arange(n, dtype=torch.int32, device="cuda")
+        h.mf_sort_by_count(a_cnt.data_ptr(), a_idx.data_ptr(), n, st)
+        need = h.mf_sort_by_count_workspace_bytes(n)
+        assert need >= 8 * n
+        ws = torch.full((need,), 0x5A, dtype=torch.uint8, device="cuda")
+        h.mf_sort_by_count_ws(b_cnt.data_ptr(), b_idx.data_ptr(), n, ws.data_ptr(), need, st)
+        torch.cuda.synchronize()
+        assert torch.equal(a_cnt, b_cnt) and torch.equal(a_idx, b_idx)
+        order = np.argsort(cnt, kind="stable")
+        assert np.array_equal(from_dev(b_idx, np.uint32), order.astype(np.uint32))
+        with pytest.raises(MfError, match="need"):
+            h.mf_sort_by_count_ws(b_cnt.data_ptr(), b_idx.data_ptr(), n, ws.data_ptr(), need - 1, st)
+        if need > 512:
+            with pytest.raises(MfError, match="256-byte aligned"):
+                h.mf_sort_by_count_ws(b_cnt.data_ptr(), b_idx.data_ptr(), n, ws.data_ptr() + 4, need - 256, st)
+        # shuffle
+        R = np.zeros(n, mfutil.NODE)
+        R["u"], R["i"], R["r"] = np.arange(n), rng.integers(0, 1000, n), rng.integers(1, 6, n)
+        dR = to_dev(R)
+        o1, o2 = torch.empty_like(dR), torch.empty_like(dR)
+        h.mf_shuffle_ratings(dR.data_ptr(), o1.data_ptr(), n, 42, st)
+        need = h.mf_shuffle_ratings_workspace_bytes(n)
+        ws = torch.full((need,), 0xA5, dtype=torch.uint8, device="cuda")
+        h.mf_shuffle_ratings_ws(dR.data_ptr(), o2.data_ptr(), n, 42, ws.data_ptr(), need, st)
+        torch.cuda.synchronize()
+        assert torch.equal(o1, o2)
+        assert np.array_equal(from_dev(o2, mfutil.NODE).view(np.uint8), orc.shuffle(42, R).view(np.uint8))
+        with pytest.raises(MfError, match="need"):
+            h.mf_shuffle_ratings_ws(dR.data_ptr(), o2.data_ptr(), n, 42, ws.data_ptr(), need - 1, st)
+    # generator: tables once, any range afterwards without allocation or synchronisation
+    for config in (1, 5):
+        c = h.synth_config(config)
+        c.n_users, c.n_items = 3000, 700
+        need = h.mf_synth_tables_bytes(C.addressof(c))
+        assert need >= 12 * 3700
+        tables = torch.full((need,), 0x33, dtype=torch.uint8, device="cuda")
+        h.mf_synth_build_tables(C.addressof(c), 9, tables.data_ptr(), need, st)
+        want = orc.generate_ratings(c, 9, 0, 50_000)
+        for first, count in ((0, 50_000), (12_345, 1_000), (49_999, 1)):
+            out = torch.empty(count * 12, dtype=torch.uint8, device="cuda")
+            h.mf_generate_ratings_ws(C.addressof(c), 9, tables.data_ptr(), first, count, out.data_ptr(), st)
+            assert np.array_equal(from_dev(out, mfutil.NODE).view(np.uint8), want[first:first + count].view(np.uint8))
+        with pytest.raises(MfError, match="need"):
+            h.mf_synth_build_tables(C.addressof(c), 9, tables.data_ptr(), need - 1, st)

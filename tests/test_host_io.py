@@ -84,6 +84,66 @@ def test_readers_and_model_files(driver, tmp_path, k):
     assert [l for l in lines if l.startswith("reread ")][0] == "reread users 3 items 3 k %d p %d q %d" % (k, 3 * k, 3 * k)
 
 
+def _dump(driver, train, test, out):
+    r = subprocess.run([driver, str(train), str(test), out, "4"], capture_output=True, text=True)
+    assert r.returncode == 0, r.stdout + r.stderr
+    lines = r.stdout.splitlines()
+    users = {int(l.split()[1]): int(l.split()[3]) for l in lines if l.startswith("user ")}
+    items = {int(l.split()[1]): int(l.split()[3]) for l in lines if l.startswith("item ")}
+    # ratings are printed with nine significant digits, which identify a binary32 value
+    got_train = [(int(a), int(b), float(np.float32(c))) for a, b, c in (l.split()[1:] for l in lines if l.startswith("train "))]
+    got_test = [(int(a), int(b), float(np.float32(c))) for a, b, c in (l.split()[1:] for l in lines if l.startswith("test "))]
+    summary = [l for l in lines if l.startswith("users ")][0].split()
+    return users, items, got_train, got_test, dict(zip(summary[0::2], summary[1::2]))
+
+
+@pytest.mark.parametrize("dirname", ["netflix_prize", "ml-25M", "plain"])
+def test_item_first_column_order_by_path(driver, tmp_path, dirname):
+    """io_utils.h:40-47: a path that contains "netflix" or "25M" holds the item in the first column and the user in the
+    second; any other path user first.  The same lines therefore load transposed."""
+    d = tmp_path / dirname
+    d.mkdir()
+    train, test = d / "train.tsv", d / "test.tsv"
+    lines = [(11, 500, 4.0), (12, 500, 3.0), (11, 600, 1.5), (13, 700, 5.0)]
+    train.write_text("".join("%d\t%d\t%g\n" % t for t in lines))
+    test.write_text("11\t700\t2.5\n13\t500\t1.0\n99\t500\t3.0\n")
+    users, items, got_train, got_test, summary = _dump(driver, train, test, str(tmp_path / ("m_" + dirname)))
+    swapped = dirname != "plain"
+    first, second = [a for a, _, _ in lines], [b for _, b, _ in lines]
+    want_users = list(dict.fromkeys(second if swapped else first))          # first-seen order of the user column
+    want_items = list(dict.fromkeys(first if swapped else second))
+    assert [users[i] for i in range(len(users))] == want_users
+    assert [items[i] for i in range(len(items))] == want_items
+    u2d, i2d = {v: i for i, v in enumerate(want_users)}, {v: i for i, v in enumerate(want_items)}
+    assert got_train == [((u2d[b], i2d[a], r) if swapped else (u2d[a], i2d[b], r)) for a, b, r in lines]
+    if swapped:      # test lines are (item, user, rating): item 11 user 700, item 13 user 500; item 99 never occurred
+        assert got_test == sorted([(u2d[700], i2d[11], 2.5), (u2d[500], i2d[13], 1.0)])
+        assert (d / "remove_item.txt").read_text().split() == ["99"] and (d / "remove_user.txt").read_text().split() == []
+    else:
+        assert got_test == sorted([(u2d[11], i2d[700], 2.5), (u2d[13], i2d[500], 1.0)])
+        assert (d / "remove_user.txt").read_text().split() == ["99"]
+    assert summary["missing"] == "1"
+
+
+def test_yahoo_block_format(driver, tmp_path):
+    """io_utils.h:49-79,139-181: a path that contains "Yahoo" holds blocks "user|count" followed by count lines
+    "item<TAB>rating" with ratings 0..100, which are mapped to rating / 25 + 1; ids are numbered in first-seen order;
+    in the test file a rating of an unknown item is dropped and counted, a block of an unknown user is counted whole."""
+    d = tmp_path / "YahooMusic"
+    d.mkdir()
+    train, test = d / "train.txt", d / "test.txt"
+    train.write_text("7|3\n100\t90\n200\t0\n300\t50\n5|1\n200\t100\n9|2\n300\t25\n400\t75\n")
+    test.write_text("5|2\n100\t80\n999\t10\n8|2\n100\t1\n200\t2\n9|1\n100\t30\n")
+    users, items, got_train, got_test, summary = _dump(driver, train, test, str(tmp_path / "m"))
+    assert [users[i] for i in range(3)] == [7, 5, 9] and [items[i] for i in range(4)] == [100, 200, 300, 400]
+    f = lambda r: float(np.float32(np.float32(r) / np.float32(25.0)) + np.float32(1.0))
+    assert got_train == [(0, 0, f(90)), (0, 1, f(0)), (0, 2, f(50)), (1, 1, f(100)), (2, 2, f(25)), (2, 3, f(75))]
+    assert f(0) == 1.0 and f(100) == 5.0 and f(90) == 4.599999904632568
+    # user 5: item 100 kept, item 999 unknown (1 missing); user 8 unknown: its 2 ratings missing, and the block after it parses
+    assert got_test == [(1, 0, f(80)), (2, 0, f(30))]
+    assert summary["missing"] == "3" and summary["test"] == "2"
+
+
 def test_many_rows_are_written_in_order(driver, tmp_path):
     """More rows than one formatting block per thread: the blocks must land in the file in row order."""
     n_users, n_items, k = 70_001, 3, 2
