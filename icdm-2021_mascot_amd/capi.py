@@ -63,6 +63,8 @@ SIGNATURES = {
     "mf_replicate_threshold": (f32, [f32, f32]),
     "mf_sort_by_count_workspace_bytes": (C.c_size_t, [u32]),
     "mf_sort_by_count_ws": (i32, [vp, vp, u32, vp, C.c_size_t, vp]),
+    "mf_sort_by_count_static_max": (u32, []),
+    "mf_sort_by_count_static": (i32, [vp, vp, u32, vp]),
     "mf_shuffle_ratings_workspace_bytes": (C.c_size_t, [u32]),
     "mf_shuffle_ratings_ws": (i32, [vp, vp, u32, u64, vp, C.c_size_t, vp]),
     "mf_synth_tables_bytes": (C.c_size_t, [vp]),

@@ -4,6 +4,7 @@
 #include "mf_host.h"
 #include "mf_device.h"
 #include <cstring>
+#include <mutex>
 #include <rocprim/device/device_radix_sort.hpp>
 
 namespace mf {
@@ -63,6 +64,35 @@ static int shuffle_layout(uint32_t n, size_t* tmp_bytes, size_t* total)
     return MF_OK;
 }
 
+// ---- scratch of mf_sort_by_count_static ------------------------------------------------------------------------
+// Device memory that belongs to the library image: every GPU the library runs on holds its own copy from the moment
+// the code object is loaded until the process ends.  20 MiB: the two output buffers of a sort of kStaticSortMax
+// counts (8 MiB) and rocPRIM's temporary storage for that size (8.4 MB on gfx950 with rocPRIM 4: its own pair of
+// buffers and its counters).
+constexpr uint32_t kStaticSortMax = 1u << 20;
+constexpr size_t kStaticScratchBytes = 20u << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+// The array's name is a host-side stand-in, not a device address: the address of each device's copy is asked for once,
+// with that device current, and everything below uses that pointer.
+constexpr int kMaxDevices = 64;
+static std::mutex g_scratch_mutex;
+static void* g_scratch_ptr[kMaxDevices] = {};
+static int static_scratch(void** out)
+{
+    int dev = 0;
+    if (int rc = check_hip(hipGetDevice(&dev), "mf_sort_by_count_static: hipGetDevice")) return rc;
+    if (dev < 0 || dev >= kMaxDevices) return invalid("mf_sort_by_count_static: device %d is beyond the %d devices this library keeps scratch addresses for", dev, kMaxDevices);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* ptr = nullptr;
+        if (int rc = check_hip(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)), "mf_sort_by_count_static: hipGetSymbolAddress(scratch)")) return rc;
+        if (!ptr) return invalid("mf_sort_by_count_static: the scratch array has no address on device %d", dev);
+        g_scratch_ptr[dev] = ptr;
+    }
+    *out = g_scratch_ptr[dev];
+    return MF_OK;
+}
+
 }  // namespace mf
 
 using namespace mf;
@@ -96,6 +126,22 @@ int mf_sort_by_count(uint32_t* cnt, uint32_t* idx, uint32_t n, void* stream)
     if (int rc = sort_in(cnt, idx, n, static_cast<uint8_t*>(b.ptr[0]), tmp, as_stream(stream))) return rc;
     return check_hip(hipStreamSynchronize(as_stream(stream)), "mf_sort_by_count: synchronize");      // the workspace is freed on return
 }
+uint32_t mf_sort_by_count_static_max(void) { return kStaticSortMax; }
+int mf_sort_by_count_static(uint32_t* cnt, uint32_t* idx, uint32_t n, void* stream)
+{
+    if (n == 0) return MF_OK;
+    if (!cnt || !idx) return invalid("mf_sort_by_count_static: null pointer");
+    if (n > kStaticSortMax) return invalid("mf_sort_by_count_static: %u counts, the library's own scratch holds at most %u (use mf_sort_by_count_ws with a workspace)", n, kStaticSortMax);
+    size_t tmp = 0, total = 0;
+    if (int rc = sort_layout(n, &tmp, &total)) return rc;
+    if (total > kStaticScratchBytes) return invalid("mf_sort_by_count_static: %u counts need %zu bytes of scratch, the library's own holds %zu", n, total, kStaticScratchBytes);
+    void* ptr = nullptr;
+    if (int rc = static_scratch(&ptr)) return rc;
+    // nothing in the scratch has to start at zero: the sort writes its output buffers before it reads them and rocPRIM
+    // initialises what it keeps in its temporary storage
+    return sort_in(cnt, idx, n, static_cast<uint8_t*>(ptr), tmp, as_stream(stream));
+}
+
 size_t mf_shuffle_ratings_workspace_bytes(uint32_t n)
 {
     if (n == 0) return 0;

@@ -325,6 +325,15 @@ int mf_sort_by_count(uint32_t* cnt, uint32_t* idx, uint32_t n, void* stream);
  * on `stream`, allocates nothing, synchronises nothing.  The size query needs a current device (0 on failure). */
 size_t mf_sort_by_count_workspace_bytes(uint32_t n);
 int mf_sort_by_count_ws(uint32_t* cnt, uint32_t* idx, uint32_t n, void* workspace, size_t workspace_bytes, void* stream);
+/* mf_sort_by_count for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc); no counterpart in the reference.  The sort's workspace is a 20 MiB array in the
+ * library's own device image (each GPU the library runs on holds its copy until the process ends), so the call
+ * allocates and frees nothing and is asynchronous on `stream`.  At most mf_sort_by_count_static_max() = 1,048,576
+ * counts; more are refused with MF_EINVAL.  All calls on one GPU share that array: calls that overlap on one GPU
+ * (different streams, different host threads) race -- run them one after another.  Nothing in the array has to
+ * start at zero between calls. */
+uint32_t mf_sort_by_count_static_max(void);
+int mf_sort_by_count_static(uint32_t* cnt, uint32_t* idx, uint32_t n, void* stream);
 /* matrix_reconst_gpu_triplet, preprocess_utils.h:28-36 (in place). */
 int mf_matrix_reconst_triplet(mf_node* R, const uint32_t* user2sorted_idx, const uint32_t* item2sorted_idx,
                               uint32_t n, void* stream);

@@ -1,0 +1,40 @@
+"""mf_sort_by_count_static, the count sort that allocates nothing (its workspace is an array in the library's own device
+image), against mf_sort_by_count through the C ABI: bit for bit, on two calls in a row, the second with a smaller input,
+so that what the first call left in the shared scratch cannot leak into the second."""
+import numpy as np
+import pytest
+
+import mfutil
+
+pytestmark = pytest.mark.gpu
+
+
+def _sorted_by(h, entry, cnt):
+    import torch
+    n = cnt.size
+    d_cnt = mfutil.to_dev(cnt)
+    d_idx = torch.arange(n, dtype=torch.int32, device="cuda")
+    entry(d_cnt.data_ptr(), d_idx.data_ptr(), n, mfutil.stream_ptr())
+    torch.cuda.synchronize()
+    return mfutil.from_dev(d_cnt, np.uint32), mfutil.from_dev(d_idx, np.uint32)
+
+
+def test_static_scratch_sort_equals_the_allocating_sort():
+    from importlib import import_module
+    MfError = import_module("icdm-2021_mascot_amd.capi").MfError
+    h = mfutil.hip()
+    rng = np.random.default_rng(2024)
+    limit = h.mf_sort_by_count_static_max()
+    assert limit == 1 << 20
+    # the largest size it takes (Zipf-like counts with many ties), then smaller ones, then a larger one again
+    for n in (limit, 480_000, 17_800, 1, 1_000_000):
+        cnt = (rng.zipf(1.3, n) % 100_000).astype(np.uint32)
+        want_cnt, want_idx = _sorted_by(h, h.mf_sort_by_count, cnt)
+        got_cnt, got_idx = _sorted_by(h, h.mf_sort_by_count_static, cnt)
+        assert np.array_equal(got_cnt, want_cnt) and np.array_equal(got_idx, want_idx), n
+        assert np.array_equal(got_idx, np.argsort(cnt, kind="stable").astype(np.uint32))        # ascending, stable
+    with pytest.raises(MfError, match="at most 1048576"):
+        import torch
+        big = torch.zeros(limit + 1, dtype=torch.int32, device="cuda")
+        h.mf_sort_by_count_static(big.data_ptr(), big.data_ptr(), limit + 1, mfutil.stream_ptr())
+    h.mf_sort_by_count_static(None, None, 0, mfutil.stream_ptr())           # nothing to do
