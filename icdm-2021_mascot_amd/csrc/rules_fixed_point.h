@@ -35,16 +35,17 @@ __device__ __forceinline__ int f2i_sat(float f)
 }
 // The hardware's own float-to-integer conversions truncate, saturate and map NaN to 0, which is what CUDA's casts do;
 // spelled as instructions because an out-of-range cast has no defined value in C++.
-// The compiler's hazard bookkeeping does not look inside an asm statement, so each one is self-contained: its input
-// comes from an ordinary VALU instruction (an add, a minimum), its result goes to one, and the one wait state a
-// transcendental's result needs before another VALU instruction reads it is spelled out.
-__device__ __forceinline__ int hw_cvt_i32(float f) { int r; asm("v_cvt_i32_f32_e32 %0, %1" : "=v"(r) : "v"(f)); return r; }
+// The compiler's hazard bookkeeping does not look inside an asm statement, so each one is self-contained whatever
+// produced its input: it starts with the wait state a transcendental's result needs before a VALU instruction may read
+// it (s_nop is not a VALU instruction: the other wavefronts of the SIMD issue meanwhile), and a transcendental inside
+// is followed by one before its result is read.  Results leave through an ordinary (non-transcendental) conversion.
+__device__ __forceinline__ int hw_cvt_i32(float f) { int r; asm("s_nop 0\n\tv_cvt_i32_f32_e32 %0, %1" : "=v"(r) : "v"(f)); return r; }
 // (unsigned)floorf(log2f(x)) for x that is not subnormal: the conversion truncates, and negative logarithms and NaN
 // give 0 with or without the floor
 __device__ __forceinline__ uint32_t floor_log2_u32(float x)
 {
     uint32_t r;
-    asm("v_log_f32_e32 %0, %1\n\ts_nop 0\n\tv_cvt_u32_f32_e32 %0, %0" : "=v"(r) : "v"(x));
+    asm("s_nop 0\n\tv_log_f32_e32 %0, %1\n\ts_nop 0\n\tv_cvt_u32_f32_e32 %0, %0" : "=v"(r) : "v"(x));
     return r;
 }
 // (signed char) of roundf(x), saturating, NaN -> 0: the conversion truncates by itself, so round_half_away's own
@@ -116,7 +117,16 @@ __device__ __forceinline__ float max4_by_rows(float a, float b, float c, float d
 // get_only_scaling_factor (muppet_sgd_kernel.h:7-18) for two value ranges at once.  `extreme` holds, by half-wave, the
 // largest value (lower) and the negated smallest value (upper) of a range, the same in both rows of a half-wave or a
 // different range in each; the result is the scale index of the lane's range.
-__device__ __forceinline__ uint32_t muppet_scale_index_by_rows(unsigned bitwidth, float extreme, bool upper)
+//
+// The reference evaluates (unsigned)floorf(log2f(fminf(|max_val / max|, |min_val / min|))).  floor and log2 are
+// monotonic, so that is the smaller of the two sides' floor(log2(bound / |x|)), and each of those follows from the
+// bits of x: with bound = t * 2^eb and |x| = m * 2^e (1 <= t, m < 2) it is eb - e when m <= t and eb - e - 1
+// otherwise.  The quotient overflows to infinity exactly when that index reaches 128 (index 2^32 - 1 after the
+// unsigned conversion, as for x = 0), an infinite or NaN x gives 0, a negative index 0.  Only within a few ulps of
+// m = t can the rounding of the division and of the logarithm decide differently (the result of log2f next to an
+// integer n rounds to n within about 2^(log2 n - 24) of it: up to 45 ulps of m for indices below 128); those lanes
+// take the division and the logarithm, as before (muppet_scale_index_slow).
+__device__ __forceinline__ uint32_t muppet_scale_index_slow(unsigned bitwidth, float extreme, bool upper)
 {
     const float val = (float)(1 << (bitwidth - 1));
     const float bound = upper ? (-val) - 0.5f : (val - 1) + 0.5f;
@@ -126,6 +136,23 @@ __device__ __forceinline__ uint32_t muppet_scale_index_by_rows(unsigned bitwidth
     // x is never subnormal (|bound| >= 127.5 over a finite extreme), so the bare v_log_f32 equals log2f
     const uint32_t idx = floor_log2_u32(range_best);
     return both_zero ? 0u : idx;
+}
+struct OpUMin { __device__ __forceinline__ uint32_t operator()(uint32_t a, uint32_t b) const { return a < b ? a : b; } };
+__device__ __forceinline__ uint32_t muppet_scale_index_by_rows(unsigned bitwidth, float extreme, bool upper)
+{
+    // bound = 2^(b-1) - 0.5 = (2 - 2^-(b-1)) * 2^(b-2) for the maximum, 2^(b-1) + 0.5 = (1 + 2^-b) * 2^(b-1) for the minimum
+    const uint32_t eb = upper ? bitwidth - 1u : bitwidth - 2u;
+    const uint32_t t_mant = upper ? (0x800000u >> bitwidth) : 0x800000u - (0x800000u >> (bitwidth - 1u));
+    const uint32_t xb = bits(extreme) & 0x7fffffffu;
+    const uint32_t mant = xb & 0x7fffffu;
+    const int idx = (int)(eb + 127u) - (int)(xb >> 23) - (mant > t_mant ? 1 : 0);
+    const bool near = mant - t_mant + 64u <= 128u;                                      // |mant - t_mant| <= 64
+    if (__builtin_amdgcn_ballot_w64(near) != 0ull) return muppet_scale_index_slow(bitwidth, extreme, upper);
+    // 2^32 - 1 marks x = 0, 2^32 - 2 an overflowing quotient: the smaller of the two sides plus one when it is a mark
+    // gives 0 for two zeros (the reference's special case) and 2^32 - 1 when the finite side overflows as well
+    const uint32_t side = xb == 0u ? 0xffffffffu : (idx < 0 ? 0u : (idx >= 128 ? 0xfffffffeu : (uint32_t)idx));
+    const uint32_t both = step_xor32(side, OpUMin());
+    return both + (both >= 0xfffffffeu ? 1u : 0u);
 }
 
 template <int K, bool COH> struct MuppetRule : DenseBase<K, COH> {

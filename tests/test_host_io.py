@@ -170,6 +170,16 @@ def test_round_half_away_identity_is_exhaustive(tmp_path):
     assert r.returncode == 0 and r.stdout.strip() == "0", r.stdout + r.stderr
 
 
+def test_scale_index_from_bits_equals_its_definition(tmp_path):
+    """The MuPPET kernels take floor(log2(bound / x)) from the exponent and mantissa of x; the reference divides and calls
+    log2f (muppet/muppet_sgd_kernel.h:7-18).  Outside 64 ulps around the threshold mantissa (where the kernels evaluate the
+    definition) the two agree for every exponent, both signs, zeros, subnormals, infinities and NaN, at every bit width."""
+    exe = str(tmp_path / "scale_index_identity_check")
+    subprocess.run(["gcc", "-O2", "-ffp-contract=off", "-o", exe, os.path.join(ROOT, "tests", "scale_index_identity_check.c"), "-lm"], check=True)
+    r = subprocess.run([exe], capture_output=True, text=True, timeout=600)
+    assert r.returncode == 0 and r.stdout.strip() == "0", r.stdout + r.stderr
+
+
 def test_bench_refuses_more_than_one_gpu():
     """bench.py measures one GPU; asked for more it says so and exits without touching a device."""
     import subprocess
