@@ -29,6 +29,11 @@ TRAIN = dict(epochs=50, lr=0.01, decay=0.1, lam=0.015, sample_ratio=0.05, interv
 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of a plain epoch's update kernels (KiB per epoch, scaled by the factors a 1 GiB
 # device copy gives), recorded in the profile named here; reported only for the workload they were taken on
 PROFILED_TRAFFIC = {
+    # (config, training ratings, k, seed, workers): bytes per epoch (four launches of the update kernel)
+    (4, 100_000_000, 128, 2021, 6104): dict(
+        bytes=(2 * 14_908_600 + 29_211_562) * 1024,
+        source="rocprofv3 --pmc FETCH_SIZE (x2.0) and WRITE_SIZE (x1.0) of the four update launches of epoch 2, recorded in "
+               "profiles/hogwild_mascot_k128_config4_hbm_traffic.md; not re-measured by this run"),
 }
 
 
@@ -215,6 +220,7 @@ def main():
     bytes_per_update = 12 + 2 * k * (2 + 2)
     gbs = updates * bytes_per_update / (ms / 1e3) / 1e9
     epochs_done_timed = a.warmup + a.steps
+    launches = int(prm.replica_merges) if (rep_u or rep_v) and prm.replica_merges else 1
     plain = [m for i, m in enumerate(main_run["timed"]) if not is_check_epoch(a.warmup + i)] or list(main_run["timed"])
     out = {
         "metric": "SGD ratings/sec/epoch & % HBM roofline at k=128 on 1 MI355X; test RMSE delta",
@@ -236,9 +242,11 @@ def main():
                              "bounded by the HBM peak only for traffic that misses",
                      "traffic": None,
                      "kernel": "hogwild_kernel<MascotRuleT<%d,true,false>,true>" % k,
-                     "bytes_per_update": bytes_per_update, "updates_per_launch": updates,
-                     "launches_per_step": "the driver's update call: the epoch cut into replica_merges kernel launches, replica averaging "
-                                          "after each; check epochs add the sampled launch"},
+                     "bytes_per_update": bytes_per_update, "updates_per_step": updates,
+                     "kernel_launches_per_step": launches,
+                     "per": "step: achieved, traffic and updates are those of one epoch = the driver's update call, which cuts the epoch into "
+                            "kernel_launches_per_step launches of this kernel with the replica averaging between them; the time is the driver's "
+                            "hipEvent time around that call on its stream (check epochs add the sampled launch)"},
         "ms_steps": [round(float(x), 3) for x in timed],
         "epoch_wall_ms": main_run["wall_s"] * 1e3 / a.steps,
         "plain_epoch_ms": float(np.mean(plain)),

@@ -119,7 +119,8 @@ int report_epoch(Common& c, uint32_t e, double rmse, float sgd_ms)
     if (c.prm->verbose) { std::printf("%u %g %g\n", e + 1, (double)c.lr[e], rmse); std::fflush(stdout); }   // mf_methods.cu:396
     if (c.test_n && !std::isfinite(rmse))
         return invalid("mf_train: the model diverged in epoch %u (the test RMSE is not finite); lower the learning rate, or the "
-                       "hot-row caps (hot_row_inflight_early, hot_row_inflight) if hot rows are on", e + 1);
+                       "number of updates in flight up to which a popular row is added to (replicate_inflight; the thinning caps "
+                       "hot_row_inflight_early and hot_row_inflight if thinning is on)", e + 1);
     return 0;
 }
 

@@ -30,6 +30,18 @@
  *     rounds every operation.  parity unpinned for that choice (the update is
  *     pinned as a gradient step within binary32 rounding, the summation order
  *     by a crafted row).
+ *   - orc_mascot_epoch, sampled epochs: the order in which the per-group
+ *     squared norms and gradient sums of racing warps are added
+ *     (mascot/mascot_sgd_kernel.h:259-276: atomics and an unsynchronised +=)
+ *     is not fixed by the reference; this restatement adds them in rating
+ *     order.  parity unpinned for that order (any order agrees to 1e-5
+ *     relative, which is what the tests hold the GPU's sums to).
+ *
+ * Pinned by tests/test_oracle_pins.py with engines that share no code with this
+ * file (numpy.float16, Python integers, math.frexp) and hand-worked rows:
+ * orc_mpt_update, orc_muppet_update and its scale index, orc_afp_* (scale,
+ * QEM / QEM_BP, QPA, the re-measurement schedule) and the MuPPET ladder
+ * (orc_muppet_ladder_step).
  */
 #ifndef MASCOT_ORACLE_H
 #define MASCOT_ORACLE_H
