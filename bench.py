@@ -170,6 +170,7 @@ def main():
     ap.add_argument("--skip-full-run", action="store_true", help="stop after the timed epochs instead of running on to epoch 50")
     ap.add_argument("--reference-semantics", action="store_true", help="also time two epochs without hot rows (-hot 0: every row stored, last writer wins)")
     ap.add_argument("--every-rule", action="store_true", help="also run MPT, MuPPET, AFP and binary16 storage (-v 4, 3, 2, 7) for eight epochs each")
+    ap.add_argument("--rules", default="mpt,muppet,afp,mem_quant", help="the rules --every-rule runs")
     ap.add_argument("--pmc-copy", action="store_true", help="profiling aid: also run three 1 GiB device copies, the known-size kernel that FETCH_SIZE / WRITE_SIZE are scaled by")
     ap.add_argument("--only-timed", action="store_true", help="profiling aid: the MASCOT warm-up and timed epochs only")
     a = ap.parse_args()
@@ -313,6 +314,8 @@ def main():
     if a.every_rule:
         out["every_rule"] = {}
         for name, version, half in (("mpt", 4, True), ("muppet", 3, False), ("afp", 2, False), ("mem_quant", 7, True)):
+            if name not in a.rules.split(","):
+                continue
             out["every_rule"][name] = side_leg(version, 2, 6, "mf_train -v %d, epochs 2..7" % version, half)
     if not a.skip_cpu:
         threads = min(os.cpu_count() or 1, 16)

@@ -56,8 +56,21 @@ __device__ __forceinline__ int round_to_i8(float x)
     const int v = hw_cvt_i32(x + __builtin_copysignf(0x1.fffffep-2f, x));
     return v < -128 ? -128 : (v > 127 ? 127 : v);
 }
+// (signed char) of roundf(x * s) for a scale s = 2^n, n >= 0: the product by a power of two is exact (or infinite), so
+// the fused multiply-add rounds exactly as the product followed by the addition does, and the sign of the product is
+// the sign of x (0 * inf and NaN give NaN -> 0 either way); the sign constant is shared by every quantisation of x.
+__device__ __forceinline__ int round_to_i8_scaled(float x, float s)
+{
+    const int v = hw_cvt_i32(__builtin_fmaf(x, s, __builtin_copysignf(0x1.fffffep-2f, x)));
+    return v < -128 ? -128 : (v > 127 ? 127 : v);
+}
+// roundf(x * s) for s = 2^n, n >= 0, likewise
+__device__ __forceinline__ float round_half_away_scaled(float x, float s) { return __builtin_truncf(__builtin_fmaf(x, s, __builtin_copysignf(0x1.fffffep-2f, x))); }
 // 2^n for an integer-valued exponent, exact (exp2f of an integer in the reference).
 __device__ __forceinline__ float pow2u(uint32_t n) { return __builtin_ldexpf(1.0f, n > 1000u ? 1000 : (int)n); }
+// The same from integer arithmetic on the exponent field (infinity from n = 128 on): for a wave-uniform n these are
+// scalar instructions, where ldexp is a vector one.
+__device__ __forceinline__ float pow2u_bits(uint32_t n) { return from_bits<float>(((n > 128u ? 128u : n) + 127u) << 23); }
 __device__ __forceinline__ float pow2i(int n) { return __builtin_ldexpf(1.0f, n > 1000 ? 1000 : (n < -1000 ? -1000 : n)); }
 
 // Mirror: v[j] = element (L mod 32) + 32 j of the row, own[] = which of them this lane stores.
@@ -89,7 +102,7 @@ __device__ __forceinline__ uint32_t muppet_scale_index(unsigned bitwidth, float 
     float range_best = fminf(fabsf(max_val / max_v), fabsf(min_val / min_v));
     return f2u_sat(floorf(__builtin_log2f(range_best)));
 }
-__device__ __forceinline__ half_t grid_h(float v, float s, float s_rev) { return (half_t)(round_half_away(v * s) * s_rev); }
+__device__ __forceinline__ half_t grid_h(float v, float s, float s_rev) { return (half_t)(round_half_away_scaled(v, s) * s_rev); }
 // 1 / 2^n as the reference's division yields it: 2^n is infinite from n = 128 on, and 1 / inf = 0
 __device__ __forceinline__ float pow2_reciprocal(uint32_t n) { return n > 127u ? 0.0f : __builtin_ldexpf(1.0f, -(int)n); }
 // x / 2^n, likewise: scaling by a power of two is exact (and rounds like the division where the result is subnormal)
@@ -143,17 +156,55 @@ __device__ __forceinline__ uint32_t muppet_scale_index_by_rows(unsigned bitwidth
     // bound = 2^(b-1) - 0.5 = (2 - 2^-(b-1)) * 2^(b-2) for the maximum, 2^(b-1) + 0.5 = (1 + 2^-b) * 2^(b-1) for the minimum
     const uint32_t eb = upper ? bitwidth - 1u : bitwidth - 2u;
     const uint32_t t_mant = upper ? (0x800000u >> bitwidth) : 0x800000u - (0x800000u >> (bitwidth - 1u));
-    const uint32_t xb = bits(extreme) & 0x7fffffffu;
+    const uint32_t xb = bits(extreme);
     const uint32_t mant = xb & 0x7fffffu;
-    const int idx = (int)(eb + 127u) - (int)(xb >> 23) - (mant > t_mant ? 1 : 0);
-    const bool near = mant - t_mant + 64u <= 128u;                                      // |mant - t_mant| <= 64
-    if (__builtin_amdgcn_ballot_w64(near) != 0ull) return muppet_scale_index_slow(bitwidth, extreme, upper);
-    // 2^32 - 1 marks x = 0, 2^32 - 2 an overflowing quotient: the smaller of the two sides plus one when it is a mark
-    // gives 0 for two zeros (the reference's special case) and 2^32 - 1 when the finite side overflows as well
-    const uint32_t side = xb == 0u ? 0xffffffffu : (idx < 0 ? 0u : (idx >= 128 ? 0xfffffffeu : (uint32_t)idx));
-    const uint32_t both = step_xor32(side, OpUMin());
-    return both + (both >= 0xfffffffeu ? 1u : 0u);
+    const uint32_t idx = (eb + 127u) - ((xb >> 23) & 0xffu) - (mant > t_mant ? 1u : 0u);
+    // Everything that is not a plain index 0..127 on a side goes the long way: a mantissa within 64 ulps of the
+    // threshold, an extreme of zero or below 2^-121 (index 128 and more: the quotient is infinite), one above the
+    // bound (negative index), an infinity or a NaN.  None of them occurs on rows of a model that is being trained.
+    const bool rare = (mant - t_mant + 64u <= 128u) | (idx >= 128u);
+    if (__builtin_amdgcn_ballot_w64(rare) != 0ull) return muppet_scale_index_slow(bitwidth, extreme, upper);
+    return step_xor32(idx, OpUMin());
 }
+
+// The same without the long way: false when any lane would need it (`both` is then meaningless).
+__device__ __forceinline__ bool muppet_scale_index_plain(unsigned bitwidth, float extreme, bool upper, uint32_t& both)
+{
+    const uint32_t eb = upper ? bitwidth - 1u : bitwidth - 2u;
+    const uint32_t t_mant = upper ? (0x800000u >> bitwidth) : 0x800000u - (0x800000u >> (bitwidth - 1u));
+    const uint32_t xb = bits(extreme);
+    const uint32_t mant = xb & 0x7fffffu;
+    const uint32_t idx = (eb + 127u) - ((xb >> 23) & 0xffu) - (mant > t_mant ? 1u : 0u);
+    const bool rare = (mant - t_mant + 64u <= 128u) | (idx >= 128u);
+    both = step_xor32(idx, OpUMin());
+    return __builtin_amdgcn_ballot_w64(rare) == 0ull;
+}
+// (signed char) of roundf(x * 2^n) when |x| is at most the extreme that a plain scale index n was taken from: the
+// product then lies inside (-128.5, 127.5) by more than 64 ulps of the extreme, so nothing saturates and x is a number
+__device__ __forceinline__ int round_to_i8_in_range(float x, float s) { return hw_cvt_i32(__builtin_fmaf(x, s, __builtin_copysignf(0x1.fffffep-2f, x))); }
+
+// round_to_i8(x * 2^n) for a wave-uniform x and n on the scalar unit: |x| = m * 2^-c with an integer m < 2^24, so
+// roundf(|x| * 2^n) = (m + 2^(sh-1)) >> sh with sh = c - n (halves away from zero), saturated at `bound` (127 for a
+// positive x, 128 for a negative one); sh <= 0 means |x| * 2^n >= 2^23, which saturates like sh = 1.
+struct UniformI8 {
+    uint32_t m; int c; int bound; int sign; bool finite;
+    __device__ __forceinline__ void set(float x)
+    {
+        const uint32_t b = bits(x), e = (b >> 23) & 0xffu, mant = b & 0x7fffffu;
+        m = e ? (mant | 0x800000u) : mant;
+        c = 150 - (int)(e ? e : 1u);
+        sign = (b >> 31) ? -1 : 1;
+        bound = (b >> 31) ? 128 : 127;
+        finite = e != 0xffu;
+    }
+    __device__ __forceinline__ int scaled(uint32_t n) const
+    {
+        const int sh = c - (int)n;
+        const uint32_t r = (m + (1u << ((uint32_t)(sh - 1) & 31u))) >> ((uint32_t)sh & 31u);
+        const uint32_t mag = sh < 1 ? (uint32_t)bound : (sh > 31 ? 0u : (r > (uint32_t)bound ? (uint32_t)bound : r));
+        return sign * (int)mag;
+    }
+};
 
 template <int K, bool COH> struct MuppetRule : DenseBase<K, COH> {
     using Base = DenseBase<K, COH>;
@@ -173,6 +224,11 @@ template <int K, bool COH> struct MuppetRule : DenseBase<K, COH> {
     float lrate, lambda; uint32_t first_sample; float* sum_updated_val; int fwd, bwd;
     float sum_norms_reg;
     float grad_acc[K / 64];
+    // 8-bit backward pass on the short path: -lambda as an integer mantissa and exponent, and the largest scale index
+    // for which lrate * 2^(-2 index) is a normal number computed exactly by exponent arithmetic
+    UniformI8 neg_lambda_q;
+    bool plain_8bit;
+    static constexpr uint32_t kShortPathMaxIndex = 48;
 
     __device__ __forceinline__ void init(const Params& a, uint8_t*, int lane_, uint32_t)
     {
@@ -182,6 +238,10 @@ template <int K, bool COH> struct MuppetRule : DenseBase<K, COH> {
         sum_norms_reg = 0.f;
 #pragma unroll
         for (int e = 0; e < E; ++e) grad_acc[e] = 0.f;
+        neg_lambda_q.set(-1 * lambda);
+        // lrate in [2^-20, 2^20]: with 2 * index <= 96 the product lrate * 2^(-2 index) and every float(int) * that stay normal
+        const uint32_t le = (bits(lrate) >> 23) & 0x1ffu;
+        plain_8bit = fwd == 8 && bwd == 8 && neg_lambda_q.finite && le >= 107u && le <= 147u;
     }
     // sum over the k values x[j]^2 in the reference's order: per lane (x0^2 + x1^2) + (x2^2 + x3^2); sq[e] = own squares
     static __device__ __forceinline__ float lane_sum_of_squares(const float* sq)
@@ -190,9 +250,11 @@ template <int K, bool COH> struct MuppetRule : DenseBase<K, COH> {
         if constexpr (E == 2) { const float b = step_xor32(sq[1], OpAdd()); a = a + b; }
         return a;
     }
-    template <int CLS, bool HOT> __device__ __forceinline__ void update(Row& row, const Info& i, uint32_t processed)
+    // The change of a row is lrate * g.  Both gradient functions return g as g_base * g_scale and lrate * g as
+    // g_base * d_scale, one rounding each.
+    // Every bit width and every input, as the reference computes it.
+    __device__ __forceinline__ void gradients(const float* p, const float* q, float r, float* gbp, float* gbq, float& g_scale, float& d_scale) const
     {
-        const float* p = row.p; const float* q = row.q;
         const bool upper = this->lane >= 32;
         // extrema by rows of 16 lanes: max p, max q, -min p, -min q (all 0 when the forward pass is binary32, as in the reference)
         float extrema = 0, sp = 0, sq = 0, pred;
@@ -206,14 +268,17 @@ template <int K, bool COH> struct MuppetRule : DenseBase<K, COH> {
             extrema = max4_by_rows(a, b, c, d);
             const uint32_t idx = muppet_scale_index_by_rows((unsigned)fwd, extrema, upper);      // rows 0,2: p   rows 1,3: q
             ip = bcast(idx, 0); iq = bcast(idx, 16);
-            sp = pow2u(ip); sq = pow2u(iq);
+            sp = pow2u_bits(ip); sq = pow2u_bits(iq);
         }
         if (fwd == 8) {
             int acc = 0;
 #pragma unroll
-            for (int e = 0; e < E; ++e) acc += round_to_i8(p[e] * sp) * round_to_i8(q[e] * sq);
+            for (int e = 0; e < E; ++e) acc += round_to_i8_scaled(p[e], sp) * round_to_i8_scaled(q[e], sq);
             acc = reduce_wave(acc, OpAdd());
-            pred = div_pow2((float)acc, ip + iq);                        // acc / (sp * sq)
+            // acc / (sp * sq): the divisor is a power of two, or infinite from 2^128 on (quotient 0 with the sign of acc,
+            // which is what 2^-1000 gives)
+            const uint32_t n = (ip > 1000u ? 1000u : ip) + (iq > 1000u ? 1000u : iq);
+            pred = __builtin_ldexpf((float)acc, n > 127u ? -1000 : -(int)n);
         } else if (fwd == 32) {
             float m[E];
 #pragma unroll
@@ -227,33 +292,32 @@ template <int K, bool COH> struct MuppetRule : DenseBase<K, COH> {
             t = reduce_half_wave(t, OpAdd());
             pred = (float)(half_t)step_xor32(t, OpAdd());
         }
-        const float ruv = i.r - pred;
+        const float ruv = r - pred;
         float sb = 0;
         uint32_t ib = 0;
         if (bwd != 32) {
             // max(p_max, q_max, -lambda, ruv) in the lower half-wave, -min(p_min, q_min, -lambda, ruv) in the upper one
-            const float neg_lambda = -1 * lambda;
-            const float pq = step_xor16(extrema, OpMaximum());
-            const float lr_ = upper ? OpMaximum()(-neg_lambda, -ruv) : OpMaximum()(neg_lambda, ruv);
-            ib = bcast(muppet_scale_index_by_rows((unsigned)bwd, OpMaximum()(pq, lr_), upper), 0);
-            sb = pow2u(ib);
+            const uint32_t flip = upper ? 0x80000000u : 0u;
+            const float pq = OpMaximum()(step_xor16(extrema, OpMaximum()), from_bits<float>(bits(-1 * lambda) ^ flip));
+            ib = bcast(muppet_scale_index_by_rows((unsigned)bwd, OpMaximum()(pq, from_bits<float>(bits(ruv) ^ flip)), upper), 0);
+            sb = pow2u_bits(ib);
         }
-        float gp[E], gq[E];
+        g_scale = 1.0f; d_scale = lrate;
         if (bwd == 8) {
+            const int ruv_i = round_to_i8_scaled(ruv, sb);
             const float sq_rev = pow2_reciprocal(2u * ib);
-            const int ruv_i = round_to_i8(ruv * sb);
-            const int lam_i = round_to_i8(-1.0f * lambda * sb);
+            const int lam_i = round_to_i8_scaled(-1.0f * lambda, sb);
 #pragma unroll
             for (int e = 0; e < E; ++e) {
-                const int pi = round_to_i8(p[e] * sb), qi = round_to_i8(q[e] * sb);
-                gp[e] = (float)(qi * ruv_i + pi * lam_i) * sq_rev;
-                gq[e] = (float)(pi * ruv_i + qi * lam_i) * sq_rev;
+                const int pi = round_to_i8_scaled(p[e], sb), qi = round_to_i8_scaled(q[e], sb);
+                gbp[e] = (float)(qi * ruv_i + pi * lam_i) * sq_rev;
+                gbq[e] = (float)(pi * ruv_i + qi * lam_i) * sq_rev;
             }
         } else if (bwd == 32) {
 #pragma unroll
             for (int e = 0; e < E; ++e) {
-                gp[e] = ruv * q[e] - lambda * p[e];
-                gq[e] = ruv * p[e] - lambda * q[e];
+                gbp[e] = ruv * q[e] - lambda * p[e];
+                gbq[e] = ruv * p[e] - lambda * q[e];
             }
         } else {
             const float sb_rev = pow2_reciprocal(ib);
@@ -261,21 +325,72 @@ template <int K, bool COH> struct MuppetRule : DenseBase<K, COH> {
 #pragma unroll
             for (int e = 0; e < E; ++e) {
                 const half_t ph = grid_h(p[e], sb, sb_rev), qh = grid_h(q[e], sb, sb_rev);
-                gp[e] = (float)(half_t)(qh * t_ruv + ph * t_lam);
-                gq[e] = (float)(half_t)(ph * t_ruv + qh * t_lam);
+                gbp[e] = (float)(half_t)(qh * t_ruv + ph * t_lam);
+                gbq[e] = (float)(half_t)(ph * t_ruv + qh * t_lam);
             }
         }
+    }
+    // 8-bit forward and backward pass when both scale indices are plain ones and the backward index is small: nothing
+    // saturates, the quantised -lambda comes from the scalar unit, and lrate * 2^(-2 index) from exponent arithmetic
+    // (g = integer * 2^(-2 index) is exact, so lrate * g = integer * (lrate * 2^(-2 index)) with the same one
+    // rounding).  False, with nothing written, when the inputs are not of that kind.
+    __device__ __forceinline__ bool gradients_8bit_plain(const float* p, const float* q, float r, float* gbp, float* gbq, float& g_scale, float& d_scale) const
+    {
+        const bool upper = this->lane >= 32;
+        float a = p[0], b = -p[0], c = q[0], d = -q[0];
+        if constexpr (E == 2) {
+            a = OpMaximum()(a, p[1]); b = OpMaximum()(b, -p[1]);
+            c = OpMaximum()(c, q[1]); d = OpMaximum()(d, -q[1]);
+        }
+        const float extrema = max4_by_rows(a, b, c, d);
+        uint32_t idx;
+        if (!muppet_scale_index_plain(8u, extrema, upper, idx)) return false;
+        const uint32_t ip = bcast(idx, 0), iq = bcast(idx, 16);
+        const float sp = pow2u_bits(ip), sq = pow2u_bits(iq);
+        int acc = 0;
+#pragma unroll
+        for (int e = 0; e < E; ++e) acc += round_to_i8_in_range(p[e], sp) * round_to_i8_in_range(q[e], sq);
+        acc = reduce_wave(acc, OpAdd());
+        const uint32_t n = ip + iq;                                            // at most 254
+        const float pred = __builtin_ldexpf((float)acc, n > 127u ? -1000 : -(int)n);
+        const float ruv = r - pred;
+        const uint32_t flip = upper ? 0x80000000u : 0u;
+        const float pq = OpMaximum()(step_xor16(extrema, OpMaximum()), from_bits<float>(bits(-1 * lambda) ^ flip));
+        uint32_t idx_b;
+        if (!muppet_scale_index_plain(8u, OpMaximum()(pq, from_bits<float>(bits(ruv) ^ flip)), upper, idx_b)) return false;
+        const uint32_t ib = bcast(idx_b, 0);
+        if (ib > kShortPathMaxIndex) return false;
+        const float sb = pow2u_bits(ib);
+        const int ruv_i = round_to_i8_in_range(ruv, sb);
+        const int lam_i = neg_lambda_q.scaled(ib);
+        g_scale = from_bits<float>((127u - 2u * ib) << 23);
+        d_scale = from_bits<float>(bits(lrate) - (ib << 24));
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+            const int pi = round_to_i8_in_range(p[e], sb), qi = round_to_i8_in_range(q[e], sb);
+            gbp[e] = (float)(qi * ruv_i + pi * lam_i);
+            gbq[e] = (float)(pi * ruv_i + qi * lam_i);
+        }
+        return true;
+    }
+    template <int CLS, bool HOT> __device__ __forceinline__ void update(Row& row, const Info& i, uint32_t processed)
+    {
+        float gbp[E], gbq[E], g_scale, d_scale;
+        if (!(plain_8bit && gradients_8bit_plain(row.p, row.q, i.r, gbp, gbq, g_scale, d_scale)))
+            gradients(row.p, row.q, i.r, gbp, gbq, g_scale, d_scale);
         float dp[E], dq[E];
 #pragma unroll
         for (int e = 0; e < E; ++e) {
-            dp[e] = lrate * gp[e];
-            dq[e] = lrate * gq[e];
+            dp[e] = d_scale * gbp[e];
+            dq[e] = d_scale * gbq[e];
             row.p[e] = (i.thin & 1u) ? row.p[e] : row.p[e] + dp[e];
             row.q[e] = (i.thin & 2u) ? row.q[e] : row.q[e] + dq[e];
         }
         this->template store<HOT>(row, i, dp, dq);
         if (fwd != 32 && bwd != 32 && processed >= first_sample) {
-            float sp2[E], sq2[E];
+            float gp[E], gq[E], sp2[E], sq2[E];
+#pragma unroll
+            for (int e = 0; e < E; ++e) { gp[e] = gbp[e] * g_scale; gq[e] = gbq[e] * g_scale; }
 #pragma unroll
             for (int e = 0; e < E; ++e) { sp2[e] = gp[e] * gp[e]; sq2[e] = gq[e] * gq[e]; }
             float npq = lane_sum_of_squares(sp2) + lane_sum_of_squares(sq2);
@@ -306,6 +421,8 @@ __device__ __forceinline__ float afp_scale_index(unsigned bitwidth, float max_v)
     return fabsf(ceilf(__builtin_log2f(max_v / denom)));
 }
 __device__ __forceinline__ float afp_grid(float v, float s, float s_rev) { return round_half_away(v * s) * s_rev; }
+// the same for a scale s = 2^n, n >= 0 (the product is exact or infinite, so the fused form rounds alike)
+__device__ __forceinline__ float afp_grid_pow2(float v, float s, float s_rev) { return round_half_away_scaled(v, s) * s_rev; }
 // QPA, afp_sgd_kernel.h:104-125
 __device__ __forceinline__ AfpQ afp_qpa(float diff, float range, float prev)
 {
@@ -337,6 +454,13 @@ template <int K, bool COH> struct AfpRule : DenseBase<K, COH> {
     int upd_u, upd_i, upd_b, cur_iter;
     float sp, sq, sb;
     bool upper;
+    // What follows from the three quantisers alone, computed when one of them is re-measured (wave-uniform, kept in
+    // scalar registers): the exponent that turns the int8 dot into the prediction, the reciprocal scales of the 16-bit
+    // paths, the quantised -lambda of both backward paths, 2^(-2 r) and, where it is exact, lrate * 2^(-2 r).
+    int pred_exp; float sp_rev, sq_rev;
+    int lam_i8; float sb_rev2, d_scale8; bool fused8;
+    float sb_rev; half_t t_lam16;
+    bool lrate_plain;
 
     __device__ __forceinline__ void init(const Params& a, uint8_t*, int lane_, uint32_t)
     {
@@ -345,6 +469,27 @@ template <int K, bool COH> struct AfpRule : DenseBase<K, COH> {
         afp_epoch = a.afp_epoch; init_threshold = a.init_threshold;
         uq = AfpQ{0, 0, 0, 0.f}; iq = uq; bq = uq;
         upd_u = upd_i = upd_b = cur_iter = 0; sp = sq = sb = 0.f; upper = lane_ >= 32;
+        pred_exp = 0; sp_rev = sq_rev = sb_rev = sb_rev2 = d_scale8 = 0.f; lam_i8 = 0; fused8 = false; t_lam16 = (half_t)0.f;
+        // lrate in [2^-20, 2^20]: with 2 r <= 96, lrate * 2^(-2 r) and every float(int) * that stay normal numbers
+        const uint32_t le = (bits(lrate) >> 23) & 0x1ffu;
+        lrate_plain = le >= 107u && le <= 147u;
+    }
+    __device__ __forceinline__ void forward_changed()
+    {
+        const uint32_t n = (uint32_t)uq.r + (uint32_t)iq.r;                      // r >= 0
+        pred_exp = n > 127u ? -1000 : -(int)n;                                   // acc / (sp * sq): 2^-n, or 0 with the sign of acc
+        sp_rev = ufirst(pow2_reciprocal((uint32_t)uq.r)); sq_rev = ufirst(pow2_reciprocal((uint32_t)iq.r));
+    }
+    __device__ __forceinline__ void backward_changed()
+    {
+        const uint32_t r = (uint32_t)bq.r;
+        lam_i8 = ufirst(round_to_i8_scaled(-1.0f * lambda, sb));
+        sb_rev2 = ufirst(pow2_reciprocal(2u * r));
+        // g = integer * 2^(-2 r) is exact for small r, so lrate * g = integer * (lrate * 2^(-2 r)) with the same one rounding
+        fused8 = lrate_plain && r <= 48u;
+        d_scale8 = from_bits<float>(bits(lrate) - ((fused8 ? r : 0u) << 24));
+        sb_rev = ufirst(pow2_reciprocal(r));
+        t_lam16 = from_bits<half_t>((uint32_t)__builtin_amdgcn_readfirstlane((int)bits((half_t)afp_grid_pow2(-1.0f * lambda, sb, sb_rev))));
     }
     // QEM / QEM_64, afp_sgd_kernel.h:32-59
     __device__ __forceinline__ float qem(const float* v, float max_v) const
@@ -389,6 +534,7 @@ template <int K, bool COH> struct AfpRule : DenseBase<K, COH> {
             if (cur_iter == 0) uq.mov_avg_range = mx;
             uq = uniform(afp_qpa(diff, mx, uq.mov_avg_range));
             sp = pow2i(uq.r);
+            forward_changed();
             if (afp_epoch == 0 && cur_iter < init_threshold) uq.itv = 1;
             upd_u += uq.itv;
         }
@@ -399,6 +545,7 @@ template <int K, bool COH> struct AfpRule : DenseBase<K, COH> {
             if (cur_iter == 0) iq.mov_avg_range = mx;
             iq = uniform(afp_qpa(diff, mx, iq.mov_avg_range));
             sq = pow2i(iq.r);
+            forward_changed();
             if (afp_epoch == 0 && cur_iter < init_threshold) iq.itv = 1;
             upd_i += iq.itv;
         }
@@ -406,14 +553,13 @@ template <int K, bool COH> struct AfpRule : DenseBase<K, COH> {
         if (uq.n == 8 && iq.n == 8) {
             int acc = 0;
 #pragma unroll
-            for (int e = 0; e < E; ++e) acc += round_to_i8(p[e] * sp) * round_to_i8(q[e] * sq);
+            for (int e = 0; e < E; ++e) acc += round_to_i8_scaled(p[e], sp) * round_to_i8_scaled(q[e], sq);
             acc = reduce_wave(acc, OpAdd());
-            pred = div_pow2((float)acc, (uint32_t)uq.r + (uint32_t)iq.r);            // acc / (sp * sq); r >= 0
+            pred = __builtin_ldexpf((float)acc, pred_exp);                           // acc / (sp * sq)
         } else {
-            const float sp_rev = pow2_reciprocal((uint32_t)uq.r), sq_rev = pow2_reciprocal((uint32_t)iq.r);
             // the reference's half2 lanes: .x sums elements l, l+64 (lower half-wave here), .y elements l+32, l+96 (upper)
-            half_t t = (half_t)afp_grid(p[0], sp, sp_rev) * (half_t)afp_grid(q[0], sq, sq_rev);
-            if constexpr (E == 2) t = t + (half_t)afp_grid(p[1], sp, sp_rev) * (half_t)afp_grid(q[1], sq, sq_rev);
+            half_t t = (half_t)afp_grid_pow2(p[0], sp, sp_rev) * (half_t)afp_grid_pow2(q[0], sq, sq_rev);
+            if constexpr (E == 2) t = t + (half_t)afp_grid_pow2(p[1], sp, sp_rev) * (half_t)afp_grid_pow2(q[1], sq, sq_rev);
             t = reduce_half_wave(t, OpAdd());
             pred = (float)(half_t)step_xor32(t, OpAdd());
         }
@@ -427,35 +573,39 @@ template <int K, bool COH> struct AfpRule : DenseBase<K, COH> {
             if (cur_iter == 0) bq.mov_avg_range = mx;
             bq = uniform(afp_qpa(diff, mx, bq.mov_avg_range));
             sb = pow2i(bq.r);
+            backward_changed();
             if (afp_epoch == 0 && cur_iter < init_threshold) bq.itv = 1;
             upd_b += bq.itv;
         }
-        float gp[E], gq[E];
+        // the change of a row is lrate * g = g_base * d_scale
+        float gbp[E], gbq[E], d_scale = lrate;
         if (bq.n == 8) {
-            const int lam_i = round_to_i8(-1.0f * lambda * sb);
-            const int ruv_i = round_to_i8(ruv * sb);
-            const float sq_rev = pow2_reciprocal(2u * (uint32_t)bq.r);
+            const int ruv_i = round_to_i8_scaled(ruv, sb);
 #pragma unroll
             for (int e = 0; e < E; ++e) {
-                const int pi = round_to_i8(p[e] * sb), qi = round_to_i8(q[e] * sb);
-                gp[e] = (float)(qi * ruv_i + pi * lam_i) * sq_rev;
-                gq[e] = (float)(pi * ruv_i + qi * lam_i) * sq_rev;
+                const int pi = round_to_i8_scaled(p[e], sb), qi = round_to_i8_scaled(q[e], sb);
+                gbp[e] = (float)(qi * ruv_i + pi * lam_i8);
+                gbq[e] = (float)(pi * ruv_i + qi * lam_i8);
+            }
+            if (fused8) d_scale = d_scale8;
+            else {
+#pragma unroll
+                for (int e = 0; e < E; ++e) { gbp[e] = gbp[e] * sb_rev2; gbq[e] = gbq[e] * sb_rev2; }
             }
         } else {
-            const float sb_rev = pow2_reciprocal((uint32_t)bq.r);
-            const half_t t_ruv = (half_t)afp_grid(ruv, sb, sb_rev), t_lam = (half_t)afp_grid(-1.0f * lambda, sb, sb_rev);
+            const half_t t_ruv = (half_t)afp_grid_pow2(ruv, sb, sb_rev);
 #pragma unroll
             for (int e = 0; e < E; ++e) {
-                const half_t ph = (half_t)afp_grid(p[e], sb, sb_rev), qh = (half_t)afp_grid(q[e], sb, sb_rev);
-                gp[e] = (float)(half_t)(qh * t_ruv + ph * t_lam);
-                gq[e] = (float)(half_t)(ph * t_ruv + qh * t_lam);
+                const half_t ph = (half_t)afp_grid_pow2(p[e], sb, sb_rev), qh = (half_t)afp_grid_pow2(q[e], sb, sb_rev);
+                gbp[e] = (float)(half_t)(qh * t_ruv + ph * t_lam16);
+                gbq[e] = (float)(half_t)(ph * t_ruv + qh * t_lam16);
             }
         }
         float dp[E], dq[E];
 #pragma unroll
         for (int e = 0; e < E; ++e) {
-            dp[e] = lrate * gp[e];
-            dq[e] = lrate * gq[e];
+            dp[e] = d_scale * gbp[e];
+            dq[e] = d_scale * gbq[e];
             row.p[e] = (i.thin & 1u) ? row.p[e] : row.p[e] + dp[e];
             row.q[e] = (i.thin & 2u) ? row.q[e] : row.q[e] + dq[e];
         }
