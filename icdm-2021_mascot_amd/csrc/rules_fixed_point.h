@@ -168,20 +168,35 @@ __device__ __forceinline__ uint32_t muppet_scale_index_by_rows(unsigned bitwidth
 }
 
 // The same without the long way: false when any lane would need it (`both` is then meaningless).
-__device__ __forceinline__ bool muppet_scale_index_plain(unsigned bitwidth, float extreme, bool upper, uint32_t& both)
+// `side` is the lane's own side's index; the index of a range is the smaller of its two sides' (lanes L and L ^ 32).
+__device__ __forceinline__ bool muppet_scale_index_plain(unsigned bitwidth, float extreme, bool upper, uint32_t& side)
 {
     const uint32_t eb = upper ? bitwidth - 1u : bitwidth - 2u;
     const uint32_t t_mant = upper ? (0x800000u >> bitwidth) : 0x800000u - (0x800000u >> (bitwidth - 1u));
+    const uint32_t near_bias = 64u - t_mant;
     const uint32_t xb = bits(extreme);
     const uint32_t mant = xb & 0x7fffffu;
-    const uint32_t idx = (eb + 127u) - ((xb >> 23) & 0xffu) - (mant > t_mant ? 1u : 0u);
-    const bool rare = (mant - t_mant + 64u <= 128u) | (idx >= 128u);
-    both = step_xor32(idx, OpUMin());
+    side = (eb + 127u) - ((xb >> 23) & 0xffu) - (mant > t_mant ? 1u : 0u);
+    const bool rare = (mant + near_bias <= 128u) | (side >= 128u);
     return __builtin_amdgcn_ballot_w64(rare) == 0ull;
 }
 // (signed char) of roundf(x * 2^n) when |x| is at most the extreme that a plain scale index n was taken from: the
-// product then lies inside (-128.5, 127.5) by more than 64 ulps of the extreme, so nothing saturates and x is a number
-__device__ __forceinline__ int round_to_i8_in_range(float x, float s) { return hw_cvt_i32(__builtin_fmaf(x, s, __builtin_copysignf(0x1.fffffep-2f, x))); }
+// product then lies inside (-128.5, 127.5) by more than 64 ulps of the extreme, so nothing saturates, x is a number,
+// and the conversion is an ordinary truncating cast
+__device__ __forceinline__ int round_to_i8_in_range(float x, float s) { return (int)__builtin_fmaf(x, s, __builtin_copysignf(0x1.fffffep-2f, x)); }
+// Products of such values as 24-bit multiplications (full rate, where the 32-bit one is not); the compiler chooses them
+// by itself only behind a clamp that shows it the range.  Ordinary vector instructions: no wait states of their own.
+__device__ __forceinline__ int mul_i24(int a, int b) { int r; asm("v_mul_i32_i24_e32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b)); return r; }
+__device__ __forceinline__ int mad_i24(int a, int b, int c) { int r; asm("v_mad_i32_i24 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c)); return r; }
+// the same with a wave-uniform second factor in a scalar register
+__device__ __forceinline__ int mad_i24_uniform(int a, int b, int c) { int r; asm("v_mad_i32_i24 %0, %1, %2, %3" : "=v"(r) : "v"(a), "s"(b), "v"(c)); return r; }
+// Sum of an int over the 64 lanes as a wave-uniform value: rotations inside the rows, then the four row sums meet on
+// the scalar unit (integer addition: any order)
+__device__ __forceinline__ int sum_wave_uniform(int x)
+{
+    x = reduce_row16(x, OpAdd());
+    return __builtin_amdgcn_readlane(x, 0) + __builtin_amdgcn_readlane(x, 16) + __builtin_amdgcn_readlane(x, 32) + __builtin_amdgcn_readlane(x, 48);
+}
 
 // round_to_i8(x * 2^n) for a wave-uniform x and n on the scalar unit: |x| = m * 2^-c with an integer m < 2^24, so
 // roundf(|x| * 2^n) = (m + 2^(sh-1)) >> sh with sh = c - n (halves away from zero), saturated at `bound` (127 for a
@@ -345,12 +360,17 @@ template <int K, bool COH> struct MuppetRule : DenseBase<K, COH> {
         const float extrema = max4_by_rows(a, b, c, d);
         uint32_t idx;
         if (!muppet_scale_index_plain(8u, extrema, upper, idx)) return false;
-        const uint32_t ip = bcast(idx, 0), iq = bcast(idx, 16);
+        // rows 0, 2: the two sides of p; rows 1, 3: of q
+        const uint32_t ip0 = bcast(idx, 0), ip1 = bcast(idx, 32), iq0 = bcast(idx, 16), iq1 = bcast(idx, 48);
+        const uint32_t ip = ip0 < ip1 ? ip0 : ip1, iq = iq0 < iq1 ? iq0 : iq1;
         const float sp = pow2u_bits(ip), sq = pow2u_bits(iq);
         int acc = 0;
 #pragma unroll
-        for (int e = 0; e < E; ++e) acc += round_to_i8_in_range(p[e], sp) * round_to_i8_in_range(q[e], sq);
-        acc = reduce_wave(acc, OpAdd());
+        for (int e = 0; e < E; ++e) {
+            const int pi = round_to_i8_in_range(p[e], sp), qi = round_to_i8_in_range(q[e], sq);
+            acc = e == 0 ? mul_i24(pi, qi) : mad_i24(pi, qi, acc);
+        }
+        acc = sum_wave_uniform(acc);
         const uint32_t n = ip + iq;                                            // at most 254
         const float pred = __builtin_ldexpf((float)acc, n > 127u ? -1000 : -(int)n);
         const float ruv = r - pred;
@@ -358,18 +378,19 @@ template <int K, bool COH> struct MuppetRule : DenseBase<K, COH> {
         const float pq = OpMaximum()(step_xor16(extrema, OpMaximum()), from_bits<float>(bits(-1 * lambda) ^ flip));
         uint32_t idx_b;
         if (!muppet_scale_index_plain(8u, OpMaximum()(pq, from_bits<float>(bits(ruv) ^ flip)), upper, idx_b)) return false;
-        const uint32_t ib = bcast(idx_b, 0);
+        const uint32_t ib0 = bcast(idx_b, 0), ib1 = bcast(idx_b, 32);
+        const uint32_t ib = ib0 < ib1 ? ib0 : ib1;
         if (ib > kShortPathMaxIndex) return false;
         const float sb = pow2u_bits(ib);
         const int ruv_i = round_to_i8_in_range(ruv, sb);
-        const int lam_i = neg_lambda_q.scaled(ib);
+        const int lam_v = neg_lambda_q.scaled(ib);
         g_scale = from_bits<float>((127u - 2u * ib) << 23);
         d_scale = from_bits<float>(bits(lrate) - (ib << 24));
 #pragma unroll
         for (int e = 0; e < E; ++e) {
             const int pi = round_to_i8_in_range(p[e], sb), qi = round_to_i8_in_range(q[e], sb);
-            gbp[e] = (float)(qi * ruv_i + pi * lam_i);
-            gbq[e] = (float)(pi * ruv_i + qi * lam_i);
+            gbp[e] = (float)mad_i24_uniform(pi, lam_v, mul_i24(qi, ruv_i));
+            gbq[e] = (float)mad_i24_uniform(qi, lam_v, mul_i24(pi, ruv_i));
         }
         return true;
     }
