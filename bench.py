@@ -30,8 +30,8 @@ TRAIN = dict(epochs=50, lr=0.01, decay=0.1, lam=0.015, sample_ratio=0.05, interv
 # device copy gives), recorded in the profile named here; reported only for the workload they were taken on
 PROFILED_TRAFFIC = {
     # (config, training ratings, k, seed, workers): bytes per epoch (four launches of the update kernel)
-    (4, 100_000_000, 128, 2021, 6104): dict(
-        bytes=(2 * 14_908_600 + 29_211_562) * 1024,
+    (4, 100_000_000, 128, 2021, 48832): dict(
+        bytes=(2 * 15_071_100 + 29_504_070) * 1024,
         source="rocprofv3 --pmc FETCH_SIZE (x2.0) and WRITE_SIZE (x1.0) of the four update launches of epoch 2, recorded in "
                "profiles/hogwild_mascot_k128_config4_hbm_traffic.md; not re-measured by this run"),
 }
@@ -158,7 +158,7 @@ def main():
     ap.add_argument("--config", type=int, default=4, choices=(2, 3, 4, 5), help="BASELINE.json configuration (4 = the one the metric is quoted on)")
     ap.add_argument("--ratings", type=int, default=0, help="training ratings (default: the configuration's; the test set is scaled alike)")
     ap.add_argument("--k", type=int, default=128, choices=(64, 128))
-    ap.add_argument("--workers", type=int, default=0, help="-wg (default 0: mf_auto_workers(ratings); 6104 at config 4)")
+    ap.add_argument("--workers", type=int, default=0, help="-wg (default 0: mf_auto_workers(ratings); 48832 at config 4)")
     ap.add_argument("--seed", type=int, default=2021)
     ap.add_argument("--replicate", type=float, default=-1.0, help="mf_params.replicate_inflight (default: derived from learning rate and mean rating)")
     ap.add_argument("--merges", type=int, default=0, help="mf_params.replica_merges (default: the library's)")
@@ -221,7 +221,7 @@ def main():
     bytes_per_update = 12 + 2 * k * (2 + 2)
     gbs = updates * bytes_per_update / (ms / 1e3) / 1e9
     epochs_done_timed = a.warmup + a.steps
-    launches = int(prm.replica_merges) if (rep_u or rep_v) and prm.replica_merges else 1
+    launches = capi.HogwildOptions.from_address(sess.device_state(a.warmup)[1]).launches or 1
     plain = [m for i, m in enumerate(main_run["timed"]) if not is_check_epoch(a.warmup + i)] or list(main_run["timed"])
     out = {
         "metric": "SGD ratings/sec/epoch & % HBM roofline at k=128 on 1 MI355X; test RMSE delta",
@@ -277,6 +277,7 @@ def main():
         rep = sess.report
         out["whole_job"] = {"note": "the 50-epoch run this session ended up being: update launches of all epochs, switching included",
                             "epochs": TRAIN["epochs"], "sgd_ms_total": float(np.sum(main_run["ms"])), "sgd_ms_per_epoch": float(np.mean(main_run["ms"])),
+                            "sgd_ms_epochs": [round(float(x), 2) for x in main_run["ms"]],
                             "ratings_per_s": n_train * TRAIN["epochs"] / (float(np.sum(main_run["ms"])) / 1e3),
                             "preprocess_ms": rep.preprocess_ms, "error_ms": rep.error_ms, "switching_ms": rep.switching_ms,
                             "final_test_rmse": main_run["rmse"][-1]}

@@ -107,7 +107,7 @@ int main(int argc, const char* argv[])
         std::cout << "updates of rows with more than one update in flight are added";
         if (prm.replicate_inflight < 0) std::cout << "; rows above 0.3 / (learning rate x mean rating) in flight are replicated per XCD";
         else if (prm.replicate_inflight > 0) std::cout << "; rows above " << prm.replicate_inflight << " in flight are replicated per XCD";
-        if (prm.replicate_inflight != 0) std::cout << ", merged " << prm.replica_merges << " times per epoch";
+        if (prm.replicate_inflight != 0 && prm.replica_merges) std::cout << ", merged " << prm.replica_merges << " times per epoch";
         if (prm.hot_row_inflight > 0) std::cout << "; rows above " << prm.hot_row_inflight << " in flight are thinned";
     }
     std::cout << std::endl;

@@ -184,12 +184,6 @@ __device__ __forceinline__ bool muppet_scale_index_plain(unsigned bitwidth, floa
 // product then lies inside (-128.5, 127.5) by more than 64 ulps of the extreme, so nothing saturates, x is a number,
 // and the conversion is an ordinary truncating cast
 __device__ __forceinline__ int round_to_i8_in_range(float x, float s) { return (int)__builtin_fmaf(x, s, __builtin_copysignf(0x1.fffffep-2f, x)); }
-// Products of such values as 24-bit multiplications (full rate, where the 32-bit one is not); the compiler chooses them
-// by itself only behind a clamp that shows it the range.  Ordinary vector instructions: no wait states of their own.
-__device__ __forceinline__ int mul_i24(int a, int b) { int r; asm("v_mul_i32_i24_e32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b)); return r; }
-__device__ __forceinline__ int mad_i24(int a, int b, int c) { int r; asm("v_mad_i32_i24 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c)); return r; }
-// the same with a wave-uniform second factor in a scalar register
-__device__ __forceinline__ int mad_i24_uniform(int a, int b, int c) { int r; asm("v_mad_i32_i24 %0, %1, %2, %3" : "=v"(r) : "v"(a), "s"(b), "v"(c)); return r; }
 // Sum of an int over the 64 lanes as a wave-uniform value: rotations inside the rows, then the four row sums meet on
 // the scalar unit (integer addition: any order)
 __device__ __forceinline__ int sum_wave_uniform(int x)
@@ -368,7 +362,7 @@ template <int K, bool COH> struct MuppetRule : DenseBase<K, COH> {
 #pragma unroll
         for (int e = 0; e < E; ++e) {
             const int pi = round_to_i8_in_range(p[e], sp), qi = round_to_i8_in_range(q[e], sq);
-            acc = e == 0 ? mul_i24(pi, qi) : mad_i24(pi, qi, acc);
+            acc += pi * qi;
         }
         acc = sum_wave_uniform(acc);
         const uint32_t n = ip + iq;                                            // at most 254
@@ -383,14 +377,14 @@ template <int K, bool COH> struct MuppetRule : DenseBase<K, COH> {
         if (ib > kShortPathMaxIndex) return false;
         const float sb = pow2u_bits(ib);
         const int ruv_i = round_to_i8_in_range(ruv, sb);
-        const int lam_v = neg_lambda_q.scaled(ib);
+        const int lam_i = neg_lambda_q.scaled(ib);
         g_scale = from_bits<float>((127u - 2u * ib) << 23);
         d_scale = from_bits<float>(bits(lrate) - (ib << 24));
 #pragma unroll
         for (int e = 0; e < E; ++e) {
             const int pi = round_to_i8_in_range(p[e], sb), qi = round_to_i8_in_range(q[e], sb);
-            gbp[e] = (float)mad_i24_uniform(pi, lam_v, mul_i24(qi, ruv_i));
-            gbq[e] = (float)mad_i24_uniform(qi, lam_v, mul_i24(pi, ruv_i));
+            gbp[e] = (float)(qi * ruv_i + pi * lam_i);
+            gbq[e] = (float)(pi * ruv_i + qi * lam_i);
         }
         return true;
     }

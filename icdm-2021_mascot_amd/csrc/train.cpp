@@ -232,7 +232,12 @@ struct HotRows {
         o.user_slot_row = u.slot_row.as<uint32_t>(); o.item_slot_row = v.slot_row.as<uint32_t>();
         o.user_replicas = u.replicas.p; o.item_replicas = v.replicas.p;
         o.user_slots = u.slots; o.item_slots = v.slots;
-        if ((u.slots || v.slots) && prm.epoch_splits == 0) o.launches = prm.replica_merges ? prm.replica_merges : 1u;
+        if ((u.slots || v.slots) && prm.epoch_splits == 0) {
+            // replica_merges = 0: a launch of at least 25M ratings, at most four launches (the end of a launch, where the
+            // last workers run alone, costs a short epoch 13 % per extra launch and a 100M-rating one 0.1 %)
+            const uint32_t by_size = n / 25000000u;
+            o.launches = prm.replica_merges ? prm.replica_merges : (by_size < 1u ? 1u : (by_size > 4u ? 4u : by_size));
+        }
         opt_early = o;
         if (early) { opt_early.user_keep = u.early.as<uint8_t>(); opt_early.item_keep = v.early.as<uint8_t>(); }
         return 0;
@@ -756,7 +761,7 @@ void mf_default_params(mf_params* out)       // main.cu:19-32
     // no reference counterpart (mf_hogwild_options): rows with more updates in flight than added updates can safely
     // sum (mf_replicate_threshold) get a copy per XCD, averaged four times per epoch; rows with more than one have
     // their updates added; nothing is thinned
-    out->hot_rows = 1; out->replicate_inflight = -1.0f; out->replica_merges = 4;
+    out->hot_rows = 1; out->replicate_inflight = -1.0f; out->replica_merges = 0;
     out->hot_row_inflight = 0.0f; out->hot_row_inflight_early = 0.0f; out->hot_row_early_epochs = 0;
 }
 
@@ -854,10 +859,15 @@ float mf_replicate_threshold(float learning_rate, float mean_rating)
 
 uint32_t mf_auto_workers(uint32_t n)
 {
-    // about 128 windows of 128 ratings per worker: the ratio at which the runs on 8M and on 100M ratings stay
-    // within 0.005 test RMSE of the reference rule run on the CPU; at most 24 wavefronts on each of the 256 CUs
-    uint32_t w = (n / 16384u + 3u) / 4u * 4u;
-    return w < 16u ? 16u : (w > 6144u ? 6144u : w);
+    // About 128 windows of 128 ratings per worker: the ratio at which the runs on 8M and on 100M ratings stay
+    // within 0.005 test RMSE of the reference rule run on the CPU.  From about 95M ratings on that count fills the chip
+    // (24 wavefronts on each of the 256 CUs = 6144 resident workers): the updates in flight, which decide the distance
+    // to a sequential run, no longer grow with the worker count, and workers with 16 windows each, eight times as many
+    // as are resident, even out the end of every launch (4 % of the epoch at 100M ratings).
+    const uint32_t w = (n / 16384u + 3u) / 4u * 4u;
+    if (w < 16u) return 16u;
+    if (w < 5800u) return w;
+    return (uint32_t)((((uint64_t)n + 2047u) / 2048u + 3u) / 4u * 4u);
 }
 
 int mf_train(const mf_params* params, const mf_node* R, uint32_t n, uint32_t n_users, uint32_t n_items,

@@ -164,8 +164,10 @@ uint32_t mf_mascot_norm_blocks(uint32_t num_workers);
 /* Host-side closed forms of the schedule (mf_methods.cu:94-111,170-175). */
 uint32_t mf_update_count(uint32_t n, uint32_t num_workers, uint32_t update_vector_size);
 /* Worker count mf_train uses for mf_params.num_workers == 0: n / 16384 (about 128 windows per worker), a multiple
- * of 4, between 16 and 6144.  The updates in flight grow with the workers and so does the distance to a sequential
- * run; the reference's fixed default (2048, main.cu:28) suits neither 400k nor 100M ratings on this GPU. */
+ * of 4, at least 16.  The updates in flight grow with the workers and so does the distance to a sequential run, until
+ * the chip is full (6144 resident workers, reached at about 95M ratings); from there on the count is n / 2048 (16
+ * windows per worker), which changes nothing in flight and evens out the end of every launch.  The reference's fixed
+ * default (2048, main.cu:28) suits neither 400k nor 100M ratings on this GPU. */
 uint32_t mf_auto_workers(uint32_t n);
 uint32_t mf_first_sample_rating_idx(uint32_t e, uint32_t interval, uint32_t epochs, uint32_t update_count,
                                     uint32_t update_vector_size, float sample_ratio);
@@ -381,7 +383,7 @@ typedef struct {
     float replicate_inflight; /* rows expected to have more than this many updates in flight get a copy per XCD
                                  (MF_KEEP_REPLICATED); the expectation is mf_hogwild_inflight() x the row's share of the
                                  ratings.  < 0 (default): mf_replicate_threshold(learning_rate, mean rating); 0 = no replicas */
-    uint32_t replica_merges;  /* launches per epoch when rows are replicated (default 4): their copies are averaged after each */
+    uint32_t replica_merges;  /* launches per epoch when rows are replicated: their copies are averaged after each (default 0: n / 25M, between 1 and 4) */
     float replica_add_inflight; /* > 0: replicated rows with at most this many updates in flight per XCD have their updates
                                  added to the XCD's copy (MF_KEEP_REPLICATED_ADDED) instead of stored.  Default 0: at
                                  100M ratings the extra atomic adds cost 9 ms per epoch and gain 0.0007 test RMSE */

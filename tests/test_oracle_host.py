@@ -21,7 +21,7 @@ def lib():
 
 # ---- schedules ---------------------------------------------------------------------------------
 def test_auto_workers(lib):
-    for n, want in ((1, 16), (400_000, 24), (8_000_000, 488), (100_000_000, 6104), (250_000_000, 6144)):
+    for n, want in ((1, 16), (400_000, 24), (8_000_000, 488), (90_000_000, 5496), (100_000_000, 48832), (250_000_000, 122072)):
         assert lib.mf_auto_workers(n) == want
         assert lib.mf_auto_workers(n) % 4 == 0
 
