@@ -144,3 +144,30 @@ def test_config5_full_size():
     del raw, low, u, i, r
     # nothing to learn beyond the mean (the ratings are noise around two modes): the RMSE falls from |r| to the spread
     _zero_rate_then_learning(d, 1_000_000, 625_000, 0.5)
+
+
+def test_full_size_run_tracks_the_committed_cpu_curves():
+    """mf_train -v 1 on configuration 4 at full size (the workload and parameters of bench.py and of the committed CPU
+    curves, tests/golden/reference_curve_config4_run*.json: the reference rule run by the checker on host cores) for
+    the configured 50 epochs with the library's defaults: every row update carried out, the test RMSE within 0.005 of
+    the CPU curves from epoch 12 on and at epoch 50, the figure BASELINE.json's metric names."""
+    import glob
+    import json
+    sys.path.insert(0, ROOT)
+    import bench
+    h = mfutil.hip()
+    cfg, train, test = bench.generate(h, 4, 2021, 100_000_000, 1_400_000)
+    curves = [json.load(open(f)) for f in sorted(glob.glob(os.path.join(ROOT, "tests", "golden", "reference_curve_config4_run*.json")))]
+    assert len(curves) >= 2 and all(c["n_train"] == train.size and c["n_test"] == test.size and c["seed"] == 2021 for c in curves)
+    cpu = np.mean([c["test_rmse"] for c in curves], axis=0)
+    t = bench.TRAIN
+    prm = h.default_params(k=128, num_workers=0, epoch=t["epochs"], learning_rate=t["lr"], lam=t["lam"], decay=t["decay"], version=1, seed=2021,
+                           user_group_num=t["ug"], item_group_num=t["ig"], sample_ratio=t["sample_ratio"], interval=t["interval"],
+                           error_threshold=t["threshold"])
+    assert prm.hot_row_inflight == 0                      # nothing thinned
+    p, q = h.init_model(cfg.n_users, cfg.n_items, 128, 2021)
+    gpu = h.train(prm, train, cfg.n_users, cfg.n_items, test, p, q)["rmse"]
+    print("epoch 1, 5, 12, 25, 50: gpu", np.round(gpu[[0, 4, 11, 24, 49]], 5), "cpu", np.round(cpu[[0, 4, 11, 24, 49]], 5))
+    assert np.all(np.isfinite(gpu)) and np.all(np.diff(gpu[:30]) < 0)
+    assert np.all(np.abs(gpu[11:] - cpu[11:]) < 0.005)
+    assert abs(gpu[49] - cpu[49]) < 0.002
