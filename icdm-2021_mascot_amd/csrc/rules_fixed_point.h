@@ -461,7 +461,7 @@ template <int K, bool COH> struct AfpRule : DenseBase<K, COH> {
     static constexpr int E = Base::E;
     static constexpr int J = K / 32;
     static constexpr int kAhead = 1, kRing = 4;    // as for MuPPET: three ratings ahead measured no faster (k = 128) or slower (k = 64)
-    static constexpr int kMinWavesPerSimd = 6;     // 24 wavefronts per CU: the 6104 workers of a 100M-rating launch all resident (85 VGPRs otherwise: 5)
+    static constexpr int kMinWavesPerSimd = 6;     // 24 wavefronts per CU: 6144 workers resident at a time (85 VGPRs otherwise: 5 per SIMD, 5120)
     static constexpr bool kSplittable = false;    // the per-worker quantiser state lives for one launch
     struct Params { float* p; float* q; float lrate; float lambda; int afp_epoch; int init_threshold; bool accumulate; void* rep_p; void* rep_q; };
     float lrate, lambda; int afp_epoch, init_threshold;
