@@ -162,6 +162,8 @@ def main():
     ap.add_argument("--seed", type=int, default=2021)
     ap.add_argument("--replicate", type=float, default=-1.0, help="mf_params.replicate_inflight (default: derived from learning rate and mean rating)")
     ap.add_argument("--merges", type=int, default=0, help="mf_params.replica_merges (default: the library's)")
+    ap.add_argument("--step-epochs", type=int, default=-1, help="mf_params.replica_step_epochs (default: the library's 5; 0 = every epoch)")
+    ap.add_argument("--step-scale", type=float, default=-1.0, help="mf_params.replica_step_scale (default: the library's; 0 = unscaled steps on replicated rows)")
     ap.add_argument("--thin", type=float, default=0.0, help="mf_params.hot_row_inflight: opt-in thinning of hot rows (0 = every update carried out)")
     ap.add_argument("--cpu-updates", type=int, default=32_000_000, help="size of the CPU baseline sample (about 10 s on 16 threads)")
     ap.add_argument("--skip-cpu", action="store_true")
@@ -197,6 +199,10 @@ def main():
     extra = dict(replicate_inflight=a.replicate, hot_row_inflight=a.thin, is_yahoo=yahoo)
     if a.merges:
         extra["replica_merges"] = a.merges
+    if a.step_scale >= 0:
+        extra["replica_step_scale"] = a.step_scale
+    if a.step_epochs >= 0:
+        extra["replica_step_epochs"] = a.step_epochs
     if a.pmc_copy:
         src = torch.empty(1 << 28, dtype=torch.float32, device="cuda").normal_()
         dst = torch.empty_like(src)

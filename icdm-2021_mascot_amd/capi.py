@@ -60,7 +60,10 @@ SIGNATURES = {
     "mf_session_workers": (u32, [vp]),
     "mf_session_hot_rows": (i32, [vp, vp, vp, vp]),
     "mf_session_device_state": (i32, [vp, u32, vp, vp]),
+    "mf_session_groups": (i32, [vp, i32, vp, vp, vp]),
+    "mf_session_promote_groups": (i32, [vp, i32, vp, u32]),
     "mf_replicate_threshold": (f32, [f32, f32]),
+    "mf_replica_step_scale": (f32, [f32, f32]),
     "mf_sort_by_count_workspace_bytes": (C.c_size_t, [u32]),
     "mf_sort_by_count_ws": (i32, [vp, vp, u32, vp, C.c_size_t, vp]),
     "mf_sort_by_count_static_max": (u32, []),
@@ -92,13 +95,13 @@ class MfParams(C.Structure):
                 ("interval", u32), ("user_group_num", u32), ("item_group_num", u32), ("k", u32), ("num_workers", u32),
                 ("epoch", u32), ("thread_block_size", u32), ("version", u32), ("is_yahoo", u32), ("seed", u64),
                 ("verbose", u32), ("cached_rows", u32), ("epoch_splits", u32), ("hot_row_inflight", f32), ("hot_row_inflight_early", f32), ("hot_row_early_epochs", u32),
-                ("hot_rows", u32), ("replicate_inflight", f32), ("replica_merges", u32), ("replica_add_inflight", f32)]
+                ("hot_rows", u32), ("replicate_inflight", f32), ("replica_merges", u32), ("replica_add_inflight", f32), ("replica_step_scale", f32), ("replica_step_epochs", u32)]
 
 
 class HogwildOptions(C.Structure):
     """mf_hogwild_options of include/mascot_hip.h."""
     _fields_ = [("cached_rows", u32), ("launches", u32), ("user_keep", vp), ("item_keep", vp), ("user_slot", vp), ("item_slot", vp),
-                ("user_slot_row", vp), ("item_slot_row", vp), ("user_replicas", vp), ("item_replicas", vp), ("user_slots", u32), ("item_slots", u32)]
+                ("user_slot_row", vp), ("item_slot_row", vp), ("user_replicas", vp), ("item_replicas", vp), ("user_slots", u32), ("item_slots", u32), ("replica_step_scale", f32)]
 
 
 class MfReport(C.Structure):
@@ -238,6 +241,17 @@ class Session:
         r, o = vp(), vp()
         self.h.call("mf_session_device_state", self.ptr, epoch, C.byref(r), C.byref(o))
         return r.value, o.value
+
+    def groups(self, side):
+        """(precision byte per group, training ratings per group) of side 0 (users) or 1 (items); empty without groups."""
+        cap = max(1, self.prm.item_group_num if side else self.prm.user_group_num)
+        n, prec, ratings = u32(0), np.zeros(cap, np.uint8), np.zeros(cap, np.uint64)
+        self.h.call("mf_session_groups", self.ptr, side, C.byref(n), prec.ctypes.data, ratings.ctypes.data)
+        return prec[:n.value].copy(), ratings[:n.value].copy()
+
+    def promote_groups(self, side, mask):
+        mask = np.ascontiguousarray(mask, np.uint8)
+        self.h.call("mf_session_promote_groups", self.ptr, side, mask.ctypes.data, mask.size)
 
     def finish(self):
         self.h.call("mf_session_finish", self.ptr, self.p.ctypes.data, self.q.ctypes.data)

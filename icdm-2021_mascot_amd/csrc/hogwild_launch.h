@@ -12,8 +12,10 @@ namespace mf {
 // One side's replicated rows: slot s of replica block x (x = 0..kXcds-1) is at replicas + (x * slots + s) * k * 4 bytes
 // and holds a copy of row slot_row[s] in the precision the row is stored in (a binary16 row fills the first half).
 struct ReplicaSide { RowStorage rows; uint8_t* replicas = nullptr; const uint32_t* slot_row = nullptr; uint32_t slots = 0; };
-// merge = false: every replica := the row.  merge = true: the row and every replica := the mean of the replicas.
-int replica_sync(const ReplicaSide& user, const ReplicaSide& item, int k, bool merge, void* stream);
+// merge = false: every replica := the row.  merge = true: the row and every replica := the mean of the replicas --
+// of those that differ from the row (in_play = 0), or of the in_play copies the launch's workgroups could reach,
+// untouched ones counting as the row itself (in_play > 0: the merge that goes with scaled steps, Call::step_scale).
+int replica_sync(const ReplicaSide& user, const ReplicaSide& item, int k, bool merge, void* stream, uint32_t in_play = 0);
 
 // A call's schedule (what the kernel gets) and the host-side part of its options.
 struct Call {
@@ -24,6 +26,7 @@ struct Call {
     uint8_t* rep_v = nullptr;
     const uint32_t* slot_row_u = nullptr;
     const uint32_t* slot_row_v = nullptr;
+    float step_scale = 0.f;         // mf_hogwild_options::replica_step_scale
     bool replicated() const { return s.slots_u != 0 || s.slots_v != 0; }
 };
 
@@ -44,6 +47,7 @@ static int check_schedule(const char* who, const void* R, uint32_t nnz, int k, u
         if (o->user_slots && (!o->user_slot || !o->user_slot_row || !o->user_replicas)) return invalid("%s: options: user_slots > 0 needs user_slot, user_slot_row and user_replicas", who);
         if (o->item_slots && (!o->item_slot || !o->item_slot_row || !o->item_replicas)) return invalid("%s: options: item_slots > 0 needs item_slot, item_slot_row and item_replicas", who);
         if (o->user_slots > 65535u || o->item_slots > 65535u) return invalid("%s: options: at most 65535 replicated rows per side", who);
+        if (!(o->replica_step_scale >= 0.f) || o->replica_step_scale > 64.f) return invalid("%s: options.replica_step_scale is 0 (off) or between 1 and 64", who);
         if (rep && ((reinterpret_cast<uintptr_t>(o->user_replicas) | reinterpret_cast<uintptr_t>(o->item_replicas)) & 255u))
             return invalid("%s: options: replica arrays must be 256-byte aligned", who);
     }
@@ -66,6 +70,7 @@ static Call make_call(const mf_node* R, uint32_t nnz, uint32_t num_workers, uint
         s.slot_u = o->user_slot; s.slot_v = o->item_slot; s.slots_u = o->user_slots; s.slots_v = o->item_slots;
         c.rep_u = static_cast<uint8_t*>(o->user_replicas); c.rep_v = static_cast<uint8_t*>(o->item_replicas);
         c.slot_row_u = o->user_slot_row; c.slot_row_v = o->item_slot_row;
+        c.step_scale = o->replica_step_scale;
     }
     return c;
 }
@@ -97,11 +102,20 @@ static int launch_hot(const char* who, const Call& c, const typename Rule::Param
     if (s0.update_count == 0 || s0.update_vector_size == 0 || r.begin >= r.end) return MF_OK;
     Schedule s = s0;
     typename Rule::Params prm = prm0;
-    prm.rep_p = c.rep_u; prm.rep_q = c.rep_v;
+    prm.rep_p = c.rep_u; prm.rep_q = c.rep_v; prm.rep_scale = 1.0f;
     // Replicated rows: every XCD's copy starts as the row, and after every kernel the row and the copies become the
     // mean of the copies (a kernel boundary is where the L2s of the XCDs are written back).
     ReplicaSide ru, rv;
     const bool replicated = HOT && c.replicated();
+    // Scaled steps on replicated rows (Call::step_scale > 0): a copy sees the ratings of one XCD only, and the mean of X
+    // copies moves by the X-th part of what the copies moved together, so an update of a copy takes a step that many times
+    // as long (at most step_scale, the caller's bound for a stable step) and the merge is the mean over all X copies in play.
+    uint32_t in_play = 0;
+    auto scaled_steps = [&](uint32_t workgroups) {
+        if (!replicated || !(c.step_scale > 0.f)) return;
+        in_play = workgroups < kXcds ? workgroups : kXcds;
+        prm.rep_scale = (in_play == kXcds || c.step_scale < (float)in_play) ? (c.step_scale < 1.f ? 1.f : c.step_scale) : (float)in_play;
+    };
     if (replicated) {
         Rule::row_storage(prm, ru.rows, rv.rows);
         ru.replicas = c.rep_u; ru.slot_row = c.slot_row_u; ru.slots = s0.slots_u;
@@ -125,9 +139,10 @@ static int launch_hot(const char* who, const Call& c, const typename Rule::Param
         if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&hogwild_kernel<Rule, HOT>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)r.stats_lds),
                                "hipFuncSetAttribute(MaxDynamicSharedMemorySize)")) return rc;
         set_lds_stats(prm, true);
+        scaled_steps(blocks);
         hipLaunchKernelGGL((hogwild_kernel<Rule, HOT>), dim3(blocks), dim3(kMaxBlock), r.stats_lds, as_stream(stream), s, prm);
         if (int rc = launch_status(who)) return rc;
-        return replicated ? replica_sync(ru, rv, Rule::kK, true, stream) : MF_OK;
+        return replicated ? replica_sync(ru, rv, Rule::kK, true, stream, in_play) : MF_OK;
     }
     // ordinary launches, cut into c.launches pieces on window boundaries
     uint32_t splits = Rule::kSplittable ? c.launches : 1;
@@ -135,6 +150,7 @@ static int launch_hot(const char* who, const Call& c, const typename Rule::Param
     const uint32_t windows = end_window > first_window ? end_window - first_window : 0;
     if (splits > windows) splits = windows ? windows : 1;
     bool first = true;
+    scaled_steps(grid_for(s.num_workers));
     for (uint32_t i = 0; i < splits; ++i) {
         const uint32_t b = i == 0 ? r.begin : (first_window + (uint32_t)((uint64_t)windows * i / splits)) * s0.update_vector_size;
         const uint32_t e = i + 1 == splits ? r.end : (first_window + (uint32_t)((uint64_t)windows * (i + 1) / splits)) * s0.update_vector_size;
@@ -144,7 +160,7 @@ static int launch_hot(const char* who, const Call& c, const typename Rule::Param
         first = false;
         hipLaunchKernelGGL((hogwild_kernel<Rule, HOT>), dim3(grid_for(s.num_workers)), dim3(kBlock), lds, as_stream(stream), s, prm);
         if (int rc = launch_status(who)) return rc;
-        if (replicated) { if (int rc = replica_sync(ru, rv, Rule::kK, true, stream)) return rc; }
+        if (replicated) { if (int rc = replica_sync(ru, rv, Rule::kK, true, stream, in_play)) return rc; }
     }
     return MF_OK;
 }

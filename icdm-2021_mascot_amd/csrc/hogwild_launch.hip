@@ -19,10 +19,12 @@ void set_error(const char* fmt, ...)
 // One wavefront per replicated row.  merge = 0: every XCD's copy := the row.  merge = 1: the row and every copy := the
 // mean of the copies that differ from the row (an XCD that did not touch its copy -- no workgroup of the launch ran
 // there, or none of its ratings fell on the row -- has nothing to contribute), summed in binary32 in XCD order and
-// rounded once to the row's precision; if no copy differs the row stays as it is.
+// rounded once to the row's precision; if no copy differs the row stays as it is.  With in_play > 0 the mean is taken
+// over that many copies, the ones that do not differ counting as the row: the sum of the changed copies plus
+// (in_play - changed) times the row, divided by in_play.
 struct SyncSide { RowStorage rows; uint8_t* replicas; const uint32_t* slot_row; uint32_t slots; };
 template <int K>
-__global__ __launch_bounds__(kWave) void replica_sync_kernel(SyncSide user, SyncSide item, int merge)
+__global__ __launch_bounds__(kWave) void replica_sync_kernel(SyncSide user, SyncSide item, int merge, uint32_t in_play)
 {
     constexpr int E = K / kWave;
     const bool is_item = blockIdx.x >= user.slots;
@@ -63,8 +65,12 @@ __global__ __launch_bounds__(kWave) void replica_sync_kernel(SyncSide user, Sync
             }
         }
         if (changed) {
+            const uint32_t copies = in_play > changed ? in_play : changed;
 #pragma unroll
-            for (int j = 0; j < E; ++j) { out[j] = sum[j] / (float)changed; store(master, (int)threadIdx.x + j * kWave, out[j]); }
+            for (int j = 0; j < E; ++j) {
+                if (copies > changed) sum[j] += (float)(copies - changed) * base[j];
+                out[j] = sum[j] / (float)copies; store(master, (int)threadIdx.x + j * kWave, out[j]);
+            }
         }
     }
     for (uint32_t x = 0; x < kXcds; ++x) {
@@ -72,13 +78,13 @@ __global__ __launch_bounds__(kWave) void replica_sync_kernel(SyncSide user, Sync
         for (int j = 0; j < E; ++j) store(copy_of(x), (int)threadIdx.x + j * kWave, out[j]);
     }
 }
-int replica_sync(const ReplicaSide& user, const ReplicaSide& item, int k, bool merge, void* stream)
+int replica_sync(const ReplicaSide& user, const ReplicaSide& item, int k, bool merge, void* stream, uint32_t in_play)
 {
     const uint32_t blocks = user.slots + item.slots;
     if (blocks == 0) return MF_OK;
     const SyncSide u{user.rows, user.replicas, user.slot_row, user.slots}, v{item.rows, item.replicas, item.slot_row, item.slots};
-    if (k == 128) hipLaunchKernelGGL(replica_sync_kernel<128>, dim3(blocks), dim3(kWave), 0, as_stream(stream), u, v, merge ? 1 : 0);
-    else hipLaunchKernelGGL(replica_sync_kernel<64>, dim3(blocks), dim3(kWave), 0, as_stream(stream), u, v, merge ? 1 : 0);
+    if (k == 128) hipLaunchKernelGGL(replica_sync_kernel<128>, dim3(blocks), dim3(kWave), 0, as_stream(stream), u, v, merge ? 1 : 0, in_play);
+    else hipLaunchKernelGGL(replica_sync_kernel<64>, dim3(blocks), dim3(kWave), 0, as_stream(stream), u, v, merge ? 1 : 0, in_play);
     return launch_status("replica_sync");
 }
 

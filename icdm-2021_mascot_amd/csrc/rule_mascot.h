@@ -40,6 +40,7 @@ template <int K, bool COH, bool SAMPLED> struct MascotRuleT {
         uint32_t norm_stride;     // columns per group in norm_sum_* (workgroups of an ordinary launch)
         bool lds_stats;           // sampled gradient sums are kept per workgroup in LDS and flushed once
         void* rep_p; void* rep_q; // replica rows (Schedule::slot_u): slots of kReplicaSlotBytes, a binary16 row in the first half
+        float rep_scale;          // an update of a replicated row's copy takes a step this many times as long
     };
     static constexpr uint32_t kReplicaSlotBytes = K * 4u;
     static constexpr int kK = K;
@@ -65,7 +66,8 @@ template <int K, bool COH, bool SAMPLED> struct MascotRuleT {
     float* ugrad_s; float* igrad_s;      // per-workgroup [groups][K] sums in LDS, or null
     uint32_t* ulock_s; uint32_t* ilock_s; // with them: one lock per group (add_sums_locked)
     uint32_t first_sample, user_groups, item_groups;
-    float lrate, lambda;
+    float lrate, lambda, lrate_rep;
+    uint32_t lr_h_bits, lr_rep_h_bits;     // the binary16 learning rate in both halves of a dword: ordinary step, step of a replicated row's copy
     uint64_t rep_p, rep_q;
     int lane;
     // Sampled sums of the most popular group of each side (the last one; with Zipf-like data it takes half of all
@@ -96,7 +98,8 @@ template <int K, bool COH, bool SAMPLED> struct MascotRuleT {
             iprec_s[g] = a.item_prec[g]; inorm_s[g] = 0.f;
         }
         grad_sum_p = a.grad_sum_p; grad_sum_q = a.grad_sum_q;
-        first_sample = a.first_sample; lrate = a.lrate; lambda = a.lambda;
+        first_sample = a.first_sample; lrate = a.lrate; lambda = a.lambda; lrate_rep = a.lrate * a.rep_scale;
+        lr_h_bits = bits((half_t)lrate) * 0x10001u; lr_rep_h_bits = bits((half_t)lrate_rep) * 0x10001u;
         rep_p = reinterpret_cast<uint64_t>(a.rep_p); rep_q = reinterpret_cast<uint64_t>(a.rep_q);
         for (int e = 0; e < E; ++e) { top_gp[e] = 0.f; top_gq[e] = 0.f; }
         top_np = 0.f; top_nq = 0.f;
@@ -259,6 +262,10 @@ template <int K, bool COH, bool SAMPLED> struct MascotRuleT {
     {
         if constexpr (E == 2) { HV h; h.x = (half_t)f[0]; h.y = (half_t)f[1]; return h; } else return (half_t)f[0];
     }
+    static __device__ __forceinline__ HV half_pair(uint32_t both)      // a dword with the same binary16 value in both halves
+    {
+        if constexpr (E == 2) return from_bits<half2_t>(both); else return from_bits<half_t>(both & 0xffffu);
+    }
     static __device__ __forceinline__ HV splat(half_t v)
     {
         if constexpr (E == 2) { HV h; h.x = v; h.y = v; return h; } else return v;
@@ -333,7 +340,9 @@ template <int K, bool COH, bool SAMPLED> struct MascotRuleT {
         const uint32_t ug = (i.flags >> 3) & 0x3fffu, ig = (i.flags >> 17) & 0x3fffu;
         if (!up && !ip) {
             // mascot_sgd_kernel.h:188-278: everything in binary16, one rounding per operation
-            const HV lr_h = splat((half_t)lrate), lam_h = splat((half_t)lambda);
+            const HV lam_h = splat((half_t)lambda);
+            // the step of each side: a replicated row's copy (thin bit 4 / 5) takes the longer one
+            const HV lr_p = half_pair((HOT && (i.thin & 16u)) ? lr_rep_h_bits : lr_h_bits), lr_q = half_pair((HOT && (i.thin & 32u)) ? lr_rep_h_bits : lr_h_bits);
             const half_t r_h = (half_t)i.r;
             const HV P = from_bits<HV>(row.p[0]), Q = from_bits<HV>(row.q[0]);
             const half_t dot = dot_half(P * Q);
@@ -341,14 +350,14 @@ template <int K, bool COH, bool SAMPLED> struct MascotRuleT {
             const HV gp = ruv * Q - lam_h * P;
             const HV gq = ruv * P - lam_h * Q;
             if (!(i.thin & 1u)) {
-                row.p[0] = bits(HV(__builtin_elementwise_fma(lr_h, gp, P)));
+                row.p[0] = bits(HV(__builtin_elementwise_fma(lr_p, gp, P)));
                 if ((i.thin & 20u) == 16u) store_side<false>(row.p, i.pptr, false, lane);
-                else if (i.thin & 4u) add_side_half(i.pptr, lr_h * gp, lane); else store_side(row.p, i.pptr, false, lane);
+                else if (i.thin & 4u) add_side_half(i.pptr, lr_p * gp, lane); else store_side(row.p, i.pptr, false, lane);
             }
             if (!(i.thin & 2u)) {
-                row.q[0] = bits(HV(__builtin_elementwise_fma(lr_h, gq, Q)));
+                row.q[0] = bits(HV(__builtin_elementwise_fma(lr_q, gq, Q)));
                 if ((i.thin & 40u) == 32u) store_side<false>(row.q, i.qptr, false, lane);
-                else if (i.thin & 8u) add_side_half(i.qptr, lr_h * gq, lane); else store_side(row.q, i.qptr, false, lane);
+                else if (i.thin & 8u) add_side_half(i.qptr, lr_q * gq, lane); else store_side(row.q, i.qptr, false, lane);
             }
             if (sampled) {
                 float g[E];
@@ -368,13 +377,14 @@ template <int K, bool COH, bool SAMPLED> struct MascotRuleT {
 #pragma unroll
             for (int e = 0; e < E; ++e) m[e] = pf[e] * qf[e];
             const float ruv = i.r - dot_float(m);
+            const float lr_p = (HOT && (i.thin & 16u)) ? lrate_rep : lrate, lr_q = (HOT && (i.thin & 32u)) ? lrate_rep : lrate;
             float gp[E], gq[E], np_[E], nq_[E];
 #pragma unroll
             for (int e = 0; e < E; ++e) {
                 gp[e] = ruv * qf[e] - lambda * pf[e];
                 gq[e] = ruv * pf[e] - lambda * qf[e];
-                np_[e] = __builtin_fmaf(lrate, gp[e], pf[e]);
-                nq_[e] = __builtin_fmaf(lrate, gq[e], qf[e]);
+                np_[e] = __builtin_fmaf(lr_p, gp[e], pf[e]);
+                nq_[e] = __builtin_fmaf(lr_q, gq[e], qf[e]);
             }
             if (!(i.thin & 1u)) {
                 if (up) { for (int e = 0; e < E; ++e) row.p[e] = bits(np_[e]); }
@@ -382,7 +392,7 @@ template <int K, bool COH, bool SAMPLED> struct MascotRuleT {
                 if ((i.thin & 20u) == 16u) store_side<false>(row.p, i.pptr, up, lane);
                 else if (i.thin & 4u) {
                     float d[E];
-                    for (int e = 0; e < E; ++e) d[e] = lrate * gp[e];
+                    for (int e = 0; e < E; ++e) d[e] = lr_p * gp[e];
                     if (up) add_side_float(i.pptr, d, lane); else add_side_half(i.pptr, narrow(d), lane);
                 } else store_side(row.p, i.pptr, up, lane);
             }
@@ -392,7 +402,7 @@ template <int K, bool COH, bool SAMPLED> struct MascotRuleT {
                 if ((i.thin & 40u) == 32u) store_side<false>(row.q, i.qptr, ip, lane);
                 else if (i.thin & 8u) {
                     float d[E];
-                    for (int e = 0; e < E; ++e) d[e] = lrate * gq[e];
+                    for (int e = 0; e < E; ++e) d[e] = lr_q * gq[e];
                     if (ip) add_side_float(i.qptr, d, lane); else add_side_half(i.qptr, narrow(d), lane);
                 } else store_side(row.q, i.qptr, ip, lane);
             }

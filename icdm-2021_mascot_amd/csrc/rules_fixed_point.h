@@ -227,7 +227,7 @@ template <int K, bool COH> struct MuppetRule : DenseBase<K, COH> {
     struct Params {
         float* p; float* q; float lrate; float lambda; uint32_t first_sample;
         float* sum_updated_val; float* sum_norms; uint32_t num_workers; int fwd; int bwd; bool accumulate;
-        void* rep_p; void* rep_q;
+        void* rep_p; void* rep_q; float rep_scale;
     };
     static constexpr bool kSplittable = false;     // per-worker statistics span the whole launch
     float lrate, lambda; uint32_t first_sample; float* sum_updated_val; int fwd, bwd;
@@ -242,7 +242,7 @@ template <int K, bool COH> struct MuppetRule : DenseBase<K, COH> {
     __device__ __forceinline__ void init(const Params& a, uint8_t*, int lane_, uint32_t)
     {
         this->P = a.p; this->Q = a.q; this->RP = static_cast<float*>(a.rep_p); this->RQ = static_cast<float*>(a.rep_q);
-        this->lane = lane_; lrate = a.lrate; lambda = a.lambda;
+        this->lane = lane_; lrate = a.lrate; lambda = a.lambda; this->rep_scale = a.rep_scale;
         first_sample = a.first_sample; sum_updated_val = a.sum_updated_val; fwd = a.fwd; bwd = a.bwd;
         sum_norms_reg = 0.f;
 #pragma unroll
@@ -393,11 +393,13 @@ template <int K, bool COH> struct MuppetRule : DenseBase<K, COH> {
         float gbp[E], gbq[E], g_scale, d_scale;
         if (!(plain_8bit && gradients_8bit_plain(row.p, row.q, i.r, gbp, gbq, g_scale, d_scale)))
             gradients(row.p, row.q, i.r, gbp, gbq, g_scale, d_scale);
+        // d_scale carries the learning rate: a replicated row's copy takes a longer step (DenseBase::rep_scale)
+        const float ds_p = HOT ? this->step_of(d_scale, i.thin, 16u) : d_scale, ds_q = HOT ? this->step_of(d_scale, i.thin, 32u) : d_scale;
         float dp[E], dq[E];
 #pragma unroll
         for (int e = 0; e < E; ++e) {
-            dp[e] = d_scale * gbp[e];
-            dq[e] = d_scale * gbq[e];
+            dp[e] = ds_p * gbp[e];
+            dq[e] = ds_q * gbq[e];
             row.p[e] = (i.thin & 1u) ? row.p[e] : row.p[e] + dp[e];
             row.q[e] = (i.thin & 2u) ? row.q[e] : row.q[e] + dq[e];
         }
@@ -463,7 +465,7 @@ template <int K, bool COH> struct AfpRule : DenseBase<K, COH> {
     static constexpr int kAhead = 1, kRing = 4;    // as for MuPPET: three ratings ahead measured no faster (k = 128) or slower (k = 64)
     static constexpr int kMinWavesPerSimd = 6;     // 24 wavefronts per CU: 6144 workers resident at a time (85 VGPRs otherwise: 5 per SIMD, 5120)
     static constexpr bool kSplittable = false;    // the per-worker quantiser state lives for one launch
-    struct Params { float* p; float* q; float lrate; float lambda; int afp_epoch; int init_threshold; bool accumulate; void* rep_p; void* rep_q; };
+    struct Params { float* p; float* q; float lrate; float lambda; int afp_epoch; int init_threshold; bool accumulate; void* rep_p; void* rep_q; float rep_scale; };
     float lrate, lambda; int afp_epoch, init_threshold;
     AfpQ uq, iq, bq;
     int upd_u, upd_i, upd_b, cur_iter;
@@ -480,7 +482,7 @@ template <int K, bool COH> struct AfpRule : DenseBase<K, COH> {
     __device__ __forceinline__ void init(const Params& a, uint8_t*, int lane_, uint32_t)
     {
         this->P = a.p; this->Q = a.q; this->RP = static_cast<float*>(a.rep_p); this->RQ = static_cast<float*>(a.rep_q);
-        this->lane = lane_; lrate = a.lrate; lambda = a.lambda;
+        this->lane = lane_; lrate = a.lrate; lambda = a.lambda; this->rep_scale = a.rep_scale;
         afp_epoch = a.afp_epoch; init_threshold = a.init_threshold;
         uq = AfpQ{0, 0, 0, 0.f}; iq = uq; bq = uq;
         upd_u = upd_i = upd_b = cur_iter = 0; sp = sq = sb = 0.f; upper = lane_ >= 32;
@@ -616,11 +618,13 @@ template <int K, bool COH> struct AfpRule : DenseBase<K, COH> {
                 gbq[e] = (float)(half_t)(ph * t_ruv + qh * t_lam16);
             }
         }
+        // d_scale carries the learning rate: a replicated row's copy takes a longer step (DenseBase::rep_scale)
+        const float ds_p = HOT ? this->step_of(d_scale, i.thin, 16u) : d_scale, ds_q = HOT ? this->step_of(d_scale, i.thin, 32u) : d_scale;
         float dp[E], dq[E];
 #pragma unroll
         for (int e = 0; e < E; ++e) {
-            dp[e] = d_scale * gbp[e];
-            dq[e] = d_scale * gbq[e];
+            dp[e] = ds_p * gbp[e];
+            dq[e] = ds_q * gbq[e];
             row.p[e] = (i.thin & 1u) ? row.p[e] : row.p[e] + dp[e];
             row.q[e] = (i.thin & 2u) ? row.q[e] : row.q[e] + dq[e];
         }

@@ -30,7 +30,10 @@ template <int K, bool COH> struct DenseBase {
     float* Q;
     float* RP;      // replica rows (Schedule::slot_u), or null
     float* RQ;
+    float rep_scale;   // an update of a replicated row's copy takes a step this many times as long (Params::rep_scale)
     int lane;
+    // the step factor of one side of a rating: bit = 16 (user row) or 32 (item row) of Info::thin marks a replicated row
+    __device__ __forceinline__ float step_of(float lrate, uint32_t thin, uint32_t bit) const { return (thin & bit) ? lrate * rep_scale : lrate; }
 
     __device__ __forceinline__ Prep prepare(const Rating&, bool) const { return Prep(); }
     __device__ __forceinline__ int classify(const Prep&, bool) const { return 0; }
@@ -135,13 +138,13 @@ template <int K, bool COH> struct SgdRule : DenseBase<K, COH> {
     static constexpr int E = Base::E;
     static constexpr int kAhead = 3, kRing = 8;
     static constexpr bool kSplittable = true;
-    struct Params { float* p; float* q; float lrate; float lambda; bool accumulate; void* rep_p; void* rep_q; };
+    struct Params { float* p; float* q; float lrate; float lambda; bool accumulate; void* rep_p; void* rep_q; float rep_scale; };
     float lrate, lambda;
 
     __device__ __forceinline__ void init(const Params& a, uint8_t*, int lane_, uint32_t)
     {
         this->P = a.p; this->Q = a.q; this->RP = static_cast<float*>(a.rep_p); this->RQ = static_cast<float*>(a.rep_q);
-        this->lane = lane_; lrate = a.lrate; lambda = a.lambda;
+        this->lane = lane_; lrate = a.lrate; lambda = a.lambda; this->rep_scale = a.rep_scale;
     }
     template <int CLS, bool HOT> __device__ __forceinline__ void update(Row& row, const Info& i, uint32_t) const
     {
@@ -150,12 +153,13 @@ template <int K, bool COH> struct SgdRule : DenseBase<K, COH> {
         for (int e = 0; e < E; ++e) m[e] = row.p[e] * row.q[e];
         const float dot = dot_reference_order<E, float>(m);
         const float ruv = i.r - dot;
+        const float lr_p = HOT ? this->step_of(lrate, i.thin, 16u) : lrate, lr_q = HOT ? this->step_of(lrate, i.thin, 32u) : lrate;
         float dp[E], dq[E];
 #pragma unroll
         for (int e = 0; e < E; ++e) {
             const float pe = row.p[e], qe = row.q[e];
-            dp[e] = lrate * (ruv * qe - lambda * pe);
-            dq[e] = lrate * (ruv * pe - lambda * qe);
+            dp[e] = lr_p * (ruv * qe - lambda * pe);
+            dq[e] = lr_q * (ruv * pe - lambda * qe);
             row.p[e] = (i.thin & 1u) ? pe : pe + dp[e];
             row.q[e] = (i.thin & 2u) ? qe : qe + dq[e];
         }
@@ -172,14 +176,14 @@ template <int K, bool COH> struct MptRule : DenseBase<K, COH> {
     static constexpr int E = Base::E;
     static constexpr int kAhead = 3, kRing = 8;
     static constexpr bool kSplittable = true;
-    struct Params { float* p; float* q; float lrate; uint16_t scaled_lambda_half; float scaling_factor; bool accumulate; void* rep_p; void* rep_q; };
+    struct Params { float* p; float* q; float lrate; uint16_t scaled_lambda_half; float scaling_factor; bool accumulate; void* rep_p; void* rep_q; float rep_scale; };
     float lrate, scaling_factor_rev;
     half_t lambda_h, scaling_factor_h;
 
     __device__ __forceinline__ void init(const Params& a, uint8_t*, int lane_, uint32_t)
     {
         this->P = a.p; this->Q = a.q; this->RP = static_cast<float*>(a.rep_p); this->RQ = static_cast<float*>(a.rep_q);
-        this->lane = lane_; lrate = a.lrate;
+        this->lane = lane_; lrate = a.lrate; this->rep_scale = a.rep_scale;
         scaling_factor_rev = 1 / a.scaling_factor;
         scaling_factor_h = (half_t)a.scaling_factor;
         lambda_h = from_bits<half_t>(a.scaled_lambda_half);
@@ -192,13 +196,14 @@ template <int K, bool COH> struct MptRule : DenseBase<K, COH> {
         for (int e = 0; e < E; ++e) { ph[e] = (half_t)row.p[e]; qh[e] = (half_t)row.q[e]; m[e] = ph[e] * qh[e]; }
         const half_t dot = dot_reference_order<E, half_t>(m);
         const half_t ruv = scaling_factor_h * (r_h - dot);
+        const float lr_p = HOT ? this->step_of(lrate, i.thin, 16u) : lrate, lr_q = HOT ? this->step_of(lrate, i.thin, 32u) : lrate;
         float dp[E], dq[E];
 #pragma unroll
         for (int e = 0; e < E; ++e) {
             const half_t gp = ruv * qh[e] - lambda_h * ph[e];
             const half_t gq = ruv * ph[e] - lambda_h * qh[e];
-            dp[e] = lrate * (scaling_factor_rev * (float)gp);
-            dq[e] = lrate * (scaling_factor_rev * (float)gq);
+            dp[e] = lr_p * (scaling_factor_rev * (float)gp);
+            dq[e] = lr_q * (scaling_factor_rev * (float)gq);
             row.p[e] = (i.thin & 1u) ? row.p[e] : row.p[e] + dp[e];
             row.q[e] = (i.thin & 2u) ? row.q[e] : row.q[e] + dq[e];
         }
@@ -221,12 +226,13 @@ template <int K, bool COH> struct MemQuantRule {
     static constexpr int kClasses = 1;
     static constexpr int kAhead = 3, kRing = 8;
     static constexpr bool kSplittable = true;
-    struct Params { uint16_t* p; uint16_t* q; float lrate; float lambda; bool accumulate; void* rep_p; void* rep_q; };
-    uint16_t* P; uint16_t* Q; uint16_t* RP; uint16_t* RQ; float lrate, lambda; int lane;
+    struct Params { uint16_t* p; uint16_t* q; float lrate; float lambda; bool accumulate; void* rep_p; void* rep_q; float rep_scale; };
+    uint16_t* P; uint16_t* Q; uint16_t* RP; uint16_t* RQ; float lrate, lambda, rep_scale; int lane;
 
     __device__ __forceinline__ void init(const Params& a, uint8_t*, int lane_, uint32_t)
     {
         P = a.p; Q = a.q; RP = static_cast<uint16_t*>(a.rep_p); RQ = static_cast<uint16_t*>(a.rep_q); lrate = a.lrate; lambda = a.lambda; lane = lane_;
+        rep_scale = a.rep_scale;
     }
     // a replica slot is k * 4 bytes for every rule; a binary16 row fills its first half
     static __device__ __forceinline__ uint16_t* row_of(uint16_t* matrix, uint16_t* replicas, uint32_t row)
@@ -318,11 +324,13 @@ template <int K, bool COH> struct MemQuantRule {
             dot = dot_rows_in_order(pf[0] * qf[0], pf[1] * qf[1]);
         }
         const float ruv = i.r - dot;
+        // a replicated row's copy takes a longer step (Params::rep_scale)
+        const float lr_p = (HOT && (i.thin & 16u)) ? lrate * rep_scale : lrate, lr_q = (HOT && (i.thin & 32u)) ? lrate * rep_scale : lrate;
         float dp[E], dq[E], np[E], nq[E];
 #pragma unroll
         for (int e = 0; e < E; ++e) {
-            dp[e] = lrate * (ruv * qf[e] - lambda * pf[e]);
-            dq[e] = lrate * (ruv * pf[e] - lambda * qf[e]);
+            dp[e] = lr_p * (ruv * qf[e] - lambda * pf[e]);
+            dq[e] = lr_q * (ruv * pf[e] - lambda * qf[e]);
             np[e] = pf[e] + dp[e];
             nq[e] = qf[e] + dq[e];
         }

@@ -77,7 +77,15 @@ const char* mf_last_error(void);
  * user_replicas, item_replicas   caller-owned scratch of MF_XCDS * slots * k * 4 bytes, 256-byte aligned; slot s of
  *               XCD x is at (x * slots + s) * k * 4 and holds the row in the precision it is stored in.  Filled from
  *               the rows at the start of every call; nothing is kept in it between calls.
- * user_slots, item_slots   replicated rows per side (at most 65535; 0 = none) */
+ * user_slots, item_slots   replicated rows per side (at most 65535; 0 = none)
+ * replica_step_scale   0 (default): a copy of a replicated row is updated like any row, and the merge takes the mean of
+ *               the copies that changed.  >= 1: scaled steps.  A copy sees the ratings of one XCD only, and the mean of X
+ *               copies moves by the X-th part of what the copies moved together; so an update of a copy takes a step
+ *               replica_step_scale times as long (at most X when X < MF_XCDS) (the learning rate of that side of the rating is multiplied), and
+ *               the merge is the mean over the X = min(MF_XCDS, workgroups of the launch) copies in play, untouched ones
+ *               counting as the row.  With X = 1 (a launch of one workgroup) nothing changes.  The caller bounds the
+ *               factor by what keeps a single step stable: factor x learning rate x |other side's row|^2 well below 2
+ *               (mf_replica_step_scale). */
 #define MF_KEEP_ORDINARY 255
 #define MF_KEEP_ADDED 254
 #define MF_KEEP_REPLICATED 253
@@ -95,6 +103,7 @@ typedef struct {
     void* user_replicas;
     void* item_replicas;
     uint32_t user_slots, item_slots;
+    float replica_step_scale;
 } mf_hogwild_options;
 /* What the update calls do with replicated rows before and after every kernel launch, for a dense matrix [rows][k] of
  * elem_bytes-wide elements (2: binary16, 4: binary32): merge = 0 copies row slot_row[s] into slot s of every XCD's
@@ -387,6 +396,12 @@ typedef struct {
     float replica_add_inflight; /* > 0: replicated rows with at most this many updates in flight per XCD have their updates
                                  added to the XCD's copy (MF_KEEP_REPLICATED_ADDED) instead of stored.  Default 0: at
                                  100M ratings the extra atomic adds cost 9 ms per epoch and gain 0.0007 test RMSE */
+    float replica_step_scale; /* mf_hogwild_options::replica_step_scale.  < 0 (default): mf_replica_step_scale(learning_rate,
+                                 mean rating); 0 = off (unscaled steps, mean of the changed copies) */
+    uint32_t replica_step_epochs; /* the first epochs that use replica_step_scale; later ones run unscaled (default 1: the
+                                 epoch in which every row grows from its small initial value and a replicated row, which
+                                 keeps one of the many updates in flight on a copy, is furthest behind; afterwards the
+                                 unscaled mean of eight copies is the less noisy estimate.  0 = every epoch) */
 } mf_params;
 
 /* What a run reports back; every pointer is optional host memory owned by the caller. */
@@ -441,10 +456,26 @@ int mf_session_hot_rows(const mf_session* session, uint32_t* user_replicated, ui
  * its update calls of `epoch` use; both stay owned by the session and valid until mf_session_destroy.  For
  * measurements that replay the session's memory traffic (mf_row_traffic_probe). */
 int mf_session_device_state(const mf_session* session, uint32_t epoch, const mf_node** ratings, const mf_hogwild_options** options);
+/* The groups of one side of a MASCOT session (side 0: users, 1: items; no counterpart in the reference, which prints
+ * its group tables): *groups = their number (0 for the versions without groups), prec[g] = 1 where group g is held in
+ * binary32 now (precision_switching.h:8-51 has promoted it), ratings[g] = training ratings that fall on the group's
+ * rows.  prec and ratings are optional host arrays of at least the requested group count (mf_params.user_group_num /
+ * item_group_num).  An update touches one user row and one item row, so the bytes an epoch moves follow from these
+ * two tables: 12 + 2 k (2 or 4) bytes per side and rating. */
+int mf_session_groups(const mf_session* session, int side, uint32_t* groups, uint8_t* prec, uint64_t* ratings);
+/* Promotes the groups g with mask[g] != 0 of one side to binary32 now, as the precision switching does when a group's
+ * error exceeds the threshold (precision_switching.h:8-51: exact widening, pointer and precision tables refreshed);
+ * groups that are binary32 already stay.  `groups` must equal the side's group count.  For measurements of epochs
+ * after switching; waits for the device. */
+int mf_session_promote_groups(mf_session* session, int side, const uint8_t* mask, uint32_t groups);
 /* Above how many updates in flight mf_train replicates a row when mf_params.replicate_inflight < 0 (the default):
  * 0.3 / (learning_rate * mean |rating|), between 2 and 16.  Added updates of one row that are in flight together sum
  * gradients taken at the same stale row; the sum stays a contraction while their number x lr x mean rating < 2. */
 float mf_replicate_threshold(float learning_rate, float mean_rating);
+/* The step factor mf_train gives the copies of replicated rows when mf_params.replica_step_scale < 0 (the default):
+ * 0.15 / (learning_rate * mean |rating|), half the bound above, between 1 and MF_XCDS (4.3 for learning rate 0.01 and
+ * ratings around 3.5; measured there: 8 still converges, 12 diverges in the first epoch). */
+float mf_replica_step_scale(float learning_rate, float mean_rating);
 /* Host grouping, split_group_based_equal_size_not_strict_ret_end_idx, preprocess_utils.h:101-190:
  * sorted_cnt ascending rating counts; writes inclusive end indices (capacity n) and returns their number. */
 uint32_t mf_group_end_indices(const uint32_t* sorted_cnt, uint32_t n, uint32_t requested_groups, uint32_t* end_idx_out);

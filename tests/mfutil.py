@@ -89,11 +89,11 @@ class HogwildOptions:
     """mf_hogwild_options over numpy keep tables (device copies are kept alive by the object).  Rows whose keep value
     is 253 or 252 (MF_KEEP_REPLICATED, MF_KEEP_REPLICATED_ADDED) get replica slots in row order."""
 
-    def __init__(self, k, keep_u=None, keep_v=None, cached_rows=0, launches=1):
+    def __init__(self, k, keep_u=None, keep_v=None, cached_rows=0, launches=1, step_scale=0.0):
         import torch
         capi = importlib.import_module("icdm-2021_mascot_amd.capi")
         self.o = o = capi.HogwildOptions()
-        o.cached_rows, o.launches = cached_rows, launches
+        o.cached_rows, o.launches, o.replica_step_scale = cached_rows, launches, step_scale
         self.keep = []
         self.replicas = [None, None]
         self.slot_rows = [np.zeros(0, np.uint32), np.zeros(0, np.uint32)]
@@ -176,7 +176,7 @@ def test_set_order(test):
     return np.ascontiguousarray(t[last])
 
 
-def oracle_train_dense(orc, version, R, test, P, Q, k, W, epochs, lr, lam, decay, seed, threads=8, sample_ratio=0.01, sequential_threads=1):
+def oracle_train_dense(orc, version, R, test, P, Q, k, W, epochs, lr, lam, decay, seed, threads=8, sample_ratio=0.01, sequential_threads=1, progress=None):
     """training_single_mf / mixed_precision_training_mf / muppet_training_mf / adaptive_fixed_point_training_mf
     (mf_methods.cu:820-924, 713-818, 529-711, 436-527) on the CPU; returns per-epoch test RMSE.  MuPPET and AFP run one
     worker after another (what the bit-exact single-worker tests need) unless sequential_threads > 1 lets host threads race."""
@@ -210,6 +210,8 @@ def oracle_train_dense(orc, version, R, test, P, Q, k, W, epochs, lr, lam, decay
         elif version == 2:
             orc.lib.orc_afp_epoch(k, Rs.ctypes.data, Rs.size, P.ctypes.data, Q.ctypes.data, W, uc, 128, lre, lam, e, seed, e, None, sequential_threads)
         rmse.append(orc.rmse(k, test, P, Q))
+        if progress is not None:
+            progress(e, rmse[-1])
     return np.array(rmse), dict(final_bits=bits_ladder[min(pidx_c.value, 4)], bits=np.array(bits_hist, np.uint8))
 
 
@@ -289,7 +291,7 @@ def oracle_train_mascot(orc, R, test, P, Q, k, W, epochs, lr, lam, decay, seed, 
     gi = host_grouped(orc, k, Qs, iend, np.zeros(iend.size, np.uint8))
     uc = orc.lib.orc_update_count(Rs.size, W, 128)
     init_u, init_i = np.ones(uend.size, np.float32), np.ones(iend.size, np.float32)
-    rmse, switches = [], []
+    rmse, switches, switched_per_epoch = [], [], []
     for e in range(epochs):
         lre = orc.lib.orc_lr_schedule(lr, decay, e)
         first = orc.lib.orc_first_sample_rating_idx(e, interval, epochs, uc, 128, sample_ratio)
@@ -315,9 +317,10 @@ def oracle_train_mascot(orc, R, test, P, Q, k, W, epochs, lr, lam, decay, seed, 
             switches.append((e, eu.copy(), ei.copy()))
         rmse.append(orc.lib.orc_rmse_grouped(k, test.ctypes.data, test.size, gu.ptrs, gi.ptrs, gu.end_idx.ctypes.data, gi.end_idx.ctypes.data,
                                              gu.prec.ctypes.data, gi.prec.ctypes.data, gu.groups, gi.groups))
+        switched_per_epoch.append((int(gu.prec.sum()), int(gi.prec.sum())))      # groups in binary32 after this epoch
         if progress is not None:
             progress(e, rmse[-1])
-    return np.array(rmse), dict(gu=gu, gi=gi, uend=uend, iend=iend, u2s=u2s, i2s=i2s, test=test, errors=switches)
+    return np.array(rmse), dict(gu=gu, gi=gi, uend=uend, iend=iend, u2s=u2s, i2s=i2s, test=test, errors=switches, switched_per_epoch=switched_per_epoch)
 
 
 # ---- device-resident MASCOT state built with the library's own pre-processing kernels ------------------------------
