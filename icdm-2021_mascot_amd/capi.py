@@ -101,7 +101,7 @@ class MfParams(C.Structure):
 class HogwildOptions(C.Structure):
     """mf_hogwild_options of include/mascot_hip.h."""
     _fields_ = [("cached_rows", u32), ("launches", u32), ("user_keep", vp), ("item_keep", vp), ("user_slot", vp), ("item_slot", vp),
-                ("user_slot_row", vp), ("item_slot_row", vp), ("user_replicas", vp), ("item_replicas", vp), ("user_slots", u32), ("item_slots", u32), ("replica_step_scale", f32)]
+                ("user_slot_row", vp), ("item_slot_row", vp), ("user_replicas", vp), ("item_replicas", vp), ("user_slots", u32), ("item_slots", u32), ("replica_step_scale", f32), ("all_binary16", u32)]
 
 
 class MfReport(C.Structure):

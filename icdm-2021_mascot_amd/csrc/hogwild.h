@@ -195,7 +195,7 @@ void hogwild_kernel(Schedule s, typename Rule::Params prm)
             }
             const bool valid = lane < n;
             typename Rule::Prep prep = rule.prepare(my, valid);
-            const int cls = rule.classify(prep, valid);
+            const int cls = rule.classify(my, prep, valid);
             // classes (see the rules): 1 and 2 promise ratings that all take the same memory instructions; full
             // chunks of those run the straight-line pipeline, everything else the general one
             if (Rule::kClasses > 1 && cls == 1) {

@@ -1,5 +1,6 @@
-// The MASCOT launcher in three translation units: the entry point (launch_mascot.hip) and the kernels with and without
-// the sampled-statistics code (launch_mascot_sampled.hip, launch_mascot_plain.hip), which compile side by side.
+// The MASCOT launcher in four translation units: the entry point (launch_mascot.hip) and the kernels with and without
+// the sampled-statistics code (launch_mascot_sampled.hip, launch_mascot_plain.hip) and for runs whose groups are all
+// binary16 (launch_mascot_binary16.hip), which compile side by side.
 #pragma once
 #include "hogwild_launch.h"
 
@@ -25,6 +26,7 @@ struct MascotCall {
     }
 };
 int launch_mascot_plain(const MascotCall& c, Range r);        // hogwild_kernel<MascotPlainRule<k, coh>, hot>
+int launch_mascot_binary16(const MascotCall& c, Range r);     // hogwild_kernel<MascotBinary16Rule<k, coh>, hot>
 int launch_mascot_sampled(const MascotCall& c, Range r);      // hogwild_kernel<MascotRule<k, coh>, hot>
 size_t mascot_table_lds_bytes(uint32_t user_groups, uint32_t item_groups);
 

@@ -33,15 +33,19 @@ int mf_mascot_sgd_hogwild_opt(const mf_node* R, uint32_t nnz, void* const* p, vo
     c.lrate = lrate; c.lambda = lambda; c.norm_stride = grid_for(num_workers);
     const uint32_t total = c.c.s.range_end;
     Range body = whole_epoch(c.c);
-    if (first_sample_rating_idx >= total)                     // nothing is sampled: the kernel without the statistics code
-        return launch_mascot_plain(c, body);
+    // the unsampled part of an epoch: the kernel without the statistics code, in the build for all-binary16 runs if the
+    // caller says that is what this is
+    const bool binary16 = options && options->all_binary16;
+    auto plain = [&](const Range& r) { return binary16 ? launch_mascot_binary16(c, r) : launch_mascot_plain(c, r); };
+    if (first_sample_rating_idx >= total)                     // nothing is sampled
+        return plain(body);
     // A check epoch.  The sampled ratings [first_sample, total) run as their own launch with the gradient sums in
     // LDS when those fit (160 KB per workgroup); otherwise the whole epoch runs with the sums in global memory.
     const size_t need = lds + (size_t)(user_group_num + item_group_num) * ((size_t)k + 1) * sizeof(float);      // sums and one lock per group
     if (need > 160 * 1024) return launch_mascot_sampled(c, body);
     body.end = first_sample_rating_idx;
     // the body still writes the (zero) norm sums of its workgroups, which the sampled launch then adds to
-    if (int rc = launch_mascot_plain(c, body)) return rc;
+    if (int rc = plain(body)) return rc;
     Range tail;
     tail.begin = first_sample_rating_idx; tail.end = total; tail.accumulate = body.begin < body.end; tail.stats_lds = need;
     return launch_mascot_sampled(c, tail);

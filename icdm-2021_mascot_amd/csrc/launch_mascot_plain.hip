@@ -8,10 +8,6 @@ int launch_mascot_plain(const MascotCall& c, Range r)
 {
     return launch_k_coh<MascotPlainRule>(c.who, c.k, c.c, [&](auto a) { return c.fill(a); }, c.lds, c.stream, r);
 }
-float inflight_mascot(int k, uint32_t num_workers, uint32_t user_groups, uint32_t item_groups)
-{
-    return inflight_updates<MascotPlainRule>(k, num_workers, MascotRule<128, true>::lds_bytes(user_groups, item_groups));
-}
 size_t mascot_table_lds_bytes(uint32_t user_groups, uint32_t item_groups) { return MascotRule<128, true>::lds_bytes(user_groups, item_groups); }
 
 }  // namespace mf

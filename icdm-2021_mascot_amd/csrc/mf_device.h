@@ -154,6 +154,16 @@ template <bool COH> __device__ __forceinline__ void window_store(row_window_t w,
     __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(uint2_t, v), w, (int)byte_offset, 0, COH ? 16 : 0);
 }
 
+// Adds through a row window (row_add's instructions in their buffer form: dropped when the window is closed).
+__device__ __forceinline__ void window_add(row_window_t w, uint32_t byte_offset, float d)
+{
+    (void)__builtin_amdgcn_raw_ptr_buffer_atomic_fadd_f32(d, w, (int)byte_offset, 0, 0);
+}
+__device__ __forceinline__ void window_add(row_window_t w, uint32_t byte_offset, half2_t d)
+{
+    (void)__builtin_amdgcn_raw_ptr_buffer_atomic_fadd_v2f16(d, w, (int)byte_offset, 0, 0);
+}
+
 // ---- counter-based generator -----------------------------------------------------------
 __host__ __device__ __forceinline__ uint64_t mix64(uint64_t z)
 {

@@ -20,14 +20,20 @@
 namespace mf {
 
 // SAMPLED = false compiles the sampled-statistics code out: the kernel for launches in which no rating is sampled.
-template <int K, bool COH, bool SAMPLED> struct MascotRuleT {
+// MIXED = false compiles the straight-line path for chunks of mixed precisions out (such chunks take the general path,
+// so the results are the same): the kernel for runs in which every group is still binary16, which then keeps the
+// registers of the binary16 path alone and with them one more resident wavefront per SIMD.
+template <int K, bool COH, bool SAMPLED, bool MIXED = true> struct MascotRuleT {
     static constexpr int E = K / 64;                        // elements per lane
     static constexpr int kAhead = 3, kRing = 8;
     // chunk classes: 1 = every rating of the chunk touches two binary16 rows (the state every group starts in): loads
     // and arithmetic without any branching; 2 = any mix of precisions, every rating inside the group tables: every
     // path through a rating issues the same number of memory instructions; 0 = anything, including ratings that are
     // skipped (an index outside the tables)
-    static constexpr int kClasses = 3;
+    static constexpr int kClasses = MIXED ? 3 : 2;
+    // the build for all-binary16 runs asks for six wavefronts per SIMD (80 registers): its hot loop needs fewer, the
+    // general path for mixed chunks, which it should never take, is what would exceed them
+    static constexpr int kMinWavesPerSimd = 1;
     using HV = typename std::conditional<E == 2, half2_t, half_t>::type;
 
     struct Params {
@@ -50,8 +56,9 @@ template <int K, bool COH, bool SAMPLED> struct MascotRuleT {
         v.group_ptr = a.q; v.group_end = a.item_end; v.group_prec = a.item_prec; v.groups = a.item_groups;
     }
     static constexpr bool kSplittable = true;
-    // raw row registers: binary16 rows use r[0] only
-    struct Row { uint32_t p[E], q[E]; };
+    // raw row registers: binary16 rows use r[0] only.  ph, qh: chunks of mixed precisions load a binary16 row into these
+    // and a binary32 row into p, q (load_mixed); whichever the row is not comes back as zero
+    struct Row { uint32_t p[E], q[E], ph, qh; };
     struct Prep { uint64_t pptr, qptr; uint32_t flags; };
     struct Info { float r; uint64_t pptr, qptr; uint32_t flags, thin; };
     // flags: bit0 user row is fp32, bit1 item row is fp32, bit2 rating is skipped (index outside the
@@ -144,10 +151,11 @@ template <int K, bool COH, bool SAMPLED> struct MascotRuleT {
         }
         return pr;
     }
-    __device__ __forceinline__ int classify(const Prep& pr, bool valid) const
+    __device__ __forceinline__ int classify(const Rating& my, const Prep& pr, bool valid) const
     {
-        if (__builtin_amdgcn_ballot_w64(valid && (pr.flags & kSkip) != 0u) != 0ull) return 0;
-        return __builtin_amdgcn_ballot_w64(valid && (pr.flags & 3u) != 0u) == 0ull ? 1 : 2;
+        // skipped ratings and thinned updates (opt-in, Schedule::keep_u) leave out memory instructions: general path
+        if (__builtin_amdgcn_ballot_w64(valid && ((pr.flags & kSkip) != 0u || (my.thin & 3u) != 0u)) != 0ull) return 0;
+        return __builtin_amdgcn_ballot_w64(valid && (pr.flags & 3u) != 0u) == 0ull ? 1 : (MIXED ? 2 : 0);
     }
     static __device__ __forceinline__ Info no_row() { return Info{0.f, 0ull, 0ull, kSkip, 0u}; }      // null pointers: forward() matches no row
     __device__ __forceinline__ Info info(const Rating& my, const Prep& pr, int j) const
@@ -175,6 +183,57 @@ template <int K, bool COH, bool SAMPLED> struct MascotRuleT {
             else r[0] = row_load((reinterpret_cast<const uint16_t*>(ptr) + lane));
         }
     }
+    // Chunks of mixed precisions (class 2): the same instructions for a row of either precision, so that a rating takes
+    // no branch on its way to the rows and the compiler can count the loads in flight.  Every access goes through two
+    // windows over the row, one per precision, of which the one that does not apply is closed (0 bytes): both
+    // instructions are issued, the hardware drops the one through the closed window (a dropped load returns zero).
+    // A binary32 row is moved with 8-byte accesses (k = 128; 4-byte at k = 64), a binary16 row with 4-byte ones (2-byte).
+    struct Windows { row_window_t wide, narrow; };
+    static __device__ __forceinline__ Windows windows(uint64_t ptr, bool fp32)
+    {
+        return Windows{row_window(ptr, fp32 ? K * 4u : 0u), row_window(ptr, fp32 ? 0u : K * 2u)};
+    }
+    static __device__ __forceinline__ void load_mixed(uint32_t* r, uint32_t& h, uint64_t ptr, bool fp32, int lane)
+    {
+        const Windows w = windows(ptr, fp32);
+        if constexpr (E == 2) {
+            const auto v = __builtin_amdgcn_raw_buffer_load_b64(w.wide, lane * 8, 0, 0);
+            r[0] = v[0]; r[1] = v[1];
+            h = __builtin_amdgcn_raw_buffer_load_b32(w.narrow, lane * 4, 0, 0);
+        } else {
+            r[0] = __builtin_amdgcn_raw_buffer_load_b32(w.wide, lane * 4, 0, 0);
+            h = __builtin_amdgcn_raw_buffer_load_b16(w.narrow, lane * 2, 0, 0);
+        }
+    }
+    template <bool C> static __device__ __forceinline__ void store_mixed(const uint32_t* r, uint64_t ptr, bool fp32, int lane)
+    {
+        const Windows w = windows(ptr, fp32);
+        if constexpr (E == 2) {
+            window_store<C>(w.wide, (uint32_t)lane * 8u, (uint64_t)r[0] | ((uint64_t)r[1] << 32));
+            window_store<C>(w.narrow, (uint32_t)lane * 4u, r[0]);
+        } else {
+            window_store<C>(w.wide, (uint32_t)lane * 4u, r[0]);
+            window_store<C>(w.narrow, (uint32_t)lane * 2u, (uint16_t)r[0]);
+        }
+    }
+    // d: the change of this lane's elements in binary32; a binary16 row receives it rounded
+    static __device__ __forceinline__ void add_mixed(uint64_t ptr, const float* d, bool fp32, int lane)
+    {
+        const Windows w = windows(ptr, fp32);
+        if constexpr (E == 2) {
+            float lower, upper;
+            const uint32_t at = halves_of_row(d, lower, upper, lane);
+            window_add(w.wide, at, lower);
+            window_add(w.wide, at + K * 2u, upper);
+            window_add(w.narrow, (uint32_t)lane * 4u, narrow(d));
+        } else {
+            window_add(w.wide, (uint32_t)lane * 4u, d[0]);
+            // one element per lane: even lanes add the pair (own, right neighbour), odd lanes aim past the window
+            const uint32_t mine = (uint32_t)bits(narrow(d));
+            const uint32_t other = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)mine, 0xB1 /* quad_perm 1,0,3,2 */, 0xf, 0xf, false);
+            window_add(w.narrow, (lane & 1) ? 0x7ffffff0u : (uint32_t)lane * 2u, from_bits<half2_t>(mine | (other << 16)));
+        }
+    }
     // hot row (Schedule::keep_u): add the change of this lane's elements to the row in memory
     static __device__ __forceinline__ void add_side_half(uint64_t ptr, HV d, int lane)
     {
@@ -187,6 +246,20 @@ template <int K, bool COH, bool SAMPLED> struct MascotRuleT {
             if (!(lane & 1)) row_add(reinterpret_cast<half2_t*>(reinterpret_cast<uint16_t*>(ptr) + lane), from_bits<half2_t>(mine | (other << 16)));
         }
     }
+    // An add to a binary32 row at k = 128 is two instructions.  With the lane's own elements 2L, 2L+1 each of them would
+    // touch every other dword of the whole row: twice the 64-byte pieces at the memory side, where the adds are carried
+    // out.  One v_permlane32_swap turns the pairs into the row's halves instead: `lower` holds elements 0..63 (the even
+    // ones in lanes 0..31, the odd ones in lanes 32..63), `upper` elements 64..127; returns the byte offset of this
+    // lane's element of the lower half.
+    static __device__ __forceinline__ uint32_t halves_of_row(const float* d, float& lower, float& upper, int lane)
+    {
+        const auto r = __builtin_amdgcn_permlane32_swap(bits(d[0]), bits(d[1]), false, false);
+        lower = from_bits<float>(r[0]); upper = from_bits<float>(r[1]);
+        return ((((uint32_t)lane & 31u) << 1) | ((uint32_t)lane >> 5)) * 4u;
+    }
+    // The general path (class 0: the few chunks that are cut short or hold a skipped or thinned rating) adds the pairs as
+    // they are: the rearrangement above would cost the whole kernel four registers, and with them a resident wavefront
+    // per SIMD, for chunks that are hardly ever seen.
     static __device__ __forceinline__ void add_side_float(uint64_t ptr, const float* d, int lane)
     {
 #pragma unroll
@@ -207,10 +280,13 @@ template <int K, bool COH, bool SAMPLED> struct MascotRuleT {
         if constexpr (CLS == 1) {
             load_side(row.p, i.pptr, false, lane);
             load_side(row.q, i.qptr, false, lane);
+        } else if constexpr (CLS == 2) {
+            load_mixed(row.p, row.ph, i.pptr, i.flags & 1u, lane);
+            load_mixed(row.q, row.qh, i.qptr, i.flags & 2u, lane);
         } else {
 #pragma unroll
             for (int e = 0; e < E; ++e) { row.p[e] = 0; row.q[e] = 0; }
-            if (CLS == 0 && (i.flags & kSkip)) return;
+            if (i.flags & kSkip) return;
             load_side(row.p, i.pptr, i.flags & 1u, lane);
             load_side(row.q, i.qptr, i.flags & 2u, lane);
         }
@@ -224,6 +300,11 @@ template <int K, bool COH, bool SAMPLED> struct MascotRuleT {
         for (int e = 0; e < E; ++e) {
             nxt.p[e] = same_p ? cur.p[e] : nxt.p[e];
             nxt.q[e] = same_q ? cur.q[e] : nxt.q[e];
+        }
+        // a row that has been updated is in p, q whatever its precision (update() merges ph, qh into them)
+        if constexpr (MIXED) {
+            nxt.ph = same_p ? 0u : nxt.ph;
+            nxt.qh = same_q ? 0u : nxt.qh;
         }
     }
 
@@ -332,12 +413,46 @@ template <int K, bool COH, bool SAMPLED> struct MascotRuleT {
         }
     }
 
+    // Writes one side of an update: the new row `r` (raw registers) or, for an added row, its change `d` (binary32; a
+    // binary16 row receives it rounded, which is exact when it was computed in binary16).  bits: the side's thin bits
+    // shifted down -- 4 the row is added to, 16 the row is this XCD's copy of a replicated row.
+    // the same for a binary16 row whose change was computed in binary16 (mascot_sgd_kernel.h:188-278)
+    template <int CLS, bool HOT> __device__ __forceinline__ void write_side_half(const uint32_t* r, HV d, uint64_t ptr, uint32_t bits_) const
+    {
+        if constexpr (CLS == 2) {
+            float df[E];
+#pragma unroll
+            for (int e = 0; e < E; ++e) df[e] = widen(d, e);      // exact, and narrowed again exactly by add_mixed
+            write_side<CLS, HOT>(r, df, ptr, false, bits_);
+        } else {
+            if (HOT && (bits_ & 20u) == 16u) store_side<false>(r, ptr, false, lane);
+            else if (HOT && (bits_ & 4u)) add_side_half(ptr, d, lane);
+            else store_side(r, ptr, false, lane);
+        }
+    }
+    template <int CLS, bool HOT> __device__ __forceinline__ void write_side(const uint32_t* r, const float* d, uint64_t ptr, bool fp32, uint32_t bits_) const
+    {
+        if constexpr (CLS == 2) {
+            if (HOT && (bits_ & 20u) == 16u) store_mixed<false>(r, ptr, fp32, lane);
+            else if (HOT && (bits_ & 4u)) add_mixed(ptr, d, fp32, lane);
+            else store_mixed<COH>(r, ptr, fp32, lane);
+        } else {
+            if (HOT && (bits_ & 20u) == 16u) store_side<false>(r, ptr, fp32, lane);
+            else if (HOT && (bits_ & 4u)) { if (fp32) add_side_float(ptr, d, lane); else add_side_half(ptr, narrow(d), lane); }
+            else store_side(r, ptr, fp32, lane);
+        }
+    }
     template <int CLS, bool HOT> __device__ __forceinline__ void update(Row& row, const Info& i, uint32_t processed) const
     {
         if (CLS == 0 && (i.flags & kSkip)) return;
         const bool up = CLS != 1 && (i.flags & 1u), ip = CLS != 1 && (i.flags & 2u);
+        // thinned updates (only read the row) occur in chunks of class 0 only: classify() sends their chunks there
+        const bool skip_p = CLS == 0 && HOT && (i.thin & 1u), skip_q = CLS == 0 && HOT && (i.thin & 2u);
         const bool sampled = SAMPLED && processed >= first_sample;
         const uint32_t ug = (i.flags >> 3) & 0x3fffu, ig = (i.flags >> 17) & 0x3fffu;
+        if constexpr (CLS == 2) {       // load_mixed: the row came through one of two windows, the other gave zero
+            row.p[0] |= row.ph; row.q[0] |= row.qh; row.ph = 0u; row.qh = 0u;
+        }
         if (!up && !ip) {
             // mascot_sgd_kernel.h:188-278: everything in binary16, one rounding per operation
             const HV lam_h = splat((half_t)lambda);
@@ -349,15 +464,13 @@ template <int K, bool COH, bool SAMPLED> struct MascotRuleT {
             const HV ruv = splat(r_h - dot);
             const HV gp = ruv * Q - lam_h * P;
             const HV gq = ruv * P - lam_h * Q;
-            if (!(i.thin & 1u)) {
+            if (!skip_p) {
                 row.p[0] = bits(HV(__builtin_elementwise_fma(lr_p, gp, P)));
-                if ((i.thin & 20u) == 16u) store_side<false>(row.p, i.pptr, false, lane);
-                else if (i.thin & 4u) add_side_half(i.pptr, lr_p * gp, lane); else store_side(row.p, i.pptr, false, lane);
+                write_side_half<CLS, HOT>(row.p, lr_p * gp, i.pptr, i.thin);
             }
-            if (!(i.thin & 2u)) {
+            if (!skip_q) {
                 row.q[0] = bits(HV(__builtin_elementwise_fma(lr_q, gq, Q)));
-                if ((i.thin & 40u) == 32u) store_side<false>(row.q, i.qptr, false, lane);
-                else if (i.thin & 8u) add_side_half(i.qptr, lr_q * gq, lane); else store_side(row.q, i.qptr, false, lane);
+                write_side_half<CLS, HOT>(row.q, lr_q * gq, i.qptr, i.thin >> 1);
             }
             if (sampled) {
                 float g[E];
@@ -370,10 +483,14 @@ template <int K, bool COH, bool SAMPLED> struct MascotRuleT {
             }
         } else {
             float pf[E], qf[E], m[E];
-            if (up) { for (int e = 0; e < E; ++e) pf[e] = from_bits<float>(row.p[e]); }
-            else { const HV P = from_bits<HV>(row.p[0]); for (int e = 0; e < E; ++e) pf[e] = widen(P, e); }
-            if (ip) { for (int e = 0; e < E; ++e) qf[e] = from_bits<float>(row.q[e]); }
-            else { const HV Q = from_bits<HV>(row.q[0]); for (int e = 0; e < E; ++e) qf[e] = widen(Q, e); }
+            {   // selects on wave-uniform flags: a binary16 row's second register holds nothing of the row
+                const HV P = from_bits<HV>(row.p[0]), Q = from_bits<HV>(row.q[0]);
+#pragma unroll
+                for (int e = 0; e < E; ++e) {
+                    pf[e] = up ? from_bits<float>(row.p[e]) : widen(P, e);
+                    qf[e] = ip ? from_bits<float>(row.q[e]) : widen(Q, e);
+                }
+            }
 #pragma unroll
             for (int e = 0; e < E; ++e) m[e] = pf[e] * qf[e];
             const float ruv = i.r - dot_float(m);
@@ -386,25 +503,20 @@ template <int K, bool COH, bool SAMPLED> struct MascotRuleT {
                 np_[e] = __builtin_fmaf(lr_p, gp[e], pf[e]);
                 nq_[e] = __builtin_fmaf(lr_q, gq[e], qf[e]);
             }
-            if (!(i.thin & 1u)) {
-                if (up) { for (int e = 0; e < E; ++e) row.p[e] = bits(np_[e]); }
-                else row.p[0] = bits(narrow(np_));
-                if ((i.thin & 20u) == 16u) store_side<false>(row.p, i.pptr, up, lane);
-                else if (i.thin & 4u) {
-                    float d[E];
-                    for (int e = 0; e < E; ++e) d[e] = lr_p * gp[e];
-                    if (up) add_side_float(i.pptr, d, lane); else add_side_half(i.pptr, narrow(d), lane);
-                } else store_side(row.p, i.pptr, up, lane);
+            float d[E];
+            if (!skip_p) {
+                const uint32_t rounded = bits(narrow(np_));
+#pragma unroll
+                for (int e = 0; e < E; ++e) row.p[e] = up ? bits(np_[e]) : (e == 0 ? rounded : row.p[e]);
+                if (HOT && (i.thin & 4u)) { for (int e = 0; e < E; ++e) d[e] = lr_p * gp[e]; }
+                write_side<CLS, HOT>(row.p, d, i.pptr, up, i.thin);
             }
-            if (!(i.thin & 2u)) {
-                if (ip) { for (int e = 0; e < E; ++e) row.q[e] = bits(nq_[e]); }
-                else row.q[0] = bits(narrow(nq_));
-                if ((i.thin & 40u) == 32u) store_side<false>(row.q, i.qptr, ip, lane);
-                else if (i.thin & 8u) {
-                    float d[E];
-                    for (int e = 0; e < E; ++e) d[e] = lr_q * gq[e];
-                    if (ip) add_side_float(i.qptr, d, lane); else add_side_half(i.qptr, narrow(d), lane);
-                } else store_side(row.q, i.qptr, ip, lane);
+            if (!skip_q) {
+                const uint32_t rounded = bits(narrow(nq_));
+#pragma unroll
+                for (int e = 0; e < E; ++e) row.q[e] = ip ? bits(nq_[e]) : (e == 0 ? rounded : row.q[e]);
+                if (HOT && (i.thin & 8u)) { for (int e = 0; e < E; ++e) d[e] = lr_q * gq[e]; }
+                write_side<CLS, HOT>(row.q, d, i.qptr, ip, i.thin >> 1);
             }
             if (sampled) {
                 if (!up) sample(gp, ug, true);
@@ -447,5 +559,6 @@ template <int K, bool COH, bool SAMPLED> struct MascotRuleT {
 };
 template <int K, bool COH> using MascotRule = MascotRuleT<K, COH, true>;
 template <int K, bool COH> using MascotPlainRule = MascotRuleT<K, COH, false>;
+template <int K, bool COH> using MascotBinary16Rule = MascotRuleT<K, COH, false, false>;
 
 }  // namespace mf

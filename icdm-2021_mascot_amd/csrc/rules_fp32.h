@@ -36,7 +36,7 @@ template <int K, bool COH> struct DenseBase {
     __device__ __forceinline__ float step_of(float lrate, uint32_t thin, uint32_t bit) const { return (thin & bit) ? lrate * rep_scale : lrate; }
 
     __device__ __forceinline__ Prep prepare(const Rating&, bool) const { return Prep(); }
-    __device__ __forceinline__ int classify(const Prep&, bool) const { return 0; }
+    __device__ __forceinline__ int classify(const Rating&, const Prep&, bool) const { return 0; }
     static __device__ __forceinline__ Info no_row() { return Info{0.f, 0xffffffffu, 0xffffffffu, 0u}; }   // matches no rating
     // u, v: the rows to address (Rating::ru, rv); equal values are the same row, which is all forward() needs
     __device__ __forceinline__ Info info(const Rating& my, const Prep&, int j) const
@@ -242,7 +242,7 @@ template <int K, bool COH> struct MemQuantRule {
     static constexpr int kK = K;
     static void row_storage(const Params& a, RowStorage& u, RowStorage& v) { u.dense = a.p; u.elem_bytes = 2; v.dense = a.q; v.elem_bytes = 2; }
     __device__ __forceinline__ Prep prepare(const Rating&, bool) const { return Prep(); }
-    __device__ __forceinline__ int classify(const Prep&, bool) const { return 0; }
+    __device__ __forceinline__ int classify(const Rating&, const Prep&, bool) const { return 0; }
     static __device__ __forceinline__ Info no_row() { return Info{0.f, 0xffffffffu, 0xffffffffu, 0u}; }
     __device__ __forceinline__ Info info(const Rating& my, const Prep&, int j) const
     {

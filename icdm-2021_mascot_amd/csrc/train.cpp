@@ -247,10 +247,12 @@ struct HotRows {
         return 0;
     }
     // options of the launches of epoch e (valid until the next call)
+    bool all_binary16 = false;      // MASCOT runs: no group has been promoted yet
     const mf_hogwild_options* options(uint32_t e) const
     {
         opt_current = e < early_epochs ? opt_early : opt_steady;
         opt_current.replica_step_scale = (step_epochs == 0 || e < step_epochs) ? step_scale : 0.f;
+        opt_current.all_binary16 = all_binary16 ? 1u : 0u;
         return &opt_current;
     }
 };
@@ -381,6 +383,7 @@ struct DenseRun : Run {
     int epoch(uint32_t e) override
     {
         const mf_node* R = c.d_R.as<mf_node>();
+        hot.all_binary16 = version == 8 && !whole.is_float;
         const mf_hogwild_options* opt = hot.options(e);
         bool whole_check = false;
         const double err0 = now_ms();
@@ -670,6 +673,8 @@ struct MascotRun : Run {
             HIP_TRY(hipMemsetAsync(I.d_grad_sum.p, 0, (size_t)I.groups * c.k * 4, nullptr), "memset grad_sum_norm_q");
             err_ms += now_ms() - e0;
         }
+        hot.all_binary16 = std::none_of(U.prec.begin(), U.prec.end(), [](uint8_t v) { return v != 0; }) &&
+                           std::none_of(I.prec.begin(), I.prec.end(), [](uint8_t v) { return v != 0; });
         t.start();
         MF_TRY(mf_mascot_sgd_hogwild_opt(c.d_R.as<mf_node>(), c.n, U.d_ptr.as<void*>(), I.d_ptr.as<void*>(), (int)c.k,
                                          prm.num_workers, c.update_count, c.update_vector_size, c.lr[e], prm.lambda,

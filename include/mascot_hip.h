@@ -85,7 +85,11 @@ const char* mf_last_error(void);
  *               the merge is the mean over the X = min(MF_XCDS, workgroups of the launch) copies in play, untouched ones
  *               counting as the row.  With X = 1 (a launch of one workgroup) nothing changes.  The caller bounds the
  *               factor by what keeps a single step stable: factor x learning rate x |other side's row|^2 well below 2
- *               (mf_replica_step_scale). */
+ *               (mf_replica_step_scale).
+ * all_binary16  MASCOT only, a hint: 1 = every group of both sides is binary16 in this call.  The call then launches a
+ *               build of the kernel without the fast path for chunks of mixed precisions, which keeps one more
+ *               wavefront per SIMD resident (4 % per epoch at 100M ratings).  A wrong hint costs time, not results:
+ *               that build takes its general path for any chunk that touches a binary32 group. */
 #define MF_KEEP_ORDINARY 255
 #define MF_KEEP_ADDED 254
 #define MF_KEEP_REPLICATED 253
@@ -104,6 +108,7 @@ typedef struct {
     void* item_replicas;
     uint32_t user_slots, item_slots;
     float replica_step_scale;
+    uint32_t all_binary16;
 } mf_hogwild_options;
 /* What the update calls do with replicated rows before and after every kernel launch, for a dense matrix [rows][k] of
  * elem_bytes-wide elements (2: binary16, 4: binary32): merge = 0 copies row slot_row[s] into slot s of every XCD's
