@@ -14,6 +14,7 @@ through the C ABI of libmascot_hip.so.  One JSON line on stdout.
 import argparse
 import ctypes as C
 import glob
+import hashlib
 import importlib
 import json
 import os
@@ -26,15 +27,34 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 PEAK_HBM_GBS = 8000.0
 TRAIN = dict(epochs=50, lr=0.01, decay=0.1, lam=0.015, sample_ratio=0.05, interval=2, ug=100, ig=100, threshold=20.0)
-# rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of a plain epoch's update kernels (KiB per epoch, scaled by the factors a 1 GiB
-# device copy gives), recorded in the profile named here; reported only for the workload they were taken on
-PROFILED_TRAFFIC = {
-    # (config, training ratings, k, seed, workers): bytes per epoch (four launches of the update kernel)
-    (4, 100_000_000, 128, 2021, 48832): dict(
-        bytes=(2 * 15_071_100 + 29_504_070) * 1024,
-        source="rocprofv3 --pmc FETCH_SIZE (x2.0) and WRITE_SIZE (x1.0) of the four update launches of epoch 2, recorded in "
-               "profiles/hogwild_mascot_k128_config4_hbm_traffic.md; not re-measured by this run"),
-}
+# rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of a plain epoch's update kernels, recorded with the workload and the digest of
+# the kernel sources they were taken with; reported only for that workload and those sources
+PROFILED_TRAFFIC = os.path.join(ROOT, "profiles", "hogwild_mascot_k128_config4_hbm_traffic.json")
+KERNEL_SOURCES = os.path.join(ROOT, "icdm-2021_mascot_amd", "csrc")
+
+
+def kernel_sources_digest():
+    """sha256 over the device sources of the library (file names and contents, in name order)."""
+    h = hashlib.sha256()
+    for name in sorted(os.listdir(KERNEL_SOURCES)):
+        if name.endswith((".h", ".hip")):
+            h.update(name.encode())
+            with open(os.path.join(KERNEL_SOURCES, name), "rb") as f:
+                h.update(f.read())
+    return h.hexdigest()
+
+
+def profiled_traffic(config, n_train, k, seed, workers):
+    """The committed HBM-side bytes per plain epoch of this workload, or None when the record is of another workload or
+    of other kernel sources than the ones this library was built from."""
+    try:
+        rec = json.load(open(PROFILED_TRAFFIC))
+    except (OSError, ValueError):
+        return None
+    same = (rec.get("config"), rec.get("n_train"), rec.get("k"), rec.get("seed"), rec.get("workers")) == (config, n_train, k, seed, workers)
+    if not same or rec.get("kernel_sources_sha256") != kernel_sources_digest():
+        return None
+    return rec
 
 
 def generate(h, config, seed, n_train, n_test):
@@ -57,9 +77,11 @@ def generate(h, config, seed, n_train, n_test):
 
 
 def params(h, a, version, **kw):
-    return h.default_params(k=a.k, num_workers=a.workers, epoch=TRAIN["epochs"], learning_rate=TRAIN["lr"], lam=TRAIN["lam"], decay=TRAIN["decay"],
-                            version=version, seed=a.seed, user_group_num=TRAIN["ug"], item_group_num=TRAIN["ig"], sample_ratio=TRAIN["sample_ratio"],
-                            interval=TRAIN["interval"], error_threshold=TRAIN["threshold"], **kw)
+    args = dict(k=a.k, num_workers=a.workers, epoch=TRAIN["epochs"], learning_rate=TRAIN["lr"], lam=TRAIN["lam"], decay=TRAIN["decay"],
+                version=version, seed=a.seed, user_group_num=TRAIN["ug"], item_group_num=TRAIN["ig"], sample_ratio=TRAIN["sample_ratio"],
+                interval=TRAIN["interval"], error_threshold=TRAIN["threshold"])
+    args.update(kw)
+    return h.default_params(**args)
 
 
 def run_session(torch, capi, h, prm, cfg, train, test, seed, warmup, steps, run_to=0, half_init=False):
@@ -67,47 +89,68 @@ def run_session(torch, capi, h, prm, cfg, train, test, seed, warmup, steps, run_
     its update launches), then untimed on to `run_to` epochs.  Returns the figures and the still open session."""
     p, q = h.init_model(cfg.n_users, cfg.n_items, prm.k, seed, half_init)
     s = capi.Session(h, prm, train, cfg.n_users, cfg.n_items, test, p, q)
-    rmse, ms = [], []
-    for _ in range(warmup):
+    rmse, ms, prec = [], [], []
+
+    def epoch():
+        # the precision of every group while this epoch's updates run (switching comes after them)
+        prec.append((s.groups(0)[0], s.groups(1)[0]))
         r, m = s.epoch(); rmse.append(r); ms.append(m)
+    for _ in range(warmup):
+        epoch()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(steps):
-        r, m = s.epoch(); rmse.append(r); ms.append(m)
+        epoch()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     while s.epochs_done < run_to:
-        r, m = s.epoch(); rmse.append(r); ms.append(m)
-    return dict(session=s, rmse=rmse, ms=ms, wall_s=wall, timed=ms[warmup:warmup + steps])
+        epoch()
+    return dict(session=s, rmse=rmse, ms=ms, wall_s=wall, timed=ms[warmup:warmup + steps], prec=prec)
+
+
+def epoch_bytes(k, updates, prec, ratings):
+    """Algorithmic bytes of one MASCOT epoch: every update reads 12 bytes of rating and reads and writes one row per side,
+    2 k bytes for a binary16 row and 4 k for a binary32 one (mascot_sgd_kernel.h:188-443, the four cases).  The case of
+    an update follows from the groups of its two rows, so the sum over the epoch's updates is, per side, the share of
+    the ratings that falls on binary32 groups.  Returns (bytes, user share, item share)."""
+    share = []
+    for side in (0, 1):
+        r = ratings[side].astype(np.float64)
+        share.append(float((r * (prec[side] != 0)).sum() / r.sum()) if r.size else 0.0)
+    per_update = 12 + 2 * k * (2 + 2 * share[0]) + 2 * k * (2 + 2 * share[1])
+    return updates * per_update, share[0], share[1]
 
 
 def is_check_epoch(e):
     return e >= 5 and e % TRAIN["interval"] == 5 % TRAIN["interval"] and e != TRAIN["epochs"] - 1
 
 
-def reference_curve(config, n_train, k, seed):
+def reference_curve(config, n_train, k, seed, version=1):
     """Per-epoch test RMSE of the reference rule on the CPU (tests/golden/make_reference_curve.py): mean and spread of the
     committed runs of this workload, or None."""
     runs = []
-    for path in sorted(glob.glob(os.path.join(ROOT, "tests", "golden", "reference_curve_config%d_run*.json" % config))):
+    for path in sorted(glob.glob(os.path.join(ROOT, "tests", "golden", "reference_curve_config%d*_run*.json" % config))):
         d = json.load(open(path))
-        if d["n_train"] == n_train and d["train"]["k"] == k and d["seed"] == seed and d["scale"] == 1.0:
+        if d["n_train"] == n_train and d["train"]["k"] == k and d["seed"] == seed and d["scale"] == 1.0 and d.get("version", 1) == version:
             runs.append(d)
     if not runs:
         return None
     epochs = min(len(d["test_rmse"]) for d in runs)
     curves = np.array([d["test_rmse"][:epochs] for d in runs])
-    return dict(mean=curves.mean(0), spread=curves.max(0) - curves.min(0), runs=len(runs), threads=runs[0]["threads"], workers=runs[0]["workers"])
+    return dict(mean=curves.mean(0), spread=curves.max(0) - curves.min(0), runs=len(runs), threads=runs[0]["threads"], workers=runs[0]["workers"],
+                user_groups_binary32=[d.get("user_groups_binary32") for d in runs] if "user_groups_binary32" in runs[0] else None,
+                item_groups_binary32=[d.get("item_groups_binary32") for d in runs] if "item_groups_binary32" in runs[0] else None)
 
 
-def probe_ms(torch, h, sess, n, n_users, n_items, row_bytes, workers, seed, epoch, reps=3):
+def probe_ms(torch, h, sess, n, n_users, n_items, row_bytes, workers, seed, epoch, reps=3, item_row_bytes=0):
     """mf_row_traffic_probe on the session's ratings and launch options: the epoch's memory traffic without the arithmetic."""
     dev = torch.device("cuda:0")
+    item_row_bytes = item_row_bytes or row_bytes
     P = torch.zeros(n_users * row_bytes, dtype=torch.uint8, device=dev)
-    Q = torch.zeros(n_items * row_bytes, dtype=torch.uint8, device=dev)
+    Q = torch.zeros(n_items * item_row_bytes, dtype=torch.uint8, device=dev)
     r_ptr, o_ptr = sess.device_state(epoch)
     st = torch.cuda.current_stream().cuda_stream
-    run = lambda: h.mf_row_traffic_probe(r_ptr, n, P.data_ptr(), Q.data_ptr(), row_bytes, workers, seed, st, o_ptr)
+    run = lambda: h.mf_row_traffic_probe_sides(r_ptr, n, P.data_ptr(), Q.data_ptr(), row_bytes, item_row_bytes, workers, seed, st, o_ptr)
     run(); torch.cuda.synchronize()
     ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(reps)]
     for x, y in ev:
@@ -170,7 +213,7 @@ def main():
     ap.add_argument("--skip-fp32", action="store_true", help="skip the fp32-SGD leg")
     ap.add_argument("--skip-ceiling", action="store_true", help="skip the access-pattern probe")
     ap.add_argument("--skip-full-run", action="store_true", help="stop after the timed epochs instead of running on to epoch 50")
-    ap.add_argument("--reference-semantics", action="store_true", help="also time two epochs without hot rows (-hot 0: every row stored, last writer wins)")
+    ap.add_argument("--skip-reference-semantics", action="store_true", help="skip the two epochs without hot rows (-hot 0: every row stored, last writer wins; 0.25 s per epoch)")
     ap.add_argument("--every-rule", action="store_true", help="also run MPT, MuPPET, AFP and binary16 storage (-v 4, 3, 2, 7) for eight epochs each")
     ap.add_argument("--rules", default="mpt,muppet,afp,mem_quant", help="the rules --every-rule runs")
     ap.add_argument("--pmc-copy", action="store_true", help="profiling aid: also run three 1 GiB device copies, the known-size kernel that FETCH_SIZE / WRITE_SIZE are scaled by")
@@ -184,7 +227,7 @@ def main():
         print("bench.py: warmup + steps is at most %d, the epochs of the configured run" % TRAIN["epochs"], file=sys.stderr)
         sys.exit(2)
     if a.only_timed:
-        a.skip_cpu = a.skip_fp32 = a.skip_ceiling = a.skip_full_run = True
+        a.skip_cpu = a.skip_fp32 = a.skip_ceiling = a.skip_full_run = a.skip_reference_semantics = True
     import torch
     capi = importlib.import_module("icdm-2021_mascot_amd.capi")
     h = importlib.import_module("icdm-2021_mascot_amd").load()
@@ -222,10 +265,13 @@ def main():
     timed = np.array(main_run["timed"], np.float64)
     ms = float(timed.mean())
     # a rating reads 12 B and one row per side and writes both rows back: 12 + 2 k (s_user + s_item) bytes, s = 2 for a
-    # binary16 row and 4 for a binary32 one.  Groups promoted to binary32 before the timed epochs make their rows wider.
-    # The figure below counts every row as binary16 (1036 B), the least the run can need.
-    bytes_per_update = 12 + 2 * k * (2 + 2)
-    gbs = updates * bytes_per_update / (ms / 1e3) / 1e9
+    # binary16 row and 4 for a binary32 one; per epoch the sum over its updates follows from the precision of the groups
+    # during that epoch and the ratings that fall on each group (epoch_bytes)
+    group_ratings = (sess.groups(0)[1], sess.groups(1)[1])
+    per_epoch = [epoch_bytes(k, updates, pr, group_ratings) for pr in main_run["prec"]]
+    timed_bytes = float(np.mean([b for b, _, _ in per_epoch[a.warmup:a.warmup + a.steps]]))
+    bytes_per_update = timed_bytes / updates
+    gbs = timed_bytes / (ms / 1e3) / 1e9
     epochs_done_timed = a.warmup + a.steps
     launches = capi.HogwildOptions.from_address(sess.device_state(a.warmup)[1]).launches or 1
     plain = [m for i, m in enumerate(main_run["timed"]) if not is_check_epoch(a.warmup + i)] or list(main_run["timed"])
@@ -244,11 +290,13 @@ def main():
                    "replicate_above_in_flight": float(h.mf_replicate_threshold(TRAIN["lr"], float(np.abs(train["r"][:4_000_000]).mean()))) if a.replicate < 0 else a.replicate,
                    "setup_s": round(setup_s, 1)},
         "roofline": {"bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS,
-                     "note": "algorithmic bytes: every update reads and writes both rows (1036 B at k=128, binary16); rows that are "
-                             "re-used while they sit in an L2 never reach HBM, so this is the rate the update stream is served at, "
-                             "bounded by the HBM peak only for traffic that misses",
+                     "note": "algorithmic bytes: every update reads and writes both rows (12 + 2k(s_user + s_item) bytes, s = 2 for a binary16 "
+                             "and 4 for a binary32 row, summed over the epoch's updates by the precision of their groups; 1036 B while "
+                             "every group is binary16).  Rows that are re-used while they sit in an L2 never reach HBM, so `frac` is the "
+                             "rate the update stream is served at over the HBM peak, not HBM utilisation: the profiled HBM-side share is "
+                             "`hbm_side.frac`",
                      "traffic": None,
-                     "kernel": "hogwild_kernel<MascotRuleT<%d,true,false>,true>" % k,
+                     "kernel": "hogwild_kernel<MascotRuleT<%d,true,false,false>,true>" % k,
                      "bytes_per_update": bytes_per_update, "updates_per_step": updates,
                      "kernel_launches_per_step": launches,
                      "per": "step: achieved, traffic and updates are those of one epoch = the driver's update call, which cuts the epoch into "
@@ -260,11 +308,14 @@ def main():
         "test_rmse_after_timed_epochs": {"value": main_run["rmse"][epochs_done_timed - 1], "epochs": epochs_done_timed, "test_ratings": int(test.size)},
         "test_rmse_per_epoch": [round(float(x), 5) for x in main_run["rmse"]],
     }
-    traffic = PROFILED_TRAFFIC.get((a.config, n_train, k, a.seed, W))
-    if traffic is not None and a.replicate < 0 and a.thin == 0:
-        out["roofline"]["traffic"] = traffic["bytes"]
+    traffic = profiled_traffic(a.config, n_train, k, a.seed, W)
+    if traffic is not None and a.replicate < 0 and a.thin == 0 and a.step_scale < 0 and a.step_epochs < 0 and not a.merges:
+        out["roofline"]["traffic"] = traffic["bytes_per_epoch"]
         out["roofline"]["traffic_source"] = traffic["source"]
-        out["roofline"]["hbm_frac_profiled"] = traffic["bytes"] / (float(np.mean(plain)) / 1e3) / 1e9 / PEAK_HBM_GBS
+        out["roofline"]["hbm_side"] = {"frac": traffic["bytes_per_epoch"] / (float(np.mean(plain)) / 1e3) / 1e9 / PEAK_HBM_GBS,
+                                       "note": "profiled HBM bytes of a plain all-binary16 epoch (FETCH_SIZE + WRITE_SIZE, not re-measured by this run) "
+                                               "over this run's mean plain epoch, against the 8 TB/s peak: algorithmic %.2f / HBM-side %.2f"
+                                               % (gbs / PEAK_HBM_GBS, traffic["bytes_per_epoch"] / (float(np.mean(plain)) / 1e3) / 1e9 / PEAK_HBM_GBS)}
     ref = reference_curve(a.config, n_train, k, a.seed)
     if ref is not None:
         def delta(epochs):
@@ -286,7 +337,19 @@ def main():
                             "sgd_ms_epochs": [round(float(x), 2) for x in main_run["ms"]],
                             "ratings_per_s": n_train * TRAIN["epochs"] / (float(np.sum(main_run["ms"])) / 1e3),
                             "preprocess_ms": rep.preprocess_ms, "error_ms": rep.error_ms, "switching_ms": rep.switching_ms,
-                            "final_test_rmse": main_run["rmse"][-1]}
+                            "final_test_rmse": main_run["rmse"][-1],
+                            # the four precision cases per epoch: groups in binary32 while the epoch ran, the share of the
+                            # ratings on them, and the algorithmic bytes that follow (epoch_bytes)
+                            "user_groups_binary32": [int(pu.sum()) for pu, _ in main_run["prec"]],
+                            "item_groups_binary32": [int(pi.sum()) for _, pi in main_run["prec"]],
+                            "groups": {"user": int(group_ratings[0].size), "item": int(group_ratings[1].size)},
+                            "ratings_on_binary32_user_rows": [round(su, 4) for _, su, _ in per_epoch],
+                            "ratings_on_binary32_item_rows": [round(si, 4) for _, _, si in per_epoch],
+                            "algorithmic_gb_epochs": [round(b / 1e9, 2) for b, _, _ in per_epoch],
+                            "roofline_frac_epochs": [round(b / (m / 1e3) / 1e9 / PEAK_HBM_GBS, 3) for (b, _, _), m in zip(per_epoch, main_run["ms"])],
+                            "roofline_frac": float(sum(b for b, _, _ in per_epoch) / (float(np.sum(main_run["ms"])) / 1e3) / 1e9 / PEAK_HBM_GBS)}
+        if ref is not None and ref.get("user_groups_binary32") is not None:
+            out["whole_job"]["reference_rule_groups_binary32_after_50_epochs"] = {"user": ref["user_groups_binary32"], "item": ref["item_groups_binary32"]}
     if not a.skip_ceiling:
         ceil_ms = probe_ms(torch, h, sess, n_train, cfg.n_users, cfg.n_items, k * 2, W, a.seed, a.warmup)
         out["roofline"]["access_pattern_ceiling"] = {
@@ -311,10 +374,32 @@ def main():
             res["access_pattern_ceiling_ms"] = probe
         return res
 
+    def switched_leg():
+        """MASCOT epochs with every group of both sides promoted to binary32 after two binary16 epochs: the update kernel
+        on the bytes of the fp32 rule (2060 B per update at k = 128)."""
+        r = run_session(torch, capi, h, params(h, a, 1, **dict(extra, interval=0)), cfg, train, test, a.seed, 2, 0, 0)
+        s2 = r.pop("session")
+        for side in (0, 1):
+            s2.promote_groups(side, np.ones(s2.groups(side)[0].size, np.uint8))
+        t = [s2.epoch() for _ in range(4)]
+        probe = None if a.skip_ceiling else probe_ms(torch, h, s2, n_train, cfg.n_users, cfg.n_items, k * 4, s2.workers, a.seed, 2)
+        s2.close()
+        leg_ms = float(np.mean([m for _, m in t[1:]]))
+        res = {"note": "mf_train -v 1 with every group promoted to binary32 (mf_session_promote_groups) after epoch 2; epochs 4..6",
+               "ms_per_step": leg_ms, "value": n_train / (leg_ms / 1e3), "unit": "ratings/s",
+               "roofline_frac": updates * (12 + 4 * k * 4) / (leg_ms / 1e3) / 1e9 / PEAK_HBM_GBS}
+        if probe is not None:
+            res["access_pattern_ceiling_ms"] = probe
+        return res
+
     if not a.skip_fp32:
+        out["mascot_all_binary32"] = switched_leg()
         out["fp32_sgd"] = side_leg(5, a.warmup, a.steps, "fp32 SGD (mf_train -v 5) on the same ratings, workers and hot-row treatment, every row update carried out")
         out["fp32_sgd"]["mascot_speedup"] = out["fp32_sgd"]["ms_per_step"] / ms
-    if a.reference_semantics:
+        out["mascot_all_binary32"]["vs_fp32_sgd_epoch"] = out["mascot_all_binary32"]["ms_per_step"] / out["fp32_sgd"]["ms_per_step"]
+        if "whole_job" in out:
+            out["whole_job"]["speedup_vs_50_fp32_sgd_epochs"] = TRAIN["epochs"] * out["fp32_sgd"]["ms_per_step"] / out["whole_job"]["sgd_ms_total"]
+    if not a.skip_reference_semantics:
         out["reference_semantics"] = side_leg(1, 0, 2, "mf_train -v 1 without hot rows (-hot 0): every row stored with a device-coherent store, last writer "
                                               "wins -- bound by the serialisation of the stores to the hottest row at the memory side",
                                               hot_rows=0, replicate_inflight=0.0, hot_row_inflight=0.0)

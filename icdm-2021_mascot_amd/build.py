@@ -22,7 +22,7 @@ ARCH = "gfx950"
 # binary16 ulp on rare inputs, so the fused form must not be selected.
 DEVICE_FLAGS = ["--offload-arch=" + ARCH, "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off", "-munsafe-fp-atomics",
                 "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-                "-Xclang", "-target-feature", "-Xclang", "-fma-mix-insts", "-Wall", "-Wno-unused-function"]
+                "-Xclang", "-target-feature", "-Xclang", "-fma-mix-insts", "-Wall", "-Wno-unused-function"] + os.environ.get("MF_HIPCC_FLAGS", "").split()
 KERNEL_SOURCES = ["launch_mascot_plain.hip", "launch_mascot_sampled.hip", "launch_mascot_binary16.hip", "launch_muppet.hip", "launch_afp.hip", "hogwild_launch.hip", "launch_mem_quant.hip", "aux_kernels.hip",
                   "sort_shuffle.hip", "launch_mascot.hip"]
 HOST_SOURCES = ["train.cpp"]

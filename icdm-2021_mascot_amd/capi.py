@@ -28,6 +28,7 @@ SIGNATURES = {
     "mf_mem_quant_sgd_hogwild": (i32, [vp, u32, vp, vp, i32, u32, u32, u32, f32, f32, u64, u32, vp, vp]),
     "mf_hot_row_table": (i32, [vp, u32, u32, f32, f32, f32, f32, vp, vp, vp, vp]),
     "mf_row_traffic_probe": (i32, [vp, u32, vp, vp, u32, u32, u64, vp, vp]),
+    "mf_row_traffic_probe_sides": (i32, [vp, u32, vp, vp, u32, u32, u32, u64, vp, vp]),
     "mf_synth_baseline_config": (i32, [i32, vp]),
     "mf_generate_ratings": (i32, [vp, u64, u64, u64, vp, vp]),
     "mf_generate_ratings_host": (i32, [vp, u64, u64, u64, vp]),

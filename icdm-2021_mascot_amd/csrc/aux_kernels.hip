@@ -398,12 +398,13 @@ using namespace mf;
 // compiler cannot fold).  The same draw as the update kernels' thinning decides; a kept update of a hot row is a
 // store here too.  What it sustains is the ceiling the memory system sets for this sequence of addresses and this
 // write policy, the figure the update kernels' epoch time is compared with.
-template <int BYTES, bool COH>       // bytes per lane: a row is 64 * BYTES bytes
+template <int BYTES, bool COH, int BYTES_Q = BYTES>       // bytes per lane and side: a row is 64 * BYTES bytes
 __global__ __launch_bounds__(kBlock) void row_traffic_probe_kernel(const mf_node* R, uint32_t n, uint8_t* P, uint8_t* Q, uint32_t per_worker,
                                                                   const uint8_t* keep_u, const uint8_t* keep_v, const uint16_t* slot_u, const uint16_t* slot_v,
                                                                   uint32_t slots_u, uint32_t slots_v, uint8_t* RP, uint8_t* RQ, uint64_t key, uint32_t zero)
 {
     using T = typename std::conditional<BYTES == 8, uint64_t, typename std::conditional<BYTES == 4, uint32_t, uint16_t>::type>::type;
+    using TQ = typename std::conditional<BYTES_Q == 8, uint64_t, typename std::conditional<BYTES_Q == 4, uint32_t, uint16_t>::type>::type;
     constexpr int kDepth = 4;
     const int lane = threadIdx.x & (kWave - 1);
     const uint32_t worker = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
@@ -427,20 +428,20 @@ __global__ __launch_bounds__(kBlock) void row_traffic_probe_kernel(const mf_node
         }
         const int cnt = end - base < (uint32_t)kWave ? (int)(end - base) : kWave;
         for (int j0 = 0; j0 < cnt; j0 += kDepth) {
-            T a[kDepth], b[kDepth]; T* pa[kDepth]; T* pb[kDepth]; uint32_t kp[kDepth];
+            T a[kDepth]; TQ b[kDepth]; T* pa[kDepth]; TQ* pb[kDepth]; uint32_t kp[kDepth];
 #pragma unroll
             for (int d = 0; d < kDepth; ++d) {
                 const int j = j0 + d < cnt ? j0 + d : cnt - 1;
                 kp[d] = j0 + d < cnt ? bcast(keep, j) : 0u;
                 const uint32_t flags = bcast(keep, j);
                 pa[d] = reinterpret_cast<T*>(((flags & 4u) ? RP : P) + (size_t)bcast(mu, j) * (kWave * BYTES)) + lane;
-                pb[d] = reinterpret_cast<T*>(((flags & 8u) ? RQ : Q) + (size_t)bcast(mv, j) * (kWave * BYTES)) + lane;
+                pb[d] = reinterpret_cast<TQ*>(((flags & 8u) ? RQ : Q) + (size_t)bcast(mv, j) * (kWave * BYTES_Q)) + lane;
                 a[d] = row_load(pa[d]); b[d] = row_load(pb[d]);
             }
 #pragma unroll
             for (int d = 0; d < kDepth; ++d) {
                 if (kp[d] & 4u) row_store<false>(pa[d], (T)(a[d] + (T)zero)); else if (kp[d] & 1u) row_store<COH>(pa[d], (T)(a[d] + (T)zero));
-                if (kp[d] & 8u) row_store<false>(pb[d], (T)(b[d] + (T)zero)); else if (kp[d] & 2u) row_store<COH>(pb[d], (T)(b[d] + (T)zero));
+                if (kp[d] & 8u) row_store<false>(pb[d], (TQ)(b[d] + (TQ)zero)); else if (kp[d] & 2u) row_store<COH>(pb[d], (TQ)(b[d] + (TQ)zero));
             }
         }
     }
@@ -590,9 +591,15 @@ int mf_matrix_reconst_triplet(mf_node* R, const uint32_t* user2sorted_idx, const
 int mf_row_traffic_probe(const mf_node* R, uint32_t n, void* p, void* q, uint32_t row_bytes, uint32_t num_workers,
                          uint64_t seed, void* stream, const mf_hogwild_options* options)
 {
+    return mf_row_traffic_probe_sides(R, n, p, q, row_bytes, row_bytes, num_workers, seed, stream, options);
+}
+int mf_row_traffic_probe_sides(const mf_node* R, uint32_t n, void* p, void* q, uint32_t row_bytes, uint32_t item_row_bytes, uint32_t num_workers,
+                               uint64_t seed, void* stream, const mf_hogwild_options* options)
+{
     if (n == 0) return MF_OK;
     if (!R || !p || !q) return invalid("mf_row_traffic_probe: null pointer");
     if (row_bytes != 128 && row_bytes != 256 && row_bytes != 512) return invalid("mf_row_traffic_probe: row_bytes must be 128, 256 or 512 (got %u)", row_bytes);
+    if (item_row_bytes != 128 && item_row_bytes != 256 && item_row_bytes != 512) return invalid("mf_row_traffic_probe: row_bytes must be 128, 256 or 512 (got %u)", item_row_bytes);
     if (num_workers == 0) return invalid("mf_row_traffic_probe: num_workers must be positive");
     mf_hogwild_options o = {};
     if (options) o = *options;
@@ -607,9 +614,20 @@ int mf_row_traffic_probe(const mf_node* R, uint32_t n, void* p, void* q, uint32_
     uint8_t* RP = static_cast<uint8_t*>(o.user_replicas); uint8_t* RQ = static_cast<uint8_t*>(o.item_replicas);
     const uint64_t key = mix64(seed ^ 0x70726f6265ull);
 #define MF_PROBE(BYTES, COH) hipLaunchKernelGGL((row_traffic_probe_kernel<BYTES, COH>), grid, block, 0, as_stream(stream), R, n, P, Q, per_worker, user_keep, item_keep, o.user_slot, o.item_slot, o.user_slots, o.item_slots, RP, RQ, key, 0u)
-    if (row_bytes == 128) { if (coherent) MF_PROBE(2, true); else MF_PROBE(2, false); }
+#define MF_PROBE2(BP, BQ) hipLaunchKernelGGL((row_traffic_probe_kernel<BP, true, BQ>), grid, block, 0, as_stream(stream), R, n, P, Q, per_worker, user_keep, item_keep, o.user_slot, o.item_slot, o.user_slots, o.item_slots, RP, RQ, key, 0u)
+    if (row_bytes != item_row_bytes) {
+        // rows of different widths on the two sides: MASCOT after one side's groups have been promoted
+        if (!coherent) return invalid("mf_row_traffic_probe_sides: sides of different widths are probed with device-coherent stores only");
+        if (row_bytes == 256 && item_row_bytes == 512) MF_PROBE2(4, 8);
+        else if (row_bytes == 512 && item_row_bytes == 256) MF_PROBE2(8, 4);
+        else if (row_bytes == 128 && item_row_bytes == 256) MF_PROBE2(2, 4);
+        else if (row_bytes == 256 && item_row_bytes == 128) MF_PROBE2(4, 2);
+        else return invalid("mf_row_traffic_probe_sides: the wider side's rows must be twice the other's");
+    }
+    else if (row_bytes == 128) { if (coherent) MF_PROBE(2, true); else MF_PROBE(2, false); }
     else if (row_bytes == 256) { if (coherent) MF_PROBE(4, true); else MF_PROBE(4, false); }
     else { if (coherent) MF_PROBE(8, true); else MF_PROBE(8, false); }
+#undef MF_PROBE2
 #undef MF_PROBE
     return launch_status("mf_row_traffic_probe");
 }

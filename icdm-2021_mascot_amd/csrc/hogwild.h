@@ -67,10 +67,17 @@ __device__ __forceinline__ void process_chunk(Rule& rule, const Rating& my, cons
 // the compiler's wait-count bookkeeping fall back to "wait for everything", which turns the look-ahead into one
 // full memory latency per rating.  Ring slots start out with row ids nothing can match, so the first ratings
 // need no special case either.
+// A rule may look ahead by a different number of ratings in chunks of class 2 (kAheadClass2).
+template <class Rule, int CLS, class = void> struct ahead_of { static constexpr int value = Rule::kAhead; };
+template <class Rule> struct ahead_of<Rule, 2, std::void_t<decltype(Rule::kAheadClass2)>> { static constexpr int value = Rule::kAheadClass2; };
+// A rule may prepare a row whose loads have arrived before it is compared with older rows (arrive<CLS>).
+template <int CLS, class Rule, class Row> __device__ __forceinline__ auto row_arrived(const Rule& rule, Row& row, int) -> decltype(rule.template arrive<CLS>(row), void()) { rule.template arrive<CLS>(row); }
+template <int CLS, class Rule, class Row> __device__ __forceinline__ void row_arrived(const Rule&, Row&, long) {}
+
 template <class Rule, int CLS, bool HOT>
 __device__ __forceinline__ void process_full_chunk(Rule& rule, const Rating& my, const typename Rule::Prep& prep, uint32_t processed)
 {
-    constexpr int A = Rule::kAhead;
+    constexpr int A = ahead_of<Rule, CLS>::value;
     constexpr int S = Rule::kRing;
     static_assert(S >= 2 * A + 1 && kWave % S == 0, "the ring divides a full chunk");
     typename Rule::Row ring[S];
@@ -84,6 +91,7 @@ __device__ __forceinline__ void process_full_chunk(Rule& rule, const Rating& my,
     };
     auto step = [&](auto D, int j) {
         constexpr int d = decltype(D)::value;
+        row_arrived<CLS>(rule, ring[d], 0);
         static_for<0, A>([&](auto H) {
             constexpr int h = A - decltype(H)::value;          // A, A-1, ..., 1: newest wins
             constexpr int sh = (d - h + 2 * S) % S;

@@ -26,6 +26,9 @@ namespace mf {
 template <int K, bool COH, bool SAMPLED, bool MIXED = true> struct MascotRuleT {
     static constexpr int E = K / 64;                        // elements per lane
     static constexpr int kAhead = 3, kRing = 8;
+    // chunks of mixed precisions look two ratings ahead: their rows take three registers per side while in flight, and
+    // every rating compares with one older row less (measured: 3 % per mixed epoch over three ratings, 4 % over one)
+    static constexpr int kAheadClass2 = 2;
     // chunk classes: 1 = every rating of the chunk touches two binary16 rows (the state every group starts in): loads
     // and arithmetic without any branching; 2 = any mix of precisions, every rating inside the group tables: every
     // path through a rating issues the same number of memory instructions; 0 = anything, including ratings that are
@@ -184,54 +187,55 @@ template <int K, bool COH, bool SAMPLED, bool MIXED = true> struct MascotRuleT {
         }
     }
     // Chunks of mixed precisions (class 2): the same instructions for a row of either precision, so that a rating takes
-    // no branch on its way to the rows and the compiler can count the loads in flight.  Every access goes through two
-    // windows over the row, one per precision, of which the one that does not apply is closed (0 bytes): both
-    // instructions are issued, the hardware drops the one through the closed window (a dropped load returns zero).
+    // no branch on its way to the rows and the compiler can count the loads in flight.  Every access goes through a
+    // window over the row (a buffer resource of the row's size) twice, once with the instruction for each precision;
+    // the one that does not apply aims past the window and is dropped by the hardware (a dropped load returns zero).
     // A binary32 row is moved with 8-byte accesses (k = 128; 4-byte at k = 64), a binary16 row with 4-byte ones (2-byte).
-    struct Windows { row_window_t wide, narrow; };
-    static __device__ __forceinline__ Windows windows(uint64_t ptr, bool fp32)
+    static constexpr uint32_t kPast = 0x7ffff000u;       // a byte offset past every window
+    struct Access { row_window_t row; uint32_t wide, narrow; };      // this lane's byte offset for each precision's instruction
+    static __device__ __forceinline__ Access access(uint64_t ptr, bool fp32, int lane)
     {
-        return Windows{row_window(ptr, fp32 ? K * 4u : 0u), row_window(ptr, fp32 ? 0u : K * 2u)};
+        return Access{row_window(ptr, fp32 ? K * 4u : K * 2u), fp32 ? (uint32_t)lane * (E * 4u) : kPast, fp32 ? kPast : (uint32_t)lane * (E * 2u)};
     }
     static __device__ __forceinline__ void load_mixed(uint32_t* r, uint32_t& h, uint64_t ptr, bool fp32, int lane)
     {
-        const Windows w = windows(ptr, fp32);
+        const Access a = access(ptr, fp32, lane);
         if constexpr (E == 2) {
-            const auto v = __builtin_amdgcn_raw_buffer_load_b64(w.wide, lane * 8, 0, 0);
+            const auto v = __builtin_amdgcn_raw_buffer_load_b64(a.row, (int)a.wide, 0, 0);
             r[0] = v[0]; r[1] = v[1];
-            h = __builtin_amdgcn_raw_buffer_load_b32(w.narrow, lane * 4, 0, 0);
+            h = __builtin_amdgcn_raw_buffer_load_b32(a.row, (int)a.narrow, 0, 0);
         } else {
-            r[0] = __builtin_amdgcn_raw_buffer_load_b32(w.wide, lane * 4, 0, 0);
-            h = __builtin_amdgcn_raw_buffer_load_b16(w.narrow, lane * 2, 0, 0);
+            r[0] = __builtin_amdgcn_raw_buffer_load_b32(a.row, (int)a.wide, 0, 0);
+            h = __builtin_amdgcn_raw_buffer_load_b16(a.row, (int)a.narrow, 0, 0);
         }
     }
     template <bool C> static __device__ __forceinline__ void store_mixed(const uint32_t* r, uint64_t ptr, bool fp32, int lane)
     {
-        const Windows w = windows(ptr, fp32);
+        const Access a = access(ptr, fp32, lane);
         if constexpr (E == 2) {
-            window_store<C>(w.wide, (uint32_t)lane * 8u, (uint64_t)r[0] | ((uint64_t)r[1] << 32));
-            window_store<C>(w.narrow, (uint32_t)lane * 4u, r[0]);
+            window_store<C>(a.row, a.wide, (uint64_t)r[0] | ((uint64_t)r[1] << 32));
+            window_store<C>(a.row, a.narrow, r[0]);
         } else {
-            window_store<C>(w.wide, (uint32_t)lane * 4u, r[0]);
-            window_store<C>(w.narrow, (uint32_t)lane * 2u, (uint16_t)r[0]);
+            window_store<C>(a.row, a.wide, r[0]);
+            window_store<C>(a.row, a.narrow, (uint16_t)r[0]);
         }
     }
     // d: the change of this lane's elements in binary32; a binary16 row receives it rounded
     static __device__ __forceinline__ void add_mixed(uint64_t ptr, const float* d, bool fp32, int lane)
     {
-        const Windows w = windows(ptr, fp32);
+        const Access a = access(ptr, fp32, lane);
         if constexpr (E == 2) {
             float lower, upper;
-            const uint32_t at = halves_of_row(d, lower, upper, lane);
-            window_add(w.wide, at, lower);
-            window_add(w.wide, at + K * 2u, upper);
-            window_add(w.narrow, (uint32_t)lane * 4u, narrow(d));
+            const uint32_t at = fp32 ? halves_of_row(d, lower, upper, lane) : (halves_of_row(d, lower, upper, lane), kPast);
+            window_add(a.row, at, lower);
+            window_add(a.row, at + K * 2u, upper);
+            window_add(a.row, a.narrow, narrow(d));
         } else {
-            window_add(w.wide, (uint32_t)lane * 4u, d[0]);
+            window_add(a.row, a.wide, d[0]);
             // one element per lane: even lanes add the pair (own, right neighbour), odd lanes aim past the window
             const uint32_t mine = (uint32_t)bits(narrow(d));
             const uint32_t other = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)mine, 0xB1 /* quad_perm 1,0,3,2 */, 0xf, 0xf, false);
-            window_add(w.narrow, (lane & 1) ? 0x7ffffff0u : (uint32_t)lane * 2u, from_bits<half2_t>(mine | (other << 16)));
+            window_add(a.row, (lane & 1) ? kPast : a.narrow, from_bits<half2_t>(mine | (other << 16)));
         }
     }
     // hot row (Schedule::keep_u): add the change of this lane's elements to the row in memory
@@ -291,6 +295,11 @@ template <int K, bool COH, bool SAMPLED, bool MIXED = true> struct MascotRuleT {
             load_side(row.q, i.qptr, i.flags & 2u, lane);
         }
     }
+    // load_mixed: the row came through one of two windows, the other gave zero
+    template <int CLS> __device__ __forceinline__ void arrive(Row& row) const
+    {
+        if constexpr (CLS == 2) { row.p[0] |= row.ph; row.q[0] |= row.qh; }
+    }
     // selects, no branches: a branch here would sit between the row loads and their first use
     __device__ __forceinline__ void forward(Row& nxt, const Info& in, const Row& cur, const Info& ic) const
     {
@@ -301,11 +310,7 @@ template <int K, bool COH, bool SAMPLED, bool MIXED = true> struct MascotRuleT {
             nxt.p[e] = same_p ? cur.p[e] : nxt.p[e];
             nxt.q[e] = same_q ? cur.q[e] : nxt.q[e];
         }
-        // a row that has been updated is in p, q whatever its precision (update() merges ph, qh into them)
-        if constexpr (MIXED) {
-            nxt.ph = same_p ? 0u : nxt.ph;
-            nxt.qh = same_q ? 0u : nxt.qh;
-        }
+
     }
 
     // ---- reductions in the reference order ------------------------------------------------
@@ -450,9 +455,6 @@ template <int K, bool COH, bool SAMPLED, bool MIXED = true> struct MascotRuleT {
         const bool skip_p = CLS == 0 && HOT && (i.thin & 1u), skip_q = CLS == 0 && HOT && (i.thin & 2u);
         const bool sampled = SAMPLED && processed >= first_sample;
         const uint32_t ug = (i.flags >> 3) & 0x3fffu, ig = (i.flags >> 17) & 0x3fffu;
-        if constexpr (CLS == 2) {       // load_mixed: the row came through one of two windows, the other gave zero
-            row.p[0] |= row.ph; row.q[0] |= row.qh; row.ph = 0u; row.qh = 0u;
-        }
         if (!up && !ip) {
             // mascot_sgd_kernel.h:188-278: everything in binary16, one rounding per operation
             const HV lam_h = splat((half_t)lambda);

@@ -172,6 +172,10 @@ int mf_generate_ratings_host(const mf_synth_config* cfg, uint64_t seed, uint64_t
  * update kernel's time beside it. */
 int mf_row_traffic_probe(const mf_node* R, uint32_t n, void* p, void* q, uint32_t row_bytes, uint32_t num_workers,
                          uint64_t seed, void* stream, const mf_hogwild_options* options);
+/* The same with rows of different widths on the two sides (the wider twice the other: a MASCOT epoch after the groups of
+ * one side have been promoted to binary32); replica slots are as wide as their side's rows. */
+int mf_row_traffic_probe_sides(const mf_node* R, uint32_t n, void* p, void* q, uint32_t user_row_bytes, uint32_t item_row_bytes,
+                               uint32_t num_workers, uint64_t seed, void* stream, const mf_hogwild_options* options);
 /* Number of per-block columns mf_mascot_sgd_hogwild writes into norm_sum_p / norm_sum_q
  * (the reference's `block_num`, mf_methods.cu:109). */
 uint32_t mf_mascot_norm_blocks(uint32_t num_workers);
