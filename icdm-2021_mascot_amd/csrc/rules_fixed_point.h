@@ -182,7 +182,9 @@ __device__ __forceinline__ bool muppet_scale_index_plain(unsigned bitwidth, floa
 }
 // (signed char) of roundf(x * 2^n) when |x| is at most the extreme that a plain scale index n was taken from: the
 // product then lies inside (-128.5, 127.5) by more than 64 ulps of the extreme, so nothing saturates, x is a number,
-// and the conversion is an ordinary truncating cast
+// and the conversion is an ordinary truncating cast.  (A NaN element cannot reach it: the extrema are taken with the
+// IEEE 754-2019 maximum, which returns NaN when any element is one, and a NaN extreme takes the general path.  The cast
+// compiles to v_cvt_i32_f32, whose result is defined for every input in any case: NaN gives 0, excess saturates.)
 __device__ __forceinline__ int round_to_i8_in_range(float x, float s) { return (int)__builtin_fmaf(x, s, __builtin_copysignf(0x1.fffffep-2f, x)); }
 // Sum of an int over the 64 lanes as a wave-uniform value: rotations inside the rows, then the four row sums meet on
 // the scalar unit (integer addition: any order)

@@ -351,7 +351,9 @@ int mf_sort_by_count_ws(uint32_t* cnt, uint32_t* idx, uint32_t n, void* workspac
  * allocates and frees nothing and is asynchronous on `stream`.  At most mf_sort_by_count_static_max() = 1,048,576
  * counts; more are refused with MF_EINVAL.  All calls on one GPU share that array: calls that overlap on one GPU
  * (different streams, different host threads) race -- run them one after another.  Nothing in the array has to
- * start at zero between calls. */
+ * start at zero between calls.  The first call on a device asks the runtime for the address of that device's copy of the
+ * array (hipGetSymbolAddress, under a mutex): a caller that captures streams into graphs makes one call outside any
+ * capture first. */
 uint32_t mf_sort_by_count_static_max(void);
 int mf_sort_by_count_static(uint32_t* cnt, uint32_t* idx, uint32_t n, void* stream);
 /* matrix_reconst_gpu_triplet, preprocess_utils.h:28-36 (in place). */

@@ -614,15 +614,27 @@ static inline int f2i8_sat(float f)       /* float -> signed char; out-of-range 
     if (f < -128.0f) return -128;
     return (int)f;
 }
+/* Deliberate slips, for tests/test_oracle_mutants.py only: a build with -DORC_MUTATE=n (n = 1..8) puts one plausible
+ * mistake into this file, and every one of them must make a pin in tests/test_oracle_pins.py fail -- the evidence that
+ * the pins tell a right restatement from a nearly right one.  The normal build (ORC_MUTATE undefined) has none. */
+#ifndef ORC_MUTATE
+#define ORC_MUTATE 0
+#endif
 /* get_only_scaling_factor, muppet/muppet_sgd_kernel.h:7-18 (result then stored in an unsigned, :71-73,132-133) */
 static uint32_t muppet_scale_index(unsigned bitwidth, float max_v, float min_v)
 {
     if (max_v == 0 && min_v == 0) return f2u_sat(0.0f);
     float val = (float)(1 << (bitwidth - 1));
-    float max_val = (val - 1) + 0.5f;
-    float min_val = (-val) - 0.5f;
+    float max_val = (val - 1) + (ORC_MUTATE == 3 ? -0.5f : 0.5f);     /* slip 3: the half step of the upper bound with the wrong sign */
+    float min_val = (-val) - (ORC_MUTATE == 4 ? -0.5f : 0.5f);       /* slip 4: the half step of the lower bound with the wrong sign */
     float range_best = fminf(fabsf(max_val / max_v), fabsf(min_val / min_v));
+#if ORC_MUTATE == 1
+    return f2u_sat(ceilf(log2f(range_best)));                        /* slip 1: ceiling for floor */
+#elif ORC_MUTATE == 2
+    return f2u_sat(floorf(log2f(range_best)) + 1.0f);                /* slip 2: index one too large */
+#else
     return f2u_sat(floorf(log2f(range_best)));
+#endif
 }
 /* round-to-grid then binary16, muppet_sgd_kernel.h:174-181 */
 static inline float muppet_grid_h(float v, float s, float s_rev) { float a = v * s; float b = roundf(a); float c = b * s_rev; return rn16f(c); }
@@ -680,7 +692,11 @@ void orc_muppet_update(int k, float* p, float* q, float r, float lr, float lambd
     float gp[128], gq[128];
     if (backward_bits == 8) {
         float sq_rev = 1 / (sb * sb);
+#if ORC_MUTATE == 5
+        int ruv_i = f2i8_sat(ruv * sb);                              /* slip 5: the quantised error truncated, not rounded */
+#else
         int ruv_i = f2i8_sat(roundf(ruv * sb));
+#endif
         int lam_i = f2i8_sat(roundf(-1.0f * lambda * sb));
         for (int e = 0; e < k; e++) {
             int pi = f2i8_sat(roundf(p[e] * sb)), qi = f2i8_sat(roundf(q[e] * sb));
@@ -730,7 +746,11 @@ static float afp_scale_index(unsigned bitwidth, float max_v)
     if (max_v == 0) return 0;
     float denom = exp2f((float)(bitwidth - 1)) - 1;
     float ratio = max_v / denom;
+#if ORC_MUTATE == 6
+    return fabsf(floorf(log2f(ratio)));                              /* slip 6: floor for ceiling */
+#else
     return fabsf(ceilf(log2f(ratio)));
+#endif
 }
 static inline float afp_grid(float v, float s, float s_rev) { float a = v * s; float b = roundf(a); return b * s_rev; }
 
@@ -1163,11 +1183,12 @@ int orc_muppet_ladder_step(int k, int e, int* switched_epoch, int* precision_idx
     const int resolution_size = 3, gamma = 1;
     const float alpha = 1.0f, beta = 1.5f, lambda_for_threshold = 0.3f;
     float decaying_threshold = (float)(alpha + (beta * exp(-1 * lambda_for_threshold * (e))));
+    if (ORC_MUTATE == 7) decaying_threshold *= 0.9f;                 /* slip 7: a threshold 10 % lower */
     if (e - *switched_epoch >= resolution_size) {
         float sum_norms_resolution = 0, sum_updated_val_norm = 0;
         float acc[128];
         for (int i = 0; i < k; i++) acc[i] = 0;
-        for (int wi = e - resolution_size + 1; wi <= e; wi++) {
+        for (int wi = e - resolution_size + 1 + (ORC_MUTATE == 8 ? 1 : 0); wi <= e; wi++) {      /* slip 8: a window one epoch short */
             sum_norms_resolution += sum_norms_epoch[wi];
             for (int i = 0; i < k; i++) acc[i] += sum_updated_val_epoch[wi * k + i];
         }

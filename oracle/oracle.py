@@ -52,7 +52,9 @@ def _ptr(a):
 class Oracle:
     def __init__(self, soft=False):
         name = "liboracle_soft.so" if soft else "liboracle.so"
-        path = os.path.join(_BUILD, name)
+        # ORACLE_BUILD_DIR: a directory with another build of the checker (tests/test_oracle_mutants.py points the pin
+        # tests at builds with one deliberate mistake each)
+        path = os.path.join(os.environ.get("ORACLE_BUILD_DIR", _BUILD), name)
         if not os.path.exists(path):
             build()
         self.lib = lib = C.CDLL(path)

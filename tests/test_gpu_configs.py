@@ -3,11 +3,10 @@ reference rules run by the CPU checker as a 16-thread Hogwild loop on the same s
 its CPU twin), shuffle, initial model and windows.  The worker count is the one mf_train chooses and the hot-row
 treatment is the default one (rows with several updates in flight added to, or replicated per XCD), so these are the
 runs in which that treatment is active against a run of the reference rule close to its sequential limit.
-Bar: final test RMSE within 0.005 (BASELINE.json's north star).  The GPU run, with hundreds to thousands of updates in
-flight where the CPU run has 16, trails it by about half an epoch in the first epochs (0.08 after one epoch, 0.004
-after twelve at 10M ratings), a distance that shrinks with the slope of the curve; the runs here are as long as the
-CPU run's time allows (16 to 24 of the 50 configured epochs), the full 50 epochs at full size are held against the
-committed CPU curve by bench.py and tests/test_gpu_full_size.py."""
+Bar: test RMSE within 0.005 (BASELINE.json's north star) after ten epochs.  The GPU run, with hundreds to thousands of
+updates in flight where the CPU run has 16, trails it in the first epochs (0.04 after one epoch, 0.008 after five, 0.004
+after ten at 10M ratings), a distance that shrinks with the slope of the curve; the full 50 epochs at full size are held
+against the committed CPU curves by bench.py and tests/test_gpu_full_size.py."""
 import ctypes as C
 
 import numpy as np
@@ -61,7 +60,7 @@ def _run(orc, h, c, train, test, version, k, epochs, seed, **kw):
     return out["rmse"], ref
 
 
-@pytest.mark.parametrize("version,epochs", [(1, 20), (5, 16), (4, 16), (3, 16), (2, 16)])
+@pytest.mark.parametrize("version,epochs", [(1, 10), (5, 10), (4, 10), (3, 16), (2, 10)])
 def test_config4_shape_every_rule(orc, version, epochs):
     """Configuration 4 at one tenth: 48,000 x 1,780, 10M training ratings, item Zipf(1.1) (the most popular item takes a
     fifth of the ratings), user Zipf(0.8), integers 1-5; k = 128; MASCOT, fp32 SGD, MPT, MuPPET and AFP.  612 workers:
@@ -81,7 +80,7 @@ def test_config3_shape(orc, version, k):
     h = mfutil.hip()
     c, train, test = _dataset(orc, h, 3, 0.1, 7)
     assert train.size == 2_000_000
-    gpu, cpu = _run(orc, h, c, train, test, version, k, 24, 7)
+    gpu, cpu = _run(orc, h, c, train, test, version, k, 10 if k == 128 else 12, 7)
     assert np.all(np.isfinite(gpu)) and np.all(np.diff(gpu) < 0)
     assert abs(gpu[-1] - cpu[-1]) < TOL
 

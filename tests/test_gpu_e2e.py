@@ -159,6 +159,44 @@ def test_single_worker_mascot_run_is_the_checkers_run(orc, k):
     assert np.allclose(out["rmse"], ref, rtol=1e-6, atol=0)
 
 
+def test_version_6_is_the_mascot_run(tmp_path):
+    """-v 6 (mascot_training_mf_naive, mf_methods.cu:926-1301: the MASCOT kernel with the group search done from global
+    memory, mascot_sgd_kernel.h:460-820) has the schedule, arithmetic and epoch logic of -v 1 and runs the same path
+    here: with one worker (no races) mf_train leaves the same model, precisions and curve bit for bit, and the command
+    line writes the same <out>_reconst.txt."""
+    h = mfutil.hip()
+    n_users, n_items, k = 700, 300, 64
+    R = mfutil.make_ratings(61, n_users, n_items, 45_000, rank=8, alpha=1.0)
+    train, test = _split(R, 38_000)
+    runs = {}
+    for version in (1, 6):
+        prm = h.default_params(k=k, num_workers=1, epoch=9, learning_rate=0.01, lam=0.015, decay=0.1, version=version, seed=9,
+                               user_group_num=6, item_group_num=5, sample_ratio=0.05, interval=2, error_threshold=1.5)
+        p, q = h.init_model(n_users, n_items, k, 9)
+        out = h.train(prm, train, n_users, n_items, test, p, q)
+        runs[version] = (p, q, out)
+    (p1, q1, o1), (p6, q6, o6) = runs[1], runs[6]
+    assert np.array_equal(p1.view(np.uint32), p6.view(np.uint32)) and np.array_equal(q1.view(np.uint32), q6.view(np.uint32))
+    assert np.array_equal(o1["user_prec"], o6["user_prec"]) and np.array_equal(o1["item_prec"], o6["item_prec"])
+    assert o1["user_prec"].any() or o1["item_prec"].any(), "no group switched: the run does not reach the switching code"
+    assert np.array_equal(o1["rmse"], o6["rmse"]) and np.array_equal(o1["user2sorted"], o6["user2sorted"])
+    # the command line
+    assert os.path.exists(CLI), "quantized_mf is not built"
+    tr, te = str(tmp_path / "train.tsv"), str(tmp_path / "test.tsv")
+    _write_tsv(tr, train)
+    _write_tsv(te, test)
+    files = {}
+    for version in (1, 6):
+        out = str(tmp_path / ("model_v%d" % version))
+        cmd = [CLI, "-i", tr, "-y", te, "-o", out, "-v", str(version), "-k", str(k), "-l", "6", "-wg", "1", "-a", "0.01", "-b", "0.015",
+               "-d", "0.1", "-ug", "6", "-ig", "5", "-s", "0.05", "-it", "2", "-e", "1.5", "-seed", "9"]
+        res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=300)
+        assert res.returncode == 0, res.stderr
+        assert os.path.exists(out + "_reconst.txt") and not os.path.exists(out + ".txt")
+        files[version] = open(out + "_reconst.txt").read()
+    assert files[1] == files[6] and len(files[1].split("\n")[1].split()) == np.unique(train["u"]).size * k
+
+
 # AFP (-v 2) keeps its quantiser state per worker, not per row: a worker measures the range of one row and uses that
 # scale for the next `itv` ratings, whatever rows they touch, so the order in which racing workers' updates land
 # changes which scales saturate and the runs spread (final test RMSE 0.825 .. 0.833 over 16 runs of four workers,

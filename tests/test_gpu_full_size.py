@@ -150,7 +150,10 @@ def test_full_size_run_tracks_the_committed_cpu_curves():
     """mf_train -v 1 on configuration 4 at full size (the workload and parameters of bench.py and of the committed CPU
     curves, tests/golden/reference_curve_config4_run*.json: the reference rule run by the checker on host cores) for
     the configured 50 epochs with the library's defaults: every row update carried out, the test RMSE within 0.005 of
-    the CPU curves from epoch 12 on and at epoch 50, the figure BASELINE.json's metric names."""
+    the CPU curves from epoch 6 on and within 0.002 at epoch 50, the figure BASELINE.json's metric names.  The CPU curves
+    are the rule's sequential limit (6 threads); the GPU keeps 24,576 updates in flight, and a row that takes percents of
+    all ratings keeps one of the many updates in flight on it (as it would on the reference's GPU), which is what the first
+    epochs show: their bounds are the measured gaps (0.049, 0.021, 0.010, 0.008, 0.0045) plus a margin."""
     import glob
     import json
     sys.path.insert(0, ROOT)
@@ -168,6 +171,36 @@ def test_full_size_run_tracks_the_committed_cpu_curves():
     p, q = h.init_model(cfg.n_users, cfg.n_items, 128, 2021)
     gpu = h.train(prm, train, cfg.n_users, cfg.n_items, test, p, q)["rmse"]
     print("epoch 1, 5, 12, 25, 50: gpu", np.round(gpu[[0, 4, 11, 24, 49]], 5), "cpu", np.round(cpu[[0, 4, 11, 24, 49]], 5))
-    assert np.all(np.isfinite(gpu)) and np.all(np.diff(gpu[:30]) < 0)
-    assert np.all(np.abs(gpu[11:] - cpu[11:]) < 0.005)
+    assert np.all(np.isfinite(gpu)) and np.all(np.diff(gpu[:20]) < 0) and np.all(np.diff(gpu) < 2e-4)
+    for e, bound in enumerate((0.06, 0.028, 0.014, 0.011, 0.007)):
+        assert abs(gpu[e] - cpu[e]) < bound, (e + 1, gpu[e], cpu[e])
+    assert np.all(np.abs(gpu[5:] - cpu[5:]) < 0.005)
     assert abs(gpu[49] - cpu[49]) < 0.002
+
+
+@pytest.mark.parametrize("config,version,k,close_from,first", [(2, 1, 128, 10, 0.025), (3, 1, 128, 3, 0.03), (3, 1, 64, 3, 0.04), (3, 5, 128, 3, 0.03), (3, 4, 128, 3, 0.03)])
+def test_configs_2_and_3_track_the_committed_cpu_curves(config, version, k, close_from, first):
+    """BASELINE configurations 2 (8M ratings, MASCOT k = 128) and 3 (20M ratings; MASCOT at k = 128 and 64, fp32 SGD and MPT) at
+    full size, 50 epochs with the library's defaults (worker count from mf_auto_workers: 488 and 1220), against the committed
+    CPU curves of the same rule on the same ratings (tests/golden/reference_curve_config<N>*.json): within `first` after
+    the first epoch, within 0.005 from epoch `close_from` on (measured: 0.0035 at epoch 12 of configuration 2, 0.001
+    from epoch 5 on at configuration 3) and within 0.003 at epoch 50."""
+    sys.path.insert(0, ROOT)
+    import bench
+    h = mfutil.hip()
+    preset = h.synth_config(config)
+    cfg, train, test = bench.generate(h, config, 2021, preset.n_train, preset.n_test)
+    ref = bench.reference_curve(config, train.size, k, 2021, version)
+    assert ref is not None and ref["runs"] >= 1 and len(ref["mean"]) == 50
+    cpu = ref["mean"]
+    t = bench.TRAIN
+    prm = h.default_params(k=k, num_workers=0, epoch=t["epochs"], learning_rate=t["lr"], lam=t["lam"], decay=t["decay"], version=version, seed=2021,
+                           user_group_num=t["ug"], item_group_num=t["ig"], sample_ratio=t["sample_ratio"], interval=t["interval"],
+                           error_threshold=t["threshold"])
+    p, q = h.init_model(cfg.n_users, cfg.n_items, k, 2021, version == 4)       # -v 4 starts from a binary16-rounded model (main.cu:152-153)
+    gpu = h.train(prm, train, cfg.n_users, cfg.n_items, test, p, q)["rmse"]
+    print("epoch 1, 5, 12, 25, 50: gpu", np.round(gpu[[0, 4, 11, 24, 49]], 5), "cpu", np.round(cpu[[0, 4, 11, 24, 49]], 5))
+    assert np.all(np.isfinite(gpu))
+    assert abs(gpu[0] - cpu[0]) < first
+    assert np.all(np.abs(gpu[close_from - 1:] - cpu[close_from - 1:]) < 0.005)
+    assert abs(gpu[49] - cpu[49]) < 0.003
