@@ -1,6 +1,9 @@
 // quantized_mf: the reference's command line (main.cu:15-175) over libmascot_hip.
-// Same flags, same stdout lines, same model files.  Additions: `-seed <n>` (the reference seeds from
-// time(0) and clock(), so two of its runs never agree; here the default seed is fixed), `-cached <0|1>`
+// Same flags, the reference's stdout lines (plus two in the parameter echo, "Seed" and "Hot rows", for the two things
+// the reference does not have), same model files.  Additions: `-seed <n>` (the reference seeds from
+// time(0) and clock(), so two of its runs never agree; here the default seed is fixed), `-compat <0|1>` (1: `-wg`
+// counts updates in flight as it does in the reference, where a worker has one; a worker here keeps four, so the run
+// uses a quarter as many workers: mf_params.wg_counts_updates), `-cached <0|1>`
 // and `-split <n>` (row access policy and kernel launches per epoch, see include/mascot_hip.h), `-hot <0|1>`,
 // `-replicate <t>[,<merges>]` and `-thin <cap>[,<early cap>,<epochs>]` (how rows with several updates in flight are
 // treated: mf_params.hot_rows, replicate_inflight, hot_row_inflight; `-hot 0` is the reference's race semantics),
@@ -51,6 +54,7 @@ int main(int argc, const char* argv[])
             if (a == "-it" && has) prm.interval = std::atoi(argv[i + 1]);
             if (a == "-rc" && has) reconst_save = std::atoi(argv[i + 1]);
             if (a == "-seed" && has) prm.seed = std::strtoull(argv[i + 1], nullptr, 10);
+            if (a == "-compat" && has) prm.wg_counts_updates = std::atoi(argv[i + 1]) != 0;      // -wg counts updates in flight, as in the reference
             if (a == "-cached" && has) prm.cached_rows = std::atoi(argv[i + 1]);
             if (a == "-split" && has) prm.epoch_splits = std::atoi(argv[i + 1]);
             if (a == "-hot" && has) {            // 0: no hot rows at all, every row stored as the reference does; 1 (default): hot rows
@@ -95,7 +99,7 @@ int main(int argc, const char* argv[])
     std::cout << "Decay                       : " << prm.decay << std::endl;
     std::cout << "Lambda                      : " << prm.lambda << std::endl;
     std::cout << "Iteration                   : " << prm.epoch << std::endl;
-    std::cout << "Num of workers              : " << prm.num_workers << (prm.num_workers ? "" : " (chosen from the number of ratings)") << std::endl;
+    std::cout << "Num of workers              : " << prm.num_workers << (prm.num_workers ? (prm.wg_counts_updates ? " (updates in flight, as the reference counts)" : "") : " (chosen from the number of ratings)") << std::endl;
     std::cout << "Thread block size           : " << prm.thread_block_size << std::endl;
     std::cout << "Sample ratio                : " << prm.sample_ratio << std::endl;
     std::cout << "Error threshold             : " << prm.error_threshold << std::endl;

@@ -779,6 +779,12 @@ int make_run(const mf_params* params, const mf_node* R, uint32_t n, uint32_t n_u
     Run* run = (version == 1 || version == 6) ? static_cast<Run*>(new MascotRun) : static_cast<Run*>(new DenseRun);
     run->prm = *params;
     if (run->prm.num_workers == 0) run->prm.num_workers = mf_auto_workers(n);
+    else if (run->prm.wg_counts_updates) {
+        // -wg as the reference counts it: updates in flight.  A worker here keeps four ratings in flight (two for the
+        // fixed-point rules, whose pipeline looks one rating ahead).
+        const uint32_t per_worker = (version == 2 || version == 3) ? 2u : 4u;
+        run->prm.num_workers = run->prm.num_workers / per_worker ? run->prm.num_workers / per_worker : 1u;
+    }
     Common& c = run->c;
     c.prm = &run->prm; c.n = n; c.n_users = n_users; c.n_items = n_items; c.test_n = test_n; c.k = params->k; c.rep = report;
     if (report) { report->preprocess_ms = report->switching_ms = report->error_ms = report->sgd_ms = report->total_ms = 0; report->muppet_final_bits = 0; }

@@ -409,6 +409,11 @@ typedef struct {
                                  100M ratings the extra atomic adds cost 9 ms per epoch and gain 0.0007 test RMSE */
     float replica_step_scale; /* mf_hogwild_options::replica_step_scale.  < 0 (default): mf_replica_step_scale(learning_rate,
                                  mean rating); 0 = off (unscaled steps, mean of the changed copies) */
+    uint32_t wg_counts_updates; /* 0 (default): num_workers is the number of workers (wavefronts), each of which keeps four
+                                 ratings in flight (two for MuPPET and AFP), so -wg W puts 4 W updates in flight where the
+                                 reference's -wg W puts W.  1: num_workers is the reference's figure, the updates in
+                                 flight, and the run uses num_workers / 4 (/ 2) workers -- the reading under which the
+                                 reference's documented settings (-wg 2048, README.md:33) mean here what they mean there */
     uint32_t replica_step_epochs; /* the first epochs that use replica_step_scale; later ones run unscaled (default 1: the
                                  epoch in which every row grows from its small initial value and a replicated row, which
                                  keeps one of the many updates in flight on a copy, is furthest behind; afterwards the

@@ -179,7 +179,8 @@ def test_version_6_is_the_mascot_run(tmp_path):
     assert np.array_equal(p1.view(np.uint32), p6.view(np.uint32)) and np.array_equal(q1.view(np.uint32), q6.view(np.uint32))
     assert np.array_equal(o1["user_prec"], o6["user_prec"]) and np.array_equal(o1["item_prec"], o6["item_prec"])
     assert o1["user_prec"].any() or o1["item_prec"].any(), "no group switched: the run does not reach the switching code"
-    assert np.array_equal(o1["rmse"], o6["rmse"]) and np.array_equal(o1["user2sorted"], o6["user2sorted"])
+    # (the test RMSE is a sum of squares added with atomics: its last bits depend on the order)
+    assert np.allclose(o1["rmse"], o6["rmse"], rtol=1e-9, atol=0) and np.array_equal(o1["user2sorted"], o6["user2sorted"])
     # the command line
     assert os.path.exists(CLI), "quantized_mf is not built"
     tr, te = str(tmp_path / "train.tsv"), str(tmp_path / "test.tsv")

