@@ -28,7 +28,9 @@ template <int I, int N, class F> __device__ __forceinline__ void static_for(F&& 
     }
 }
 
-template <class Rule, int CLS, bool HOT>
+// SCALED: this launch gives the copies of replicated rows a longer step (Params::rep_scale != 1); otherwise the rules'
+// code for it is compiled out of the loop.
+template <class Rule, int CLS, bool HOT, bool SCALED>
 __device__ __forceinline__ void process_chunk(Rule& rule, const Rating& my, const typename Rule::Prep& prep, int n, uint32_t processed)
 {
     constexpr int A = Rule::kAhead;
@@ -56,7 +58,7 @@ __device__ __forceinline__ void process_chunk(Rule& rule, const Rating& my, cons
                     constexpr int sh = (d - h + 2 * S) % S;
                     if (j >= h) rule.forward(ring[d], inf[d], ring[sh], inf[sh]);
                 });
-                rule.template update<CLS, HOT>(ring[d], inf[d], processed + (uint32_t)j);
+                rule.template update<CLS, HOT, SCALED>(ring[d], inf[d], processed + (uint32_t)j);
             }
         });
     }
@@ -74,7 +76,7 @@ template <class Rule> struct ahead_of<Rule, 2, std::void_t<decltype(Rule::kAhead
 template <int CLS, class Rule, class Row> __device__ __forceinline__ auto row_arrived(const Rule& rule, Row& row, int) -> decltype(rule.template arrive<CLS>(row), void()) { rule.template arrive<CLS>(row); }
 template <int CLS, class Rule, class Row> __device__ __forceinline__ void row_arrived(const Rule&, Row&, long) {}
 
-template <class Rule, int CLS, bool HOT>
+template <class Rule, int CLS, bool HOT, bool SCALED>
 __device__ __forceinline__ void process_full_chunk(Rule& rule, const Rating& my, const typename Rule::Prep& prep, uint32_t processed)
 {
     constexpr int A = ahead_of<Rule, CLS>::value;
@@ -97,7 +99,7 @@ __device__ __forceinline__ void process_full_chunk(Rule& rule, const Rating& my,
             constexpr int sh = (d - h + 2 * S) % S;
             rule.forward(ring[d], inf[d], ring[sh], inf[sh]);
         });
-        rule.template update<CLS, HOT>(ring[d], inf[d], processed + (uint32_t)j);
+        rule.template update<CLS, HOT, SCALED>(ring[d], inf[d], processed + (uint32_t)j);
     };
     static_for<0, A>([&](auto D) { fetch_rows(D, decltype(D)::value); });
     for (int j0 = 0; j0 < kWave - S; j0 += S) {
@@ -206,16 +208,22 @@ void hogwild_kernel(Schedule s, typename Rule::Params prm)
             const int cls = rule.classify(my, prep, valid);
             // classes (see the rules): 1 and 2 promise ratings that all take the same memory instructions; full
             // chunks of those run the straight-line pipeline, everything else the general one
-            if (Rule::kClasses > 1 && cls == 1) {
-                if (n == kWave) process_full_chunk<Rule, 1, HOT>(rule, my, prep, processed);
-                else process_chunk<Rule, 1, HOT>(rule, my, prep, n, processed);
-            } else if (Rule::kClasses > 2 && cls == 2 && n == kWave) {
-                process_full_chunk<Rule, 2, HOT>(rule, my, prep, processed);
-            } else if (Rule::kClasses == 1 && n == kWave) {
-                process_full_chunk<Rule, 0, HOT>(rule, my, prep, processed);
-            } else {
-                process_chunk<Rule, 0, HOT>(rule, my, prep, n, processed);
-            }
+            auto run = [&](auto Scaled) {
+                constexpr bool SC = decltype(Scaled)::value;
+                if (Rule::kClasses > 1 && cls == 1) {
+                    if (n == kWave) process_full_chunk<Rule, 1, HOT, SC>(rule, my, prep, processed);
+                    else process_chunk<Rule, 1, HOT, SC>(rule, my, prep, n, processed);
+                } else if (Rule::kClasses > 2 && cls == 2 && n == kWave) {
+                    process_full_chunk<Rule, 2, HOT, SC>(rule, my, prep, processed);
+                } else if (Rule::kClasses == 1 && n == kWave) {
+                    process_full_chunk<Rule, 0, HOT, SC>(rule, my, prep, processed);
+                } else {
+                    process_chunk<Rule, 0, HOT, SC>(rule, my, prep, n, processed);
+                }
+            };
+            // the few launches with longer steps on replicated rows (the first epoch by default) take their own copy of
+            // the loops, so that every other launch pays nothing for them
+            if (HOT && prm.rep_scale != 1.0f) run(std::true_type()); else run(std::false_type());
             if (!more) break;
             processed = nprocessed; c = nc; ite = nite; start = nstart; n = nn; my = nmy;
         }

@@ -447,7 +447,7 @@ template <int K, bool COH, bool SAMPLED, bool MIXED = true> struct MascotRuleT {
             else store_side(r, ptr, fp32, lane);
         }
     }
-    template <int CLS, bool HOT> __device__ __forceinline__ void update(Row& row, const Info& i, uint32_t processed) const
+    template <int CLS, bool HOT, bool SCALED> __device__ __forceinline__ void update(Row& row, const Info& i, uint32_t processed) const
     {
         if (CLS == 0 && (i.flags & kSkip)) return;
         const bool up = CLS != 1 && (i.flags & 1u), ip = CLS != 1 && (i.flags & 2u);
@@ -459,7 +459,7 @@ template <int K, bool COH, bool SAMPLED, bool MIXED = true> struct MascotRuleT {
             // mascot_sgd_kernel.h:188-278: everything in binary16, one rounding per operation
             const HV lam_h = splat((half_t)lambda);
             // the step of each side: a replicated row's copy (thin bit 4 / 5) takes the longer one
-            const HV lr_p = half_pair((HOT && (i.thin & 16u)) ? lr_rep_h_bits : lr_h_bits), lr_q = half_pair((HOT && (i.thin & 32u)) ? lr_rep_h_bits : lr_h_bits);
+            const HV lr_p = half_pair((SCALED && (i.thin & 16u)) ? lr_rep_h_bits : lr_h_bits), lr_q = half_pair((SCALED && (i.thin & 32u)) ? lr_rep_h_bits : lr_h_bits);
             const half_t r_h = (half_t)i.r;
             const HV P = from_bits<HV>(row.p[0]), Q = from_bits<HV>(row.q[0]);
             const half_t dot = dot_half(P * Q);
@@ -496,7 +496,7 @@ template <int K, bool COH, bool SAMPLED, bool MIXED = true> struct MascotRuleT {
 #pragma unroll
             for (int e = 0; e < E; ++e) m[e] = pf[e] * qf[e];
             const float ruv = i.r - dot_float(m);
-            const float lr_p = (HOT && (i.thin & 16u)) ? lrate_rep : lrate, lr_q = (HOT && (i.thin & 32u)) ? lrate_rep : lrate;
+            const float lr_p = (SCALED && (i.thin & 16u)) ? lrate_rep : lrate, lr_q = (SCALED && (i.thin & 32u)) ? lrate_rep : lrate;
             float gp[E], gq[E], np_[E], nq_[E];
 #pragma unroll
             for (int e = 0; e < E; ++e) {

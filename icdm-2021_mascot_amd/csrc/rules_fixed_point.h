@@ -390,13 +390,14 @@ template <int K, bool COH> struct MuppetRule : DenseBase<K, COH> {
         }
         return true;
     }
-    template <int CLS, bool HOT> __device__ __forceinline__ void update(Row& row, const Info& i, uint32_t processed)
+    template <int CLS, bool HOT, bool SCALED> __device__ __forceinline__ void update(Row& row, const Info& i, uint32_t processed)
     {
         float gbp[E], gbq[E], g_scale, d_scale;
         if (!(plain_8bit && gradients_8bit_plain(row.p, row.q, i.r, gbp, gbq, g_scale, d_scale)))
             gradients(row.p, row.q, i.r, gbp, gbq, g_scale, d_scale);
-        // d_scale carries the learning rate: a replicated row's copy takes a longer step (DenseBase::rep_scale)
-        const float ds_p = HOT ? this->step_of(d_scale, i.thin, 16u) : d_scale, ds_q = HOT ? this->step_of(d_scale, i.thin, 32u) : d_scale;
+        // d_scale carries the learning rate: a replicated row's copy takes a longer step (DenseBase::rep_scale; the factor
+        // is 1 everywhere else, and a product by 1 is exact)
+        const float ds_p = SCALED ? d_scale * this->scale_of(i.thin, 16u) : d_scale, ds_q = SCALED ? d_scale * this->scale_of(i.thin, 32u) : d_scale;
         float dp[E], dq[E];
 #pragma unroll
         for (int e = 0; e < E; ++e) {
@@ -539,7 +540,7 @@ template <int K, bool COH> struct AfpRule : DenseBase<K, COH> {
         q.r = ufirst(q.r); q.n = ufirst(q.n); q.itv = ufirst(q.itv); q.mov_avg_range = ufirst(q.mov_avg_range);
         return q;
     }
-    template <int CLS, bool HOT> __device__ __forceinline__ void update(Row& row, const Info& i, uint32_t)
+    template <int CLS, bool HOT, bool SCALED> __device__ __forceinline__ void update(Row& row, const Info& i, uint32_t)
     {
         const float* p = row.p; const float* q = row.q;
         float p_abs = fabsf(p[0]), q_abs = fabsf(q[0]);
@@ -620,8 +621,9 @@ template <int K, bool COH> struct AfpRule : DenseBase<K, COH> {
                 gbq[e] = (float)(half_t)(ph * t_ruv + qh * t_lam16);
             }
         }
-        // d_scale carries the learning rate: a replicated row's copy takes a longer step (DenseBase::rep_scale)
-        const float ds_p = HOT ? this->step_of(d_scale, i.thin, 16u) : d_scale, ds_q = HOT ? this->step_of(d_scale, i.thin, 32u) : d_scale;
+        // d_scale carries the learning rate: a replicated row's copy takes a longer step (DenseBase::rep_scale; the factor
+        // is 1 everywhere else, and a product by 1 is exact)
+        const float ds_p = SCALED ? d_scale * this->scale_of(i.thin, 16u) : d_scale, ds_q = SCALED ? d_scale * this->scale_of(i.thin, 32u) : d_scale;
         float dp[E], dq[E];
 #pragma unroll
         for (int e = 0; e < E; ++e) {

@@ -32,8 +32,11 @@ template <int K, bool COH> struct DenseBase {
     float* RQ;
     float rep_scale;   // an update of a replicated row's copy takes a step this many times as long (Params::rep_scale)
     int lane;
-    // the step factor of one side of a rating: bit = 16 (user row) or 32 (item row) of Info::thin marks a replicated row
-    __device__ __forceinline__ float step_of(float lrate, uint32_t thin, uint32_t bit) const { return (thin & bit) ? lrate * rep_scale : lrate; }
+    float lrate_rep;   // learning rate x rep_scale, for the rules whose learning rate is one number
+    // the step factor of one side of a rating: bit = 16 (user row) or 32 (item row) of Info::thin marks a replicated row.
+    // Selects between two wave-uniform numbers: scalar instructions.
+    __device__ __forceinline__ float step_of(float lrate, uint32_t thin, uint32_t bit) const { return (thin & bit) ? lrate_rep : lrate; }
+    __device__ __forceinline__ float scale_of(uint32_t thin, uint32_t bit) const { return (thin & bit) ? rep_scale : 1.0f; }
 
     __device__ __forceinline__ Prep prepare(const Rating&, bool) const { return Prep(); }
     __device__ __forceinline__ int classify(const Rating&, const Prep&, bool) const { return 0; }
@@ -144,16 +147,16 @@ template <int K, bool COH> struct SgdRule : DenseBase<K, COH> {
     __device__ __forceinline__ void init(const Params& a, uint8_t*, int lane_, uint32_t)
     {
         this->P = a.p; this->Q = a.q; this->RP = static_cast<float*>(a.rep_p); this->RQ = static_cast<float*>(a.rep_q);
-        this->lane = lane_; lrate = a.lrate; lambda = a.lambda; this->rep_scale = a.rep_scale;
+        this->lane = lane_; lrate = a.lrate; lambda = a.lambda; this->rep_scale = a.rep_scale; this->lrate_rep = a.lrate * a.rep_scale;
     }
-    template <int CLS, bool HOT> __device__ __forceinline__ void update(Row& row, const Info& i, uint32_t) const
+    template <int CLS, bool HOT, bool SCALED> __device__ __forceinline__ void update(Row& row, const Info& i, uint32_t) const
     {
         float m[E];
 #pragma unroll
         for (int e = 0; e < E; ++e) m[e] = row.p[e] * row.q[e];
         const float dot = dot_reference_order<E, float>(m);
         const float ruv = i.r - dot;
-        const float lr_p = HOT ? this->step_of(lrate, i.thin, 16u) : lrate, lr_q = HOT ? this->step_of(lrate, i.thin, 32u) : lrate;
+        const float lr_p = SCALED ? this->step_of(lrate, i.thin, 16u) : lrate, lr_q = SCALED ? this->step_of(lrate, i.thin, 32u) : lrate;
         float dp[E], dq[E];
 #pragma unroll
         for (int e = 0; e < E; ++e) {
@@ -183,12 +186,12 @@ template <int K, bool COH> struct MptRule : DenseBase<K, COH> {
     __device__ __forceinline__ void init(const Params& a, uint8_t*, int lane_, uint32_t)
     {
         this->P = a.p; this->Q = a.q; this->RP = static_cast<float*>(a.rep_p); this->RQ = static_cast<float*>(a.rep_q);
-        this->lane = lane_; lrate = a.lrate; this->rep_scale = a.rep_scale;
+        this->lane = lane_; lrate = a.lrate; this->rep_scale = a.rep_scale; this->lrate_rep = a.lrate * a.rep_scale;
         scaling_factor_rev = 1 / a.scaling_factor;
         scaling_factor_h = (half_t)a.scaling_factor;
         lambda_h = from_bits<half_t>(a.scaled_lambda_half);
     }
-    template <int CLS, bool HOT> __device__ __forceinline__ void update(Row& row, const Info& i, uint32_t) const
+    template <int CLS, bool HOT, bool SCALED> __device__ __forceinline__ void update(Row& row, const Info& i, uint32_t) const
     {
         const half_t r_h = (half_t)i.r;
         half_t ph[E], qh[E], m[E];
@@ -196,7 +199,7 @@ template <int K, bool COH> struct MptRule : DenseBase<K, COH> {
         for (int e = 0; e < E; ++e) { ph[e] = (half_t)row.p[e]; qh[e] = (half_t)row.q[e]; m[e] = ph[e] * qh[e]; }
         const half_t dot = dot_reference_order<E, half_t>(m);
         const half_t ruv = scaling_factor_h * (r_h - dot);
-        const float lr_p = HOT ? this->step_of(lrate, i.thin, 16u) : lrate, lr_q = HOT ? this->step_of(lrate, i.thin, 32u) : lrate;
+        const float lr_p = SCALED ? this->step_of(lrate, i.thin, 16u) : lrate, lr_q = SCALED ? this->step_of(lrate, i.thin, 32u) : lrate;
         float dp[E], dq[E];
 #pragma unroll
         for (int e = 0; e < E; ++e) {
@@ -227,12 +230,12 @@ template <int K, bool COH> struct MemQuantRule {
     static constexpr int kAhead = 3, kRing = 8;
     static constexpr bool kSplittable = true;
     struct Params { uint16_t* p; uint16_t* q; float lrate; float lambda; bool accumulate; void* rep_p; void* rep_q; float rep_scale; };
-    uint16_t* P; uint16_t* Q; uint16_t* RP; uint16_t* RQ; float lrate, lambda, rep_scale; int lane;
+    uint16_t* P; uint16_t* Q; uint16_t* RP; uint16_t* RQ; float lrate, lambda, lrate_rep; int lane;
 
     __device__ __forceinline__ void init(const Params& a, uint8_t*, int lane_, uint32_t)
     {
         P = a.p; Q = a.q; RP = static_cast<uint16_t*>(a.rep_p); RQ = static_cast<uint16_t*>(a.rep_q); lrate = a.lrate; lambda = a.lambda; lane = lane_;
-        rep_scale = a.rep_scale;
+        lrate_rep = a.lrate * a.rep_scale;
     }
     // a replica slot is k * 4 bytes for every rule; a binary16 row fills its first half
     static __device__ __forceinline__ uint16_t* row_of(uint16_t* matrix, uint16_t* replicas, uint32_t row)
@@ -313,7 +316,7 @@ template <int K, bool COH> struct MemQuantRule {
         s = reduce_row16(s, OpAdd());
         return step_xor32(s, OpAdd());
     }
-    template <int CLS, bool HOT> __device__ __forceinline__ void update(Row& row, const Info& i, uint32_t) const
+    template <int CLS, bool HOT, bool SCALED> __device__ __forceinline__ void update(Row& row, const Info& i, uint32_t) const
     {
         float pf[E], qf[E];
         widen(pf, row.p); widen(qf, row.q);
@@ -325,7 +328,7 @@ template <int K, bool COH> struct MemQuantRule {
         }
         const float ruv = i.r - dot;
         // a replicated row's copy takes a longer step (Params::rep_scale)
-        const float lr_p = (HOT && (i.thin & 16u)) ? lrate * rep_scale : lrate, lr_q = (HOT && (i.thin & 32u)) ? lrate * rep_scale : lrate;
+        const float lr_p = (SCALED && (i.thin & 16u)) ? lrate_rep : lrate, lr_q = (SCALED && (i.thin & 32u)) ? lrate_rep : lrate;
         float dp[E], dq[E], np[E], nq[E];
 #pragma unroll
         for (int e = 0; e < E; ++e) {
