@@ -369,7 +369,7 @@ def main():
         s2.close()
         res = {"note": note, "value": n_train / (leg_ms / 1e3), "unit": "ratings/s", "ms_per_step": leg_ms, "workers": W,
                "roofline_frac": updates * (12 + 4 * row) / (leg_ms / 1e3) / 1e9 / PEAK_HBM_GBS,
-               "test_rmse_after_timed_epochs": r["rmse"][-1], "epochs": epochs_w + epochs_k}
+               "test_rmse_after_timed_epochs": r["rmse"][-1], "epochs": epochs_w + epochs_k, "test_rmse_per_epoch": [round(float(x), 5) for x in r["rmse"]]}
         if probe is not None:
             res["access_pattern_ceiling_ms"] = probe
         return res

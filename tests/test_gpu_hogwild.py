@@ -204,7 +204,9 @@ def test_afp_special_values(orc, k):
     assert _same_values(gq, Q)
 
 
-def _mascot_case(orc, k, W, uc, window, user_groups, item_groups, prec_mode, first_sample, seed, lr=LR):
+def _mascot_case(orc, k, W, uc, window, user_groups, item_groups, prec_mode, first_sample, seed, lr=LR, row_classes=None, all_binary16=0, step_scale=0.0):
+    """row_classes: keep-table values drawn at random per row (mf_hogwild_options); with them the call goes through the
+    _opt entry point, with the all_binary16 hint and the step factor of replicated rows' copies as given."""
     import torch
     h = mfutil.hip()
     R, starts, P, Q = mfutil.conflict_free_problem(seed, k, W, uc, window)
@@ -225,10 +227,18 @@ def _mascot_case(orc, k, W, uc, window, user_groups, item_groups, prec_mode, fir
     d_gsq = torch.zeros(item_groups * k, dtype=torch.float32, device="cuda")
     d_nsp = torch.full((user_groups * nb,), -3.0, dtype=torch.float32, device="cuda")
     d_nsq = torch.full((item_groups * nb,), -3.0, dtype=torch.float32, device="cuda")
-    h.mf_mascot_sgd_hogwild(dR.data_ptr(), R.size, dp.ptrs.data_ptr(), dq.ptrs.data_ptr(), k, W, uc, window, lr, LAM,
-                            dp.end.data_ptr(), dq.end.data_ptr(), dp.prec.data_ptr(), dq.prec.data_ptr(),
-                            d_gsp.data_ptr(), d_gsq.data_ptr(), d_nsp.data_ptr(), d_nsq.data_ptr(),
-                            first_sample, user_groups, item_groups, 0, 0, dS.data_ptr(), mfutil.stream_ptr())
+    args = (dR.data_ptr(), R.size, dp.ptrs.data_ptr(), dq.ptrs.data_ptr(), k, W, uc, window, lr, LAM,
+            dp.end.data_ptr(), dq.end.data_ptr(), dp.prec.data_ptr(), dq.prec.data_ptr(),
+            d_gsp.data_ptr(), d_gsq.data_ptr(), d_nsp.data_ptr(), d_nsq.data_ptr(),
+            first_sample, user_groups, item_groups, 0, 0, dS.data_ptr(), mfutil.stream_ptr())
+    if row_classes is None and not all_binary16:
+        h.mf_mascot_sgd_hogwild(*args)
+    else:
+        values = np.array(row_classes if row_classes is not None else [255], np.uint8)
+        keep = [values[rng.integers(0, values.size, n)] for n in (n_users, n_items)] if row_classes is not None else [None, None]
+        opt = mfutil.HogwildOptions(k, keep[0], keep[1], launches=2, step_scale=step_scale)
+        opt.o.all_binary16 = all_binary16
+        h.mf_mascot_sgd_hogwild_opt(*args, opt.ptr)
     torch.cuda.synchronize()
     gsp, gsq = np.zeros(user_groups * k, np.float32), np.zeros(item_groups * k, np.float32)
     nsp, nsq = np.zeros(user_groups, np.float32), np.zeros(item_groups, np.float32)
@@ -258,6 +268,21 @@ def test_mascot_bit_exact(orc, k, prec_mode):
         assert nsp.sum() > 0 and nsq.sum() > 0
     if prec_mode == "float":
         assert nsp.sum() == 0 and nsq.sum() == 0
+
+
+@pytest.mark.parametrize("k", [64, 128])
+@pytest.mark.parametrize("prec_mode", ["half", "mixed", "float"])
+def test_mascot_row_classes_and_hints_keep_the_checkers_result(orc, k, prec_mode):
+    """The straight-line path for chunks of mixed precisions and the kernel build for all-binary16 runs with the hot-row
+    code in them.  Every worker owns its rows, so a replicated row (253) changes in one XCD's copy only and the merge
+    returns that copy: with ordinary and replicated rows mixed at random the result is the checker's, bit for bit --
+    whatever the all_binary16 hint says (a wrong hint sends mixed chunks down the general path: slower, not different),
+    and with a step factor for the copies as long as the launch is one workgroup (one copy in play: factor 1)."""
+    W, uc, window = 12, 3, 128
+    for hint in (0, 1):
+        _mascot_case(orc, k, W, uc, window, 7, 5, prec_mode, first_sample=2 * window - 40, seed=150 + k, row_classes=(255, 253), all_binary16=hint)
+        _mascot_case(orc, k, W, uc, window, 7, 5, prec_mode, first_sample=uc * window, seed=151 + k, all_binary16=hint)
+    _mascot_case(orc, k, 4, uc, window, 7, 5, prec_mode, first_sample=2 * window - 40, seed=152 + k, row_classes=(255, 253), step_scale=4.0)
 
 
 @pytest.mark.parametrize("k", [64, 128])
