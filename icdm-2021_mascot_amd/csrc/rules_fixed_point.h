@@ -117,15 +117,35 @@ struct OpMinimum { __device__ __forceinline__ float operator()(float a, float b)
 // rows 0 (lanes 0-15), of c in row 1, of b in row 2 and of d in row 3.  v_permlane32_swap(a, b) leaves [a.lower, b.lower]
 // and [a.upper, b.upper], whose maximum folds the half-waves of a into the lower half and those of b into the upper
 // half; v_permlane16_swap folds the rows the same way; four rotations finish inside the rows.
+//
+// The maximum is fmaxf's, as in the reference: a NaN operand is dropped (v_max_f32 with the IEEE mode bit set, which
+// compute kernels run with; denormals are kept).  Written as instructions because the compiler puts a canonicalising
+// v_max_f32 x, x in front of every fmaxf whose operand comes out of a cross-lane move and cannot fold the rotation
+// into the maximum then, and the IEEE 754-2019 maximum it can use instead has no form that rotates: 10 vector
+// instructions here, 14 with that one.  The wait states that cross-lane reads of a just-written register need are inside
+// the block (the compiler does not count instructions in one): the first for whatever produced the inputs, the last
+// for whatever reads the result.
 __device__ __forceinline__ float max4_by_rows(float a, float b, float c, float d)
 {
-    auto ab = __builtin_amdgcn_permlane32_swap(bits(a), bits(b), false, false);
-    auto cd = __builtin_amdgcn_permlane32_swap(bits(c), bits(d), false, false);
-    const float x = OpMaximum()(from_bits<float>(ab[0]), from_bits<float>(ab[1]));      // rows 0,1: a   rows 2,3: b
-    const float y = OpMaximum()(from_bits<float>(cd[0]), from_bits<float>(cd[1]));      // rows 0,1: c   rows 2,3: d
-    auto xy = __builtin_amdgcn_permlane16_swap(bits(x), bits(y), false, false);          // [x.r0 y.r0 x.r2 y.r2], [x.r1 y.r1 x.r3 y.r3]
-    const float z = OpMaximum()(from_bits<float>(xy[0]), from_bits<float>(xy[1]));
-    return reduce_row16(z, OpMaximum());
+    asm("s_nop 1\n\t"
+        "v_permlane32_swap_b32 %0, %1\n\t"
+        "v_permlane32_swap_b32 %2, %3\n\t"
+        "v_max_f32 %0, %0, %1\n\t"                                                       // rows 0,1: a   rows 2,3: b
+        "v_max_f32 %2, %2, %3\n\t"                                                       // rows 0,1: c   rows 2,3: d
+        "s_nop 1\n\t"
+        "v_permlane16_swap_b32 %0, %2\n\t"                                               // [x.r0 y.r0 x.r2 y.r2], [x.r1 y.r1 x.r3 y.r3]
+        "v_max_f32 %0, %0, %2\n\t"
+        "s_nop 1\n\t"
+        "v_max_f32_dpp %0, %0, %0 row_ror:8 row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\t"
+        "v_max_f32_dpp %0, %0, %0 row_ror:4 row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\t"
+        "v_max_f32_dpp %0, %0, %0 row_ror:2 row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\t"
+        "v_max_f32_dpp %0, %0, %0 row_ror:1 row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1"
+        : "+v"(a), "+v"(b), "+v"(c), "+v"(d));
+    return a;
 }
 // get_only_scaling_factor (muppet_sgd_kernel.h:7-18) for two value ranges at once.  `extreme` holds, by half-wave, the
 // largest value (lower) and the negated smallest value (upper) of a range, the same in both rows of a half-wave or a
@@ -182,9 +202,9 @@ __device__ __forceinline__ bool muppet_scale_index_plain(unsigned bitwidth, floa
 }
 // (signed char) of roundf(x * 2^n) when |x| is at most the extreme that a plain scale index n was taken from: the
 // product then lies inside (-128.5, 127.5) by more than 64 ulps of the extreme, so nothing saturates, x is a number,
-// and the conversion is an ordinary truncating cast.  (A NaN element cannot reach it: the extrema are taken with the
-// IEEE 754-2019 maximum, which returns NaN when any element is one, and a NaN extreme takes the general path.  The cast
-// compiles to v_cvt_i32_f32, whose result is defined for every input in any case: NaN gives 0, excess saturates.)
+// and the conversion is an ordinary truncating cast.  (A NaN element does reach it: the extrema drop NaNs, as fmaxf and
+// fminf do in the reference.  The cast compiles to v_cvt_i32_f32, whose result is defined for every input: NaN gives 0,
+// which is what the reference's cast gives, and excess saturates.)
 __device__ __forceinline__ int round_to_i8_in_range(float x, float s) { return (int)__builtin_fmaf(x, s, __builtin_copysignf(0x1.fffffep-2f, x)); }
 // Sum of an int over the 64 lanes as a wave-uniform value: rotations inside the rows, then the four row sums meet on
 // the scalar unit (integer addition: any order)

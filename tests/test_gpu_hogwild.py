@@ -107,12 +107,17 @@ def test_afp_bit_exact(orc, k, afp_epoch):
     assert np.array_equal(gq.view(np.uint32), Q.view(np.uint32))
 
 
-def _special_rows(seed, k):
+def _special_rows(seed, k, nan_elements=False):
     """A conflict-free problem whose workers own rows with special contents: all zeros (scale index 0 by definition),
     huge values (the int8 conversion saturates), infinities (a ratio of 0, whose logarithm is -inf), exact .5 ties
-    after scaling (roundf's halves away from zero) and tiny values (scale indices near 100)."""
-    W, uc, window = 6, 1, 128
+    after scaling (roundf's halves away from zero) and tiny values (scale indices near 100).  nan_elements: a seventh
+    worker whose otherwise ordinary rows hold a NaN element each (the extrema drop it, as fmaxf does; its int8 value
+    is 0)."""
+    W, uc, window = 7 if nan_elements else 6, 1, 128
     R, starts, P, Q = mfutil.conflict_free_problem(seed, k, W, uc, window)
+    if nan_elements:
+        up, ip = P.shape[0] // W, Q.shape[0] // W
+        P[6 * up:7 * up:2, 5] = np.nan; Q[6 * ip:7 * ip:3, k - 3] = np.nan
     up, ip = P.shape[0] // W, Q.shape[0] // W
     P[1 * up] = 0.0; Q[1 * ip] = 0.0; P[1 * up + 1] = 0.0
     P[2 * up, ::3] = 1e30; Q[2 * ip, 1::5] = -3e29
@@ -178,7 +183,7 @@ def test_muppet_special_values(orc, k, bits):
     ties, very small values): the kernel uses the hardware's conversions, the checker spells CUDA's cast rules out."""
     import torch
     h = mfutil.hip()
-    R, starts, P, Q, uc, window = _special_rows(700 + k + bits, k)
+    R, starts, P, Q, uc, window = _special_rows(700 + k + bits, k, nan_elements=True)
     W = starts.shape[1]
     dR, dS, dP, dQ = to_dev(R), to_dev(starts), to_dev(P), to_dev(Q)
     d_sum = torch.zeros(k, dtype=torch.float32, device="cuda")
