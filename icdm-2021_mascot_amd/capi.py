@@ -17,6 +17,7 @@ SIGNATURES = {
     "mf_version": (i32, []),
     "mf_last_error": (C.c_char_p, []),
     "mf_hogwild_inflight": (f32, [u32, i32, u32, u32, u32]),
+    "mf_hogwild_inflight_capped": (f32, [u32, i32, u32, u32, u32, u32]),
     "mf_mascot_norm_blocks": (u32, [u32]),
     "mf_update_count": (u32, [u32, u32, u32]),
     "mf_auto_workers": (u32, [u32]),
@@ -96,13 +97,14 @@ class MfParams(C.Structure):
                 ("interval", u32), ("user_group_num", u32), ("item_group_num", u32), ("k", u32), ("num_workers", u32),
                 ("epoch", u32), ("thread_block_size", u32), ("version", u32), ("is_yahoo", u32), ("seed", u64),
                 ("verbose", u32), ("cached_rows", u32), ("epoch_splits", u32), ("hot_row_inflight", f32), ("hot_row_inflight_early", f32), ("hot_row_early_epochs", u32),
-                ("hot_rows", u32), ("replicate_inflight", f32), ("replica_merges", u32), ("replica_add_inflight", f32), ("replica_step_scale", f32), ("wg_counts_updates", u32), ("replica_step_epochs", u32)]
+                ("hot_rows", u32), ("replicate_inflight", f32), ("replica_merges", u32), ("replica_add_inflight", f32), ("replica_step_scale", f32), ("wg_counts_updates", u32), ("replica_step_epochs", u32),
+                ("early_inflight", f32), ("early_inflight_epochs", u32)]
 
 
 class HogwildOptions(C.Structure):
     """mf_hogwild_options of include/mascot_hip.h."""
     _fields_ = [("cached_rows", u32), ("launches", u32), ("user_keep", vp), ("item_keep", vp), ("user_slot", vp), ("item_slot", vp),
-                ("user_slot_row", vp), ("item_slot_row", vp), ("user_replicas", vp), ("item_replicas", vp), ("user_slots", u32), ("item_slots", u32), ("replica_step_scale", f32), ("all_binary16", u32)]
+                ("user_slot_row", vp), ("item_slot_row", vp), ("user_replicas", vp), ("item_replicas", vp), ("user_slots", u32), ("item_slots", u32), ("replica_step_scale", f32), ("all_binary16", u32), ("resident_workers", u32)]
 
 
 class MfReport(C.Structure):

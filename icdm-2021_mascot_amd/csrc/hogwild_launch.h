@@ -27,6 +27,7 @@ struct Call {
     const uint32_t* slot_row_u = nullptr;
     const uint32_t* slot_row_v = nullptr;
     float step_scale = 0.f;         // mf_hogwild_options::replica_step_scale
+    uint32_t resident_workers = 0;  // mf_hogwild_options::resident_workers
     bool replicated() const { return s.slots_u != 0 || s.slots_v != 0; }
 };
 
@@ -71,6 +72,7 @@ static Call make_call(const mf_node* R, uint32_t nnz, uint32_t num_workers, uint
         c.rep_u = static_cast<uint8_t*>(o->user_replicas); c.rep_v = static_cast<uint8_t*>(o->item_replicas);
         c.slot_row_u = o->user_slot_row; c.slot_row_v = o->item_slot_row;
         c.step_scale = o->replica_step_scale;
+        c.resident_workers = o->resident_workers;
     }
     return c;
 }
@@ -89,6 +91,34 @@ static void set_lds_stats(...) {}
 
 template <class Rule, bool HOT>
 static int launch_hot(const char* who, const Call& c, const typename Rule::Params& prm0, size_t lds, void* stream, Range r);
+// Workgroups of `kernel` (kBlock threads, `lds` bytes of LDS of their own) that share a compute unit, and the LDS size
+// to launch with so that at most `resident_workers` workers are resident on the device: the compute unit's LDS divided
+// by the workgroups wanted, which leaves no room for one more.  0 = leave the launch as it is (no cap asked for, the
+// cap is not below what the launch or the device keeps resident anyway, or a query failed).
+static size_t lds_for_resident_cap(const void* kernel, size_t lds, uint32_t resident_workers, uint32_t num_workers)
+{
+    if (resident_workers == 0 || num_workers <= resident_workers) return 0;
+    int blocks = 0, dev = 0, cus = 0, lds_cu = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&blocks, kernel, kBlock, lds) != hipSuccess || hipGetDevice(&dev) != hipSuccess
+        || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess
+        || hipDeviceGetAttribute(&lds_cu, hipDeviceAttributeMaxSharedMemoryPerMultiprocessor, dev) != hipSuccess || blocks <= 0 || cus <= 0 || lds_cu <= 0) {
+        (void)hipGetLastError();
+        return 0;
+    }
+    uint32_t want = resident_workers / (uint32_t)(kWavesPerBlock * cus);
+    if (want < 1) want = 1;
+    // one workgroup per compute unit is the least a launch can be held to
+    if (want >= (uint32_t)blocks || num_workers <= want * (uint32_t)(kWavesPerBlock * cus)) return 0;
+    const size_t padded = ((size_t)lds_cu / want) & ~(size_t)1023;
+    if (padded <= lds || (size_t)(want + 1) * padded <= (size_t)lds_cu) return 0;
+    int got = 0;
+    if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)padded) != hipSuccess
+        || hipOccupancyMaxActiveBlocksPerMultiprocessor(&got, kernel, kBlock, padded) != hipSuccess || got != (int)want) {
+        (void)hipGetLastError();
+        return 0;
+    }
+    return padded;
+}
 // the kernel comes in two builds: with and without the hot-row code (Schedule::keep_u)
 template <class Rule>
 static int launch(const char* who, const Call& c, const typename Rule::Params& prm0, size_t lds, void* stream, Range r)
@@ -151,6 +181,7 @@ static int launch_hot(const char* who, const Call& c, const typename Rule::Param
     if (splits > windows) splits = windows ? windows : 1;
     bool first = true;
     scaled_steps(grid_for(s.num_workers));
+    if (const size_t padded = lds_for_resident_cap(reinterpret_cast<const void*>(&hogwild_kernel<Rule, HOT>), lds, c.resident_workers, s.num_workers)) lds = padded;
     for (uint32_t i = 0; i < splits; ++i) {
         const uint32_t b = i == 0 ? r.begin : (first_window + (uint32_t)((uint64_t)windows * i / splits)) * s0.update_vector_size;
         const uint32_t e = i + 1 == splits ? r.end : (first_window + (uint32_t)((uint64_t)windows * (i + 1) / splits)) * s0.update_vector_size;
@@ -180,11 +211,13 @@ static int launch_k_coh(const char* who, int k, const Call& c, MakeParams make, 
 // Updates in flight during a launch of num_workers workers of Rule at this k (the build with the hot-row code and
 // coherent stores, which is what a run with hot-row tables launches): resident wavefronts x ratings per wavefront.
 template <template <int, bool> class Rule>
-static float inflight_updates(int k, uint32_t num_workers, size_t lds)
+static float inflight_updates(int k, uint32_t num_workers, size_t lds, uint32_t resident_cap)
 {
     int blocks = 0, dev = 0, cus = 0;
-    hipError_t e = k == 128 ? hipOccupancyMaxActiveBlocksPerMultiprocessor(&blocks, reinterpret_cast<const void*>(&hogwild_kernel<Rule<128, true>, true>), kBlock, lds)
-                            : hipOccupancyMaxActiveBlocksPerMultiprocessor(&blocks, reinterpret_cast<const void*>(&hogwild_kernel<Rule<64, true>, true>), kBlock, lds);
+    const void* kernel = k == 128 ? reinterpret_cast<const void*>(&hogwild_kernel<Rule<128, true>, true>) : reinterpret_cast<const void*>(&hogwild_kernel<Rule<64, true>, true>);
+    // a launch held to resident_cap workers runs with the LDS size that does the holding
+    if (const size_t padded = lds_for_resident_cap(kernel, lds, resident_cap, num_workers)) lds = padded;
+    hipError_t e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&blocks, kernel, kBlock, lds);
     if (e != hipSuccess || hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || blocks <= 0 || cus <= 0) {
         (void)hipGetLastError();
         return 0.f;
@@ -193,12 +226,13 @@ static float inflight_updates(int k, uint32_t num_workers, size_t lds)
     const double ahead = k == 128 ? Rule<128, true>::kAhead + 1 : Rule<64, true>::kAhead + 1;
     return (float)(((double)num_workers < resident ? (double)num_workers : resident) * ahead);
 }
-float inflight_sgd(int k, uint32_t num_workers);          // hogwild_launch.hip
-float inflight_mpt(int k, uint32_t num_workers);
-float inflight_mem_quant(int k, uint32_t num_workers);    // launch_mem_quant.hip
-float inflight_muppet(int k, uint32_t num_workers);       // launch_muppet.hip
-float inflight_afp(int k, uint32_t num_workers);          // launch_afp.hip
-float inflight_mascot(int k, uint32_t num_workers, uint32_t user_groups, uint32_t item_groups);   // launch_mascot_plain.hip
+// cap: mf_hogwild_options::resident_workers of the launch (0 = none)
+float inflight_sgd(int k, uint32_t num_workers, uint32_t cap);          // hogwild_launch.hip
+float inflight_mpt(int k, uint32_t num_workers, uint32_t cap);
+float inflight_mem_quant(int k, uint32_t num_workers, uint32_t cap);    // launch_mem_quant.hip
+float inflight_muppet(int k, uint32_t num_workers, uint32_t cap);       // launch_muppet.hip
+float inflight_afp(int k, uint32_t num_workers, uint32_t cap);          // launch_afp.hip
+float inflight_mascot(int k, uint32_t num_workers, uint32_t user_groups, uint32_t item_groups, uint32_t cap);   // launch_mascot_binary16.hip
 
 static Range whole_epoch(const Call& c) { Range r; r.begin = 0; r.end = c.s.range_end; return r; }
 

@@ -88,8 +88,8 @@ int replica_sync(const ReplicaSide& user, const ReplicaSide& item, int k, bool m
     return launch_status("replica_sync");
 }
 
-float inflight_sgd(int k, uint32_t num_workers) { return inflight_updates<SgdRule>(k, num_workers, 0); }
-float inflight_mpt(int k, uint32_t num_workers) { return inflight_updates<MptRule>(k, num_workers, 0); }
+float inflight_sgd(int k, uint32_t num_workers, uint32_t cap) { return inflight_updates<SgdRule>(k, num_workers, 0, cap); }
+float inflight_mpt(int k, uint32_t num_workers, uint32_t cap) { return inflight_updates<MptRule>(k, num_workers, 0, cap); }
 
 }  // namespace mf
 
@@ -110,19 +110,24 @@ int mf_replica_sync_dense(void* matrix, uint32_t elem_bytes, int k, void* replic
     side.rows.dense = matrix; side.rows.elem_bytes = elem_bytes; side.replicas = static_cast<uint8_t*>(replicas); side.slot_row = slot_row; side.slots = slots;
     return replica_sync(side, none, k, merge != 0, stream);
 }
-float mf_hogwild_inflight(uint32_t version, int k, uint32_t num_workers, uint32_t user_groups, uint32_t item_groups)
+float mf_hogwild_inflight_capped(uint32_t version, int k, uint32_t num_workers, uint32_t user_groups, uint32_t item_groups, uint32_t resident_workers)
 {
     if (k != 64 && k != 128) return 0.f;
+    const uint32_t cap = resident_workers;
     switch (version) {
-    case 0: case 5: return inflight_sgd(k, num_workers);
-    case 4: return inflight_mpt(k, num_workers);
-    case 3: return inflight_muppet(k, num_workers);
-    case 2: return inflight_afp(k, num_workers);
-    case 7: return inflight_mem_quant(k, num_workers);
-    case 8: return inflight_mascot(k, num_workers, 1, 1);
-    case 1: case 6: return inflight_mascot(k, num_workers, user_groups ? user_groups : 1, item_groups ? item_groups : 1);
+    case 0: case 5: return inflight_sgd(k, num_workers, cap);
+    case 4: return inflight_mpt(k, num_workers, cap);
+    case 3: return inflight_muppet(k, num_workers, cap);
+    case 2: return inflight_afp(k, num_workers, cap);
+    case 7: return inflight_mem_quant(k, num_workers, cap);
+    case 8: return inflight_mascot(k, num_workers, 1, 1, cap);
+    case 1: case 6: return inflight_mascot(k, num_workers, user_groups ? user_groups : 1, item_groups ? item_groups : 1, cap);
     default: return 0.f;
     }
+}
+float mf_hogwild_inflight(uint32_t version, int k, uint32_t num_workers, uint32_t user_groups, uint32_t item_groups)
+{
+    return mf_hogwild_inflight_capped(version, k, num_workers, user_groups, item_groups, 0);
 }
 uint32_t mf_mascot_norm_blocks(uint32_t num_workers) { return grid_for(num_workers); }
 

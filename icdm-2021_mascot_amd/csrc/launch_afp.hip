@@ -2,7 +2,7 @@
 #include "hogwild_launch.h"
 #include "rules_fixed_point.h"
 
-namespace mf { float inflight_afp(int k, uint32_t num_workers) { return inflight_updates<AfpRule>(k, num_workers, 0); } }
+namespace mf { float inflight_afp(int k, uint32_t num_workers, uint32_t cap) { return inflight_updates<AfpRule>(k, num_workers, 0, cap); } }
 using namespace mf;
 
 extern "C" {

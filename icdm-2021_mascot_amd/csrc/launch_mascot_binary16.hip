@@ -13,9 +13,9 @@ int launch_mascot_binary16(const MascotCall& c, Range r)
 // A run starts with every group in binary16, and its hot-row tables are built once: the wavefronts this build keeps
 // resident are the ones to count (the build with the mixed-precision path keeps one fewer per SIMD; tables made for
 // more updates in flight than there are err on the careful side).
-float inflight_mascot(int k, uint32_t num_workers, uint32_t user_groups, uint32_t item_groups)
+float inflight_mascot(int k, uint32_t num_workers, uint32_t user_groups, uint32_t item_groups, uint32_t cap)
 {
-    return inflight_updates<MascotBinary16Rule>(k, num_workers, MascotRule<128, true>::lds_bytes(user_groups, item_groups));
+    return inflight_updates<MascotBinary16Rule>(k, num_workers, MascotRule<128, true>::lds_bytes(user_groups, item_groups), cap);
 }
 
 }  // namespace mf

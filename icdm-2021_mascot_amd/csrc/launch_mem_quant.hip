@@ -2,7 +2,7 @@
 #include "hogwild_launch.h"
 #include "rules_fp32.h"
 
-namespace mf { float inflight_mem_quant(int k, uint32_t num_workers) { return inflight_updates<MemQuantRule>(k, num_workers, 0); } }
+namespace mf { float inflight_mem_quant(int k, uint32_t num_workers, uint32_t cap) { return inflight_updates<MemQuantRule>(k, num_workers, 0, cap); } }
 using namespace mf;
 
 extern "C" {

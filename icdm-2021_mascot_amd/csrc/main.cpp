@@ -7,7 +7,8 @@
 // and `-split <n>` (row access policy and kernel launches per epoch, see include/mascot_hip.h), `-hot <0|1>`,
 // `-replicate <t>[,<merges>]` and `-thin <cap>[,<early cap>,<epochs>]` (how rows with several updates in flight are
 // treated: mf_params.hot_rows, replicate_inflight, hot_row_inflight; `-hot 0` is the reference's race semantics),
-// `-synth <c>[,<n>]`
+// `-early <fraction>[,<epochs>]` (the first epochs run with that fraction of the updates in flight:
+// mf_params.early_inflight), `-synth <c>[,<n>]`
 // (no input files: the seeded synthetic stand-in of BASELINE configuration c, optionally with n training ratings
 // and the test set scaled alike, generated on the device; mf_generate_ratings).
 #include <sys/stat.h>
@@ -66,6 +67,12 @@ int main(int argc, const char* argv[])
                 const int got = std::sscanf(argv[i + 1], "%f,%u", &above, &merges);
                 if (got >= 1) prm.replicate_inflight = above;
                 if (got >= 2) prm.replica_merges = merges;
+            }
+            if (a == "-early" && has) {          // <fraction of the updates in flight during the first epochs; 0 or 1 = off>[,<epochs>]
+                float fraction = 0; unsigned ep = 0;
+                const int got = std::sscanf(argv[i + 1], "%f,%u", &fraction, &ep);
+                if (got >= 1) prm.early_inflight = fraction;
+                if (got >= 2) prm.early_inflight_epochs = ep;
             }
             if (a == "-thin" && has) {           // opt-in thinning of hot rows: <steady cap>[,<early cap>,<early epochs>]
                 float steady = 0, early = 0; unsigned ep = 0;

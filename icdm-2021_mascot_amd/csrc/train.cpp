@@ -183,9 +183,12 @@ KeepTable keep_table(const uint32_t* cnt, uint32_t rows, uint32_t n, double infl
 // -- two pairs when rows are thinned, an early cap for the first epochs, while every row still grows from its small
 // initial value and the popular rows need many updates, and the steady cap afterwards -- and the replica arrays.
 struct HotRows {
-    struct SideTables { DevBuf early, steady, slot, slot_row, replicas; uint32_t slots = 0; };
+    // low_*: the tables of the first epochs when those run with fewer updates in flight (mf_params::early_inflight): fewer
+    // rows are hot then, and the replicated ones are numbered on their own (the copies share the steady tables' array)
+    struct SideTables { DevBuf early, steady, slot, slot_row, replicas, low_keep, low_slot, low_slot_row; uint32_t slots = 0, low_slots = 0; };
     SideTables u, v;
-    mf_hogwild_options opt_early{}, opt_steady{};
+    mf_hogwild_options opt_early{}, opt_steady{}, opt_low{};
+    uint32_t low_epochs = 0;
     mutable mf_hogwild_options opt_current{};
     uint32_t early_epochs = 0;
     float step_scale = 0.f; uint32_t step_epochs = 0;      // scaled steps on replicated rows during the first step_epochs epochs (0: all)
@@ -210,6 +213,18 @@ struct HotRows {
             MF_TRY(upload(t.slot, steady.slot.data(), (size_t)rows * 2, "replica slots"));
             MF_TRY(upload(t.slot_row, steady.slot_row.data(), (size_t)t.slots * 4, "replica rows"));
             MF_TRY(t.replicas.alloc((size_t)MF_XCDS * t.slots * prm.k * 4, "hipMalloc(row replicas)"));
+        }
+        return 0;
+    }
+    int build_low(SideTables& t, const mf_params& prm, const uint32_t* cnt, uint32_t rows, uint32_t n, double low_inflight)
+    {
+        const KeepTable low = keep_table(cnt, rows, n, low_inflight, replicate_above, prm.hot_row_inflight_early > 0 ? prm.hot_row_inflight_early : prm.hot_row_inflight, prm.replica_add_inflight);
+        t.low_slots = (uint32_t)low.slot_row.size();
+        if (t.low_slots > t.slots) return invalid("mf_train: more rows are replicated with fewer updates in flight (%u > %u)", t.low_slots, t.slots);
+        MF_TRY(upload(t.low_keep, low.keep.data(), rows, "hot-row table"));
+        if (t.low_slots) {
+            MF_TRY(upload(t.low_slot, low.slot.data(), (size_t)rows * 2, "replica slots"));
+            MF_TRY(upload(t.low_slot_row, low.slot_row.data(), (size_t)t.low_slots * 4, "replica rows"));
         }
         return 0;
     }
@@ -244,13 +259,34 @@ struct HotRows {
         }
         opt_early = o;
         if (early) { opt_early.user_keep = u.early.as<uint8_t>(); opt_early.item_keep = v.early.as<uint8_t>(); }
+        // The first epochs with fewer updates in flight: resident workers capped, tables for that many updates in flight.
+        // resident = inflight / ratings a worker keeps in flight, which mf_hogwild_inflight folds in: ask it for one worker.
+        low_epochs = 0;
+        if (prm.early_inflight > 0.f && prm.early_inflight < 1.f && prm.early_inflight_epochs > 0) {
+            const double per_worker = mf_hogwild_inflight(prm.version, (int)prm.k, 1, user_groups, item_groups);
+            const uint32_t resident = per_worker > 0 ? (uint32_t)(inflight / per_worker + 0.5) : 0;
+            const uint32_t capped = (uint32_t)(resident * (double)prm.early_inflight);
+            // what a launch held to that many workers really keeps in flight (whole workgroups per compute unit)
+            const double low_inflight = capped >= 1 ? mf_hogwild_inflight_capped(prm.version, (int)prm.k, prm.num_workers, user_groups, item_groups, capped) : 0.0;
+            if (low_inflight > 0 && low_inflight < inflight) {
+                MF_TRY(build_low(u, prm, ucnt, n_users, n, low_inflight));
+                MF_TRY(build_low(v, prm, icnt, n_items, n, low_inflight));
+                opt_low = o;
+                opt_low.resident_workers = capped;
+                opt_low.user_keep = u.low_keep.as<uint8_t>(); opt_low.item_keep = v.low_keep.as<uint8_t>();
+                opt_low.user_slot = u.low_slot.as<uint16_t>(); opt_low.item_slot = v.low_slot.as<uint16_t>();
+                opt_low.user_slot_row = u.low_slot_row.as<uint32_t>(); opt_low.item_slot_row = v.low_slot_row.as<uint32_t>();
+                opt_low.user_slots = u.low_slots; opt_low.item_slots = v.low_slots;
+                low_epochs = prm.early_inflight_epochs;
+            }
+        }
         return 0;
     }
     // options of the launches of epoch e (valid until the next call)
     bool all_binary16 = false;      // MASCOT runs: no group has been promoted yet
     const mf_hogwild_options* options(uint32_t e) const
     {
-        opt_current = e < early_epochs ? opt_early : opt_steady;
+        opt_current = e < low_epochs ? opt_low : (e < early_epochs ? opt_early : opt_steady);
         opt_current.replica_step_scale = (step_epochs == 0 || e < step_epochs) ? step_scale : 0.f;
         opt_current.all_binary16 = all_binary16 ? 1u : 0u;
         return &opt_current;
@@ -812,6 +848,7 @@ void mf_default_params(mf_params* out)       // main.cu:19-32
     out->hot_rows = 1; out->replicate_inflight = -1.0f; out->replica_merges = 0;
     out->hot_row_inflight = 0.0f; out->hot_row_inflight_early = 0.0f; out->hot_row_early_epochs = 0;
     out->replica_step_scale = -1.0f; out->replica_step_epochs = 1;
+    out->early_inflight = 0.5f; out->early_inflight_epochs = 1;
 }
 
 uint32_t mf_group_end_indices(const uint32_t* sorted_cnt, uint32_t n, uint32_t requested_groups, uint32_t* end_idx_out)

@@ -89,7 +89,13 @@ const char* mf_last_error(void);
  * all_binary16  MASCOT only, a hint: 1 = every group of both sides is binary16 in this call.  The call then launches a
  *               build of the kernel without the fast path for chunks of mixed precisions, which keeps one more
  *               wavefront per SIMD resident (4 % per epoch at 100M ratings).  A wrong hint costs time, not results:
- *               that build takes its general path for any chunk that touches a binary32 group. */
+ *               that build takes its general path for any chunk that touches a binary32 group.
+ * resident_workers   0 (default): as many workers run at a time as the device keeps resident.  > 0: at most about that
+ *               many (rounded down to whole workgroups per compute unit, at least one): the ordinary launches of the call
+ *               ask for LDS they do not use, which keeps further workgroups off a compute unit.  Fewer updates in flight
+ *               bring a run closer to a sequential one and cost time; mf_train uses it for the first epoch
+ *               (mf_params.early_inflight).  The hot-row tables of such a call are the caller's to build for the lower
+ *               number of updates in flight.  The sampled launch of a MASCOT check epoch is not affected. */
 #define MF_KEEP_ORDINARY 255
 #define MF_KEEP_ADDED 254
 #define MF_KEEP_REPLICATED 253
@@ -109,6 +115,7 @@ typedef struct {
     uint32_t user_slots, item_slots;
     float replica_step_scale;
     uint32_t all_binary16;
+    uint32_t resident_workers;
 } mf_hogwild_options;
 /* What the update calls do with replicated rows before and after every kernel launch, for a dense matrix [rows][k] of
  * elem_bytes-wide elements (2: binary16, 4: binary32): merge = 0 copies row slot_row[s] into slot s of every XCD's
@@ -130,6 +137,9 @@ int mf_hot_row_table(const uint32_t* counts, uint32_t rows, uint32_t n, float in
  * min(num_workers, wavefronts the device keeps resident for that kernel) x the ratings a wavefront keeps in flight
  * (4; 2 for MuPPET and AFP).  Asks the HIP runtime for the kernel's occupancy on the current device. */
 float mf_hogwild_inflight(uint32_t version, int k, uint32_t num_workers, uint32_t user_groups, uint32_t item_groups);
+/* The same for launches with mf_hogwild_options::resident_workers set (0 = not set): what such a launch really keeps
+ * in flight -- the cap works in whole workgroups per compute unit and does nothing to a launch that is below it anyway. */
+float mf_hogwild_inflight_capped(uint32_t version, int k, uint32_t num_workers, uint32_t user_groups, uint32_t item_groups, uint32_t resident_workers);
 /* Seeded synthetic ratings (no counterpart in the reference, whose data sets are downloaded): users and items are
  * drawn independently from Zipf(alpha) over a random permutation of the ids; a rating is
  * clamp(round_to_step(U_u . V_i + mean + noise * N(0,1)), lo, hi) with rank-`rank` factors U, V ~ N(0, 0.5^2), or,
@@ -418,6 +428,16 @@ typedef struct {
                                  epoch in which every row grows from its small initial value and a replicated row, which
                                  keeps one of the many updates in flight on a copy, is furthest behind; afterwards the
                                  unscaled mean of eight copies is the less noisy estimate.  0 = every epoch) */
+    float early_inflight;     /* runs with hot-row tables: the first early_inflight_epochs epochs run with this fraction of the
+                                 updates in flight the device would keep (mf_hogwild_options::resident_workers, and tables
+                                 built for that number).  A row keeps one of the updates that are in flight on it at a
+                                 time, so while the rows are far from their optimum the distance to a sequential run
+                                 grows with the updates in flight: at 100M ratings the test RMSE after the first epoch is
+                                 0.049 / 0.024 / 0.023 / 0.015 above the sequential run's with all / half / a third / a
+                                 quarter of them, and that epoch takes 15.7 / 19.8 / 20.9 / 33.4 ms.  Between 0 and 1;
+                                 0 or 1 = off.  Default 0.5.  The cap works in workgroups per compute unit, so a run with
+                                 fewer than 1024 workers is not affected */
+    uint32_t early_inflight_epochs; /* default 1 */
 } mf_params;
 
 /* What a run reports back; every pointer is optional host memory owned by the caller. */

@@ -209,9 +209,10 @@ def test_afp_special_values(orc, k):
     assert _same_values(gq, Q)
 
 
-def _mascot_case(orc, k, W, uc, window, user_groups, item_groups, prec_mode, first_sample, seed, lr=LR, row_classes=None, all_binary16=0, step_scale=0.0):
+def _mascot_case(orc, k, W, uc, window, user_groups, item_groups, prec_mode, first_sample, seed, lr=LR, row_classes=None, all_binary16=0, step_scale=0.0, resident_workers=0):
     """row_classes: keep-table values drawn at random per row (mf_hogwild_options); with them the call goes through the
-    _opt entry point, with the all_binary16 hint and the step factor of replicated rows' copies as given."""
+    _opt entry point, with the all_binary16 hint, the step factor of replicated rows' copies and the cap on resident
+    workers as given."""
     import torch
     h = mfutil.hip()
     R, starts, P, Q = mfutil.conflict_free_problem(seed, k, W, uc, window)
@@ -236,13 +237,14 @@ def _mascot_case(orc, k, W, uc, window, user_groups, item_groups, prec_mode, fir
             dp.end.data_ptr(), dq.end.data_ptr(), dp.prec.data_ptr(), dq.prec.data_ptr(),
             d_gsp.data_ptr(), d_gsq.data_ptr(), d_nsp.data_ptr(), d_nsq.data_ptr(),
             first_sample, user_groups, item_groups, 0, 0, dS.data_ptr(), mfutil.stream_ptr())
-    if row_classes is None and not all_binary16:
+    if row_classes is None and not all_binary16 and not resident_workers:
         h.mf_mascot_sgd_hogwild(*args)
     else:
         values = np.array(row_classes if row_classes is not None else [255], np.uint8)
         keep = [values[rng.integers(0, values.size, n)] for n in (n_users, n_items)] if row_classes is not None else [None, None]
         opt = mfutil.HogwildOptions(k, keep[0], keep[1], launches=2, step_scale=step_scale)
         opt.o.all_binary16 = all_binary16
+        opt.o.resident_workers = resident_workers
         h.mf_mascot_sgd_hogwild_opt(*args, opt.ptr)
     torch.cuda.synchronize()
     gsp, gsq = np.zeros(user_groups * k, np.float32), np.zeros(item_groups * k, np.float32)
@@ -288,6 +290,39 @@ def test_mascot_row_classes_and_hints_keep_the_checkers_result(orc, k, prec_mode
         _mascot_case(orc, k, W, uc, window, 7, 5, prec_mode, first_sample=2 * window - 40, seed=150 + k, row_classes=(255, 253), all_binary16=hint)
         _mascot_case(orc, k, W, uc, window, 7, 5, prec_mode, first_sample=uc * window, seed=151 + k, all_binary16=hint)
     _mascot_case(orc, k, 4, uc, window, 7, 5, prec_mode, first_sample=2 * window - 40, seed=152 + k, row_classes=(255, 253), step_scale=4.0)
+
+
+@pytest.mark.parametrize("k", [64, 128])
+def test_resident_worker_cap_changes_when_not_what(orc, k):
+    """mf_hogwild_options.resident_workers holds a launch to fewer resident workers by asking for LDS it does not use.
+    1100 workers that own their rows, held to one workgroup per compute unit: the results are the checker's bit for bit
+    (fp32 SGD without tables; MASCOT with row classes, its own LDS tables inside the padded allocation).  And the number
+    of updates in flight the library reports for such a launch: whole workgroups per compute unit, never more than the
+    uncapped launch, unchanged for a launch that is below the cap anyway."""
+    import torch
+    h = mfutil.hip()
+    W, uc, window = 1100, 1, 64
+    R, starts, P, Q = mfutil.conflict_free_problem(170 + k, k, W, uc, window)
+    dR, dS, dP, dQ = to_dev(R), to_dev(starts), to_dev(P), to_dev(Q)
+    opt = mfutil.HogwildOptions(k)
+    opt.o.resident_workers = 1
+    h.mf_single_sgd_hogwild_opt(dR.data_ptr(), R.size, dP.data_ptr(), dQ.data_ptr(), k, W, uc, window, LR, LAM, 1234, 0, dS.data_ptr(), mfutil.stream_ptr(), opt.ptr)
+    torch.cuda.synchronize()
+    orc.lib.orc_sgd_epoch(k, R.ctypes.data, R.size, P.ctypes.data, Q.ctypes.data, W, uc, window, LR, LAM, 0, 0, starts.ctypes.data, 1)
+    assert np.array_equal(from_dev(dP, np.float32, P.shape).view(np.uint32), P.view(np.uint32))
+    assert np.array_equal(from_dev(dQ, np.float32, Q.shape).view(np.uint32), Q.view(np.uint32))
+    _mascot_case(orc, k, W, uc, window, 7, 5, "mixed", first_sample=uc * window, seed=171 + k, row_classes=(255, 253), resident_workers=1)
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    for version, per_worker in ((5, 4), (1, 4), (3, 2)):
+        full = h.lib.mf_hogwild_inflight(version, k, 1000000, 7, 5)
+        assert full > 0 and full % (4 * cus * per_worker) == 0
+        resident = int(full) // per_worker
+        assert h.lib.mf_hogwild_inflight_capped(version, k, 1000000, 7, 5, 0) == full
+        assert h.lib.mf_hogwild_inflight_capped(version, k, 1000000, 7, 5, resident) == full
+        assert h.lib.mf_hogwild_inflight_capped(version, k, 1000000, 7, 5, 1) == 4 * cus * per_worker          # one workgroup per compute unit
+        half = h.lib.mf_hogwild_inflight_capped(version, k, 1000000, 7, 5, resident // 2)
+        assert half == (resident // 2) // (4 * cus) * (4 * cus) * per_worker
+        assert h.lib.mf_hogwild_inflight_capped(version, k, 500, 7, 5, 100) == 500 * per_worker                 # 125 workgroups: below any cap
 
 
 @pytest.mark.parametrize("k", [64, 128])
