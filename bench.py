@@ -34,10 +34,11 @@ KERNEL_SOURCES = os.path.join(ROOT, "icdm-2021_mascot_amd", "csrc")
 
 
 def kernel_sources_digest():
-    """sha256 over the device sources of the library (file names and contents, in name order)."""
+    """sha256 over the sources of the library (file names and contents, in name order): the kernels, and the host code
+    whose defaults decide how rows are treated."""
     h = hashlib.sha256()
     for name in sorted(os.listdir(KERNEL_SOURCES)):
-        if name.endswith((".h", ".hip")):
+        if name.endswith((".h", ".hip", ".cpp")):
             h.update(name.encode())
             with open(os.path.join(KERNEL_SOURCES, name), "rb") as f:
                 h.update(f.read())
@@ -205,7 +206,10 @@ def main():
     ap.add_argument("--seed", type=int, default=2021)
     ap.add_argument("--replicate", type=float, default=-1.0, help="mf_params.replicate_inflight (default: derived from learning rate and mean rating)")
     ap.add_argument("--merges", type=int, default=0, help="mf_params.replica_merges (default: the library's)")
-    ap.add_argument("--step-epochs", type=int, default=-1, help="mf_params.replica_step_epochs (default: the library's 5; 0 = every epoch)")
+    ap.add_argument("--step-epochs", type=int, default=-1, help="mf_params.replica_step_epochs (default: the library's 1; 0 = every epoch)")
+    ap.add_argument("--replicate-late", type=float, default=-1.0, help="mf_params.replicate_inflight_late (default: a third of --replicate's value; 0 = the same bar throughout)")
+    ap.add_argument("--late-from", type=int, default=-1, help="mf_params.replicate_late_from (default: the library's 1, the second epoch)")
+    ap.add_argument("--early", type=float, default=-1.0, help="mf_params.early_inflight: fraction of the updates in flight during the first epoch (default: the library's 0.5; 1 = off)")
     ap.add_argument("--step-scale", type=float, default=-1.0, help="mf_params.replica_step_scale (default: the library's; 0 = unscaled steps on replicated rows)")
     ap.add_argument("--thin", type=float, default=0.0, help="mf_params.hot_row_inflight: opt-in thinning of hot rows (0 = every update carried out)")
     ap.add_argument("--cpu-updates", type=int, default=32_000_000, help="size of the CPU baseline sample (about 10 s on 16 threads)")
@@ -246,6 +250,12 @@ def main():
         extra["replica_step_scale"] = a.step_scale
     if a.step_epochs >= 0:
         extra["replica_step_epochs"] = a.step_epochs
+    if a.replicate_late >= 0:
+        extra["replicate_inflight_late"] = a.replicate_late
+    if a.late_from >= 0:
+        extra["replicate_late_from"] = a.late_from
+    if a.early >= 0:
+        extra["early_inflight"] = a.early
     if a.pmc_copy:
         src = torch.empty(1 << 28, dtype=torch.float32, device="cuda").normal_()
         dst = torch.empty_like(src)
@@ -260,6 +270,7 @@ def main():
     setup_s = time.perf_counter() - t0
     W = sess.workers
     rep_u, rep_v, inflight = sess.hot_rows()
+    replicate_bar = float(h.mf_replicate_threshold(TRAIN["lr"], float(np.abs(train["r"][:4_000_000]).mean()))) if a.replicate < 0 else a.replicate
     uc = h.mf_update_count(n_train, W, 128)
     updates = W * uc * 128
     timed = np.array(main_run["timed"], np.float64)
@@ -287,7 +298,9 @@ def main():
                    "update_vector_size": 128, "epochs_timed": "%d..%d of 50" % (a.warmup, a.warmup + a.steps - 1), "seed": a.seed,
                    "row_updates_carried_out": 1.0 if a.thin == 0 else None,
                    "updates_in_flight": inflight, "replicated_rows": {"user": rep_u, "item": rep_v},
-                   "replicate_above_in_flight": float(h.mf_replicate_threshold(TRAIN["lr"], float(np.abs(train["r"][:4_000_000]).mean()))) if a.replicate < 0 else a.replicate,
+                   "replicate_above_in_flight": {"epochs_before": prm.replicate_late_from, "bar": replicate_bar,
+                                                 "later_bar": (replicate_bar / 3.0 if prm.replicate_inflight_late < 0 else (prm.replicate_inflight_late or replicate_bar))},
+                   "first_epochs": {"epochs": prm.early_inflight_epochs, "updates_in_flight_fraction": prm.early_inflight, "replica_step_scale": "library default" if a.step_scale < 0 else a.step_scale},
                    "setup_s": round(setup_s, 1)},
         "roofline": {"bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS,
                      "note": "algorithmic bytes: every update reads and writes both rows (12 + 2k(s_user + s_item) bytes, s = 2 for a binary16 "

@@ -98,7 +98,7 @@ class MfParams(C.Structure):
                 ("epoch", u32), ("thread_block_size", u32), ("version", u32), ("is_yahoo", u32), ("seed", u64),
                 ("verbose", u32), ("cached_rows", u32), ("epoch_splits", u32), ("hot_row_inflight", f32), ("hot_row_inflight_early", f32), ("hot_row_early_epochs", u32),
                 ("hot_rows", u32), ("replicate_inflight", f32), ("replica_merges", u32), ("replica_add_inflight", f32), ("replica_step_scale", f32), ("wg_counts_updates", u32), ("replica_step_epochs", u32),
-                ("early_inflight", f32), ("early_inflight_epochs", u32)]
+                ("early_inflight", f32), ("early_inflight_epochs", u32), ("replicate_inflight_late", f32), ("replicate_late_from", u32)]
 
 
 class HogwildOptions(C.Structure):

@@ -5,7 +5,7 @@
 // counts updates in flight as it does in the reference, where a worker has one; a worker here keeps four, so the run
 // uses a quarter as many workers: mf_params.wg_counts_updates), `-cached <0|1>`
 // and `-split <n>` (row access policy and kernel launches per epoch, see include/mascot_hip.h), `-hot <0|1>`,
-// `-replicate <t>[,<merges>]` and `-thin <cap>[,<early cap>,<epochs>]` (how rows with several updates in flight are
+// `-replicate <t>[,<merges>[,<late t>[,<from epoch>]]]` and `-thin <cap>[,<early cap>,<epochs>]` (how rows with several updates in flight are
 // treated: mf_params.hot_rows, replicate_inflight, hot_row_inflight; `-hot 0` is the reference's race semantics),
 // `-early <fraction>[,<epochs>]` (the first epochs run with that fraction of the updates in flight:
 // mf_params.early_inflight), `-synth <c>[,<n>]`
@@ -62,11 +62,13 @@ int main(int argc, const char* argv[])
                 prm.hot_rows = std::atoi(argv[i + 1]) != 0;
                 if (!prm.hot_rows) { prm.replicate_inflight = 0; prm.hot_row_inflight = 0; }
             }
-            if (a == "-replicate" && has) {      // <updates in flight above which a row gets a copy per XCD; 0 = none>[,<merges per epoch>]
-                float above = 0; unsigned merges = 0;
-                const int got = std::sscanf(argv[i + 1], "%f,%u", &above, &merges);
+            if (a == "-replicate" && has) {      // <updates in flight above which a row gets a copy per XCD; 0 = none>[,<merges per epoch>[,<the bar in later epochs; 0 = the same>[,<from epoch>]]]
+                float above = 0, late = 0; unsigned merges = 0, from = 0;
+                const int got = std::sscanf(argv[i + 1], "%f,%u,%f,%u", &above, &merges, &late, &from);
                 if (got >= 1) prm.replicate_inflight = above;
                 if (got >= 2) prm.replica_merges = merges;
+                if (got >= 3) prm.replicate_inflight_late = late;
+                if (got >= 4) prm.replicate_late_from = from;
             }
             if (a == "-early" && has) {          // <fraction of the updates in flight during the first epochs; 0 or 1 = off>[,<epochs>]
                 float fraction = 0; unsigned ep = 0;
@@ -119,6 +121,8 @@ int main(int argc, const char* argv[])
         if (prm.replicate_inflight < 0) std::cout << "; rows above 0.3 / (learning rate x mean rating) in flight are replicated per XCD";
         else if (prm.replicate_inflight > 0) std::cout << "; rows above " << prm.replicate_inflight << " in flight are replicated per XCD";
         if (prm.replicate_inflight != 0 && prm.replica_merges) std::cout << ", merged " << prm.replica_merges << " times per epoch";
+        if (prm.replicate_inflight != 0 && prm.replicate_inflight_late < 0) std::cout << " (above a third of that from epoch " << prm.replicate_late_from + 1 << " on)";
+        else if (prm.replicate_inflight != 0 && prm.replicate_inflight_late > 0) std::cout << " (above " << prm.replicate_inflight_late << " from epoch " << prm.replicate_late_from + 1 << " on)";
         if (prm.hot_row_inflight > 0) std::cout << "; rows above " << prm.hot_row_inflight << " in flight are thinned";
     }
     std::cout << std::endl;

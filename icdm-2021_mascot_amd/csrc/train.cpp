@@ -183,16 +183,31 @@ KeepTable keep_table(const uint32_t* cnt, uint32_t rows, uint32_t n, double infl
 // -- two pairs when rows are thinned, an early cap for the first epochs, while every row still grows from its small
 // initial value and the popular rows need many updates, and the steady cap afterwards -- and the replica arrays.
 struct HotRows {
-    // low_*: the tables of the first epochs when those run with fewer updates in flight (mf_params::early_inflight): fewer
-    // rows are hot then, and the replicated ones are numbered on their own (the copies share the steady tables' array)
-    struct SideTables { DevBuf early, steady, slot, slot_row, replicas, low_keep, low_slot, low_slot_row; uint32_t slots = 0, low_slots = 0; };
+    // One set of tables: a keep byte per row, and the numbering of the replicated rows.  A run has up to three sets:
+    // `low` for the first epochs when those run with fewer updates in flight (mf_params::early_inflight: fewer rows are
+    // hot then), `steady` up to epoch late_from, and `late` from there on, with a lower bar for replication
+    // (mf_params::replicate_inflight_late).  The copies of all sets share one array per side, sized for the most slots.
+    struct TableSet {
+        DevBuf keep, slot, slot_row; uint32_t slots = 0;
+        int upload_from(const KeepTable& t, uint32_t rows)
+        {
+            slots = (uint32_t)t.slot_row.size();
+            MF_TRY(upload(keep, t.keep.data(), rows, "hot-row table"));
+            if (slots) {
+                MF_TRY(upload(slot, t.slot.data(), (size_t)rows * 2, "replica slots"));
+                MF_TRY(upload(slot_row, t.slot_row.data(), (size_t)slots * 4, "replica rows"));
+            }
+            return 0;
+        }
+    };
+    struct SideTables { TableSet steady, low, late; DevBuf early, replicas; };
     SideTables u, v;
-    mf_hogwild_options opt_early{}, opt_steady{}, opt_low{};
-    uint32_t low_epochs = 0;
+    mf_hogwild_options opt_early{}, opt_steady{}, opt_low{}, opt_late{};
+    uint32_t low_epochs = 0, late_from = 0xffffffffu;
     mutable mf_hogwild_options opt_current{};
     uint32_t early_epochs = 0;
     float step_scale = 0.f; uint32_t step_epochs = 0;      // scaled steps on replicated rows during the first step_epochs epochs (0: all)
-    double inflight = 0, replicate_above = 0;
+    double inflight = 0, replicate_above = 0, replicate_above_late = 0;
     static bool wanted(const mf_params& prm) { return prm.hot_rows || prm.hot_row_inflight > 0 || prm.replicate_inflight > 0; }
     static int upload(DevBuf& d, const void* src, size_t bytes, const char* what)
     {
@@ -200,33 +215,12 @@ struct HotRows {
         if (bytes) HIP_TRY(hipMemcpy(d.p, src, bytes, hipMemcpyHostToDevice), what);
         return 0;
     }
-    int build_side(SideTables& t, const mf_params& prm, const uint32_t* cnt, uint32_t rows, uint32_t n, bool early)
+    static void point_at(mf_hogwild_options& o, const TableSet& us, const TableSet& vs)
     {
-        const KeepTable steady = keep_table(cnt, rows, n, inflight, replicate_above, prm.hot_row_inflight, prm.replica_add_inflight);
-        MF_TRY(upload(t.steady, steady.keep.data(), rows, "hot-row table"));
-        if (early) {
-            const KeepTable e = keep_table(cnt, rows, n, inflight, replicate_above, prm.hot_row_inflight_early, prm.replica_add_inflight);
-            MF_TRY(upload(t.early, e.keep.data(), rows, "hot-row table"));
-        }
-        t.slots = (uint32_t)steady.slot_row.size();
-        if (t.slots) {
-            MF_TRY(upload(t.slot, steady.slot.data(), (size_t)rows * 2, "replica slots"));
-            MF_TRY(upload(t.slot_row, steady.slot_row.data(), (size_t)t.slots * 4, "replica rows"));
-            MF_TRY(t.replicas.alloc((size_t)MF_XCDS * t.slots * prm.k * 4, "hipMalloc(row replicas)"));
-        }
-        return 0;
-    }
-    int build_low(SideTables& t, const mf_params& prm, const uint32_t* cnt, uint32_t rows, uint32_t n, double low_inflight)
-    {
-        const KeepTable low = keep_table(cnt, rows, n, low_inflight, replicate_above, prm.hot_row_inflight_early > 0 ? prm.hot_row_inflight_early : prm.hot_row_inflight, prm.replica_add_inflight);
-        t.low_slots = (uint32_t)low.slot_row.size();
-        if (t.low_slots > t.slots) return invalid("mf_train: more rows are replicated with fewer updates in flight (%u > %u)", t.low_slots, t.slots);
-        MF_TRY(upload(t.low_keep, low.keep.data(), rows, "hot-row table"));
-        if (t.low_slots) {
-            MF_TRY(upload(t.low_slot, low.slot.data(), (size_t)rows * 2, "replica slots"));
-            MF_TRY(upload(t.low_slot_row, low.slot_row.data(), (size_t)t.low_slots * 4, "replica rows"));
-        }
-        return 0;
+        o.user_keep = us.keep.as<uint8_t>(); o.item_keep = vs.keep.as<uint8_t>();
+        o.user_slot = us.slot.as<uint16_t>(); o.item_slot = vs.slot.as<uint16_t>();
+        o.user_slot_row = us.slot_row.as<uint32_t>(); o.item_slot_row = vs.slot_row.as<uint32_t>();
+        o.user_slots = us.slots; o.item_slots = vs.slots;
     }
     int install(const mf_params& prm, const uint32_t* ucnt, uint32_t n_users, const uint32_t* icnt, uint32_t n_items, uint32_t n,
                 uint32_t user_groups, uint32_t item_groups, float mean_rating)
@@ -235,6 +229,7 @@ struct HotRows {
         opt_steady.cached_rows = prm.cached_rows ? 1u : 0u;
         opt_steady.launches = prm.epoch_splits ? prm.epoch_splits : 1u;
         opt_early = opt_steady;
+        low_epochs = 0; late_from = 0xffffffffu;
         if (!wanted(prm)) return 0;
         step_scale = prm.replica_step_scale < 0 ? mf_replica_step_scale(prm.learning_rate, mean_rating) : prm.replica_step_scale;
         step_epochs = prm.replica_step_epochs;
@@ -243,15 +238,48 @@ struct HotRows {
         replicate_above = prm.replicate_inflight > 0 ? prm.replicate_inflight : (prm.replicate_inflight < 0 ? mf_replicate_threshold(prm.learning_rate, mean_rating) : 0.0);
         const bool early = prm.hot_row_inflight > 0 && prm.hot_row_inflight_early > prm.hot_row_inflight && prm.hot_row_early_epochs > 0;
         early_epochs = early ? prm.hot_row_early_epochs : 0;
-        MF_TRY(build_side(u, prm, ucnt, n_users, n, early));
-        MF_TRY(build_side(v, prm, icnt, n_items, n, early));
+        const uint32_t* cnt[2] = {ucnt, icnt};
+        const uint32_t rows[2] = {n_users, n_items};
+        SideTables* side[2] = {&u, &v};
+        for (int s = 0; s < 2; ++s) {
+            MF_TRY(side[s]->steady.upload_from(keep_table(cnt[s], rows[s], n, inflight, replicate_above, prm.hot_row_inflight, prm.replica_add_inflight), rows[s]));
+            if (early) {
+                const KeepTable e = keep_table(cnt[s], rows[s], n, inflight, replicate_above, prm.hot_row_inflight_early, prm.replica_add_inflight);
+                MF_TRY(upload(side[s]->early, e.keep.data(), rows[s], "hot-row table"));
+            }
+        }
         mf_hogwild_options& o = opt_steady;
-        o.user_keep = u.steady.as<uint8_t>(); o.item_keep = v.steady.as<uint8_t>();
-        o.user_slot = u.slot.as<uint16_t>(); o.item_slot = v.slot.as<uint16_t>();
-        o.user_slot_row = u.slot_row.as<uint32_t>(); o.item_slot_row = v.slot_row.as<uint32_t>();
+        point_at(o, u.steady, v.steady);
+        // The first epochs with fewer updates in flight: resident workers capped, tables for that many updates in flight.
+        // resident = inflight / ratings a worker keeps in flight, which mf_hogwild_inflight folds in: ask it for one worker.
+        double low_inflight = 0; uint32_t capped = 0;
+        if (prm.early_inflight > 0.f && prm.early_inflight < 1.f && prm.early_inflight_epochs > 0) {
+            const double per_worker = mf_hogwild_inflight(prm.version, (int)prm.k, 1, user_groups, item_groups);
+            const uint32_t resident = per_worker > 0 ? (uint32_t)(inflight / per_worker + 0.5) : 0;
+            capped = (uint32_t)(resident * (double)prm.early_inflight);
+            // what a launch held to that many workers really keeps in flight (whole workgroups per compute unit)
+            low_inflight = capped >= 1 ? mf_hogwild_inflight_capped(prm.version, (int)prm.k, prm.num_workers, user_groups, item_groups, capped) : 0.0;
+            if (!(low_inflight > 0 && low_inflight < inflight)) low_inflight = 0;
+        }
+        if (low_inflight > 0) {
+            const double thin = prm.hot_row_inflight_early > 0 ? prm.hot_row_inflight_early : prm.hot_row_inflight;
+            for (int s = 0; s < 2; ++s)
+                MF_TRY(side[s]->low.upload_from(keep_table(cnt[s], rows[s], n, low_inflight, replicate_above, thin, prm.replica_add_inflight), rows[s]));
+        }
+        // Later epochs with a lower bar for replication (more rows kept as copies in the L2s, fewer added to at the memory side)
+        replicate_above_late = prm.replicate_inflight_late > 0 ? prm.replicate_inflight_late : (prm.replicate_inflight_late < 0 ? replicate_above / 3.0 : 0.0);
+        const bool late = replicate_above > 0 && replicate_above_late > 0 && replicate_above_late < replicate_above && prm.replicate_late_from < prm.epoch;
+        if (late) {
+            for (int s = 0; s < 2; ++s)
+                MF_TRY(side[s]->late.upload_from(keep_table(cnt[s], rows[s], n, inflight, replicate_above_late, prm.hot_row_inflight, prm.replica_add_inflight), rows[s]));
+        }
+        for (int s = 0; s < 2; ++s) {
+            const uint32_t most = std::max(side[s]->steady.slots, std::max(side[s]->low.slots, side[s]->late.slots));
+            if (most) MF_TRY(side[s]->replicas.alloc((size_t)MF_XCDS * most * prm.k * 4, "hipMalloc(row replicas)"));
+        }
         o.user_replicas = u.replicas.p; o.item_replicas = v.replicas.p;
-        o.user_slots = u.slots; o.item_slots = v.slots;
-        if ((u.slots || v.slots) && prm.epoch_splits == 0) {
+        const bool any_slots = u.steady.slots || v.steady.slots || u.late.slots || v.late.slots;
+        if (any_slots && prm.epoch_splits == 0) {
             // replica_merges = 0: a launch of at least 25M ratings, at most four launches (the end of a launch, where the
             // last workers run alone, costs a short epoch 13 % per extra launch and a 100M-rating one 0.1 %)
             const uint32_t by_size = n / 25000000u;
@@ -259,26 +287,16 @@ struct HotRows {
         }
         opt_early = o;
         if (early) { opt_early.user_keep = u.early.as<uint8_t>(); opt_early.item_keep = v.early.as<uint8_t>(); }
-        // The first epochs with fewer updates in flight: resident workers capped, tables for that many updates in flight.
-        // resident = inflight / ratings a worker keeps in flight, which mf_hogwild_inflight folds in: ask it for one worker.
-        low_epochs = 0;
-        if (prm.early_inflight > 0.f && prm.early_inflight < 1.f && prm.early_inflight_epochs > 0) {
-            const double per_worker = mf_hogwild_inflight(prm.version, (int)prm.k, 1, user_groups, item_groups);
-            const uint32_t resident = per_worker > 0 ? (uint32_t)(inflight / per_worker + 0.5) : 0;
-            const uint32_t capped = (uint32_t)(resident * (double)prm.early_inflight);
-            // what a launch held to that many workers really keeps in flight (whole workgroups per compute unit)
-            const double low_inflight = capped >= 1 ? mf_hogwild_inflight_capped(prm.version, (int)prm.k, prm.num_workers, user_groups, item_groups, capped) : 0.0;
-            if (low_inflight > 0 && low_inflight < inflight) {
-                MF_TRY(build_low(u, prm, ucnt, n_users, n, low_inflight));
-                MF_TRY(build_low(v, prm, icnt, n_items, n, low_inflight));
-                opt_low = o;
-                opt_low.resident_workers = capped;
-                opt_low.user_keep = u.low_keep.as<uint8_t>(); opt_low.item_keep = v.low_keep.as<uint8_t>();
-                opt_low.user_slot = u.low_slot.as<uint16_t>(); opt_low.item_slot = v.low_slot.as<uint16_t>();
-                opt_low.user_slot_row = u.low_slot_row.as<uint32_t>(); opt_low.item_slot_row = v.low_slot_row.as<uint32_t>();
-                opt_low.user_slots = u.low_slots; opt_low.item_slots = v.low_slots;
-                low_epochs = prm.early_inflight_epochs;
-            }
+        if (low_inflight > 0) {
+            opt_low = o;
+            opt_low.resident_workers = capped;
+            point_at(opt_low, u.low, v.low);
+            low_epochs = prm.early_inflight_epochs;
+        }
+        if (late) {
+            opt_late = o;
+            point_at(opt_late, u.late, v.late);
+            late_from = prm.replicate_late_from;
         }
         return 0;
     }
@@ -286,10 +304,16 @@ struct HotRows {
     bool all_binary16 = false;      // MASCOT runs: no group has been promoted yet
     const mf_hogwild_options* options(uint32_t e) const
     {
-        opt_current = e < low_epochs ? opt_low : (e < early_epochs ? opt_early : opt_steady);
+        opt_current = e < low_epochs ? opt_low : (e >= late_from ? opt_late : (e < early_epochs ? opt_early : opt_steady));
         opt_current.replica_step_scale = (step_epochs == 0 || e < step_epochs) ? step_scale : 0.f;
         opt_current.all_binary16 = all_binary16 ? 1u : 0u;
         return &opt_current;
+    }
+    // replicated rows per side in the tables most of the run uses
+    uint32_t replicated(int side_index) const
+    {
+        const SideTables& t = side_index ? v : u;
+        return late_from != 0xffffffffu ? t.late.slots : t.steady.slots;
     }
 };
 
@@ -849,6 +873,7 @@ void mf_default_params(mf_params* out)       // main.cu:19-32
     out->hot_row_inflight = 0.0f; out->hot_row_inflight_early = 0.0f; out->hot_row_early_epochs = 0;
     out->replica_step_scale = -1.0f; out->replica_step_epochs = 1;
     out->early_inflight = 0.5f; out->early_inflight_epochs = 1;
+    out->replicate_inflight_late = -1.0f; out->replicate_late_from = 1;
 }
 
 uint32_t mf_group_end_indices(const uint32_t* sorted_cnt, uint32_t n, uint32_t requested_groups, uint32_t* end_idx_out)
@@ -1015,8 +1040,8 @@ uint32_t mf_session_workers(const mf_session* session) { return session && sessi
 int mf_session_hot_rows(const mf_session* session, uint32_t* user_replicated, uint32_t* item_replicated, float* inflight)
 {
     if (!session || !session->run) return invalid("mf_session_hot_rows: null session");
-    if (user_replicated) *user_replicated = session->run->hot.u.slots;
-    if (item_replicated) *item_replicated = session->run->hot.v.slots;
+    if (user_replicated) *user_replicated = session->run->hot.replicated(0);
+    if (item_replicated) *item_replicated = session->run->hot.replicated(1);
     if (inflight) *inflight = (float)session->run->hot.inflight;
     return 0;
 }

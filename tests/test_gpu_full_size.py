@@ -150,11 +150,11 @@ def test_full_size_run_tracks_the_committed_cpu_curves():
     """mf_train -v 1 on configuration 4 at full size (the workload and parameters of bench.py and of the committed CPU
     curves, tests/golden/reference_curve_config4_run*.json: the reference rule run by the checker on host cores) for
     the configured 50 epochs with the library's defaults: every row update carried out, the test RMSE within 0.005 of
-    the CPU curves from epoch 4 on and within 0.002 at epoch 50, the figure BASELINE.json's metric names.  The CPU curves
+    the CPU curves from epoch 3 on and within 0.002 at epoch 50, the figure BASELINE.json's metric names.  The CPU curves
     are the rule's sequential limit (6 threads); the GPU keeps 24,576 updates in flight (half as many in the first epoch,
     mf_params.early_inflight), and a row that takes percents of all ratings keeps one of the many updates in flight on it
-    (as it would on the reference's GPU), which is what the first epochs show: their bounds are the measured gaps
-    (0.024, 0.009, 0.0035..0.0041) plus a margin; epoch 4 measures 0.0035."""
+    (as it would on the reference's GPU), which is what the first two epochs show: their bounds are the measured gaps
+    (0.024, 0.009) plus a margin; epochs 3 and 4 measure 0.003."""
     import glob
     import json
     sys.path.insert(0, ROOT)
@@ -174,9 +174,9 @@ def test_full_size_run_tracks_the_committed_cpu_curves():
     print("epoch 1, 5, 12, 25, 50: gpu", np.round(gpu[[0, 4, 11, 24, 49]], 5), "cpu", np.round(cpu[[0, 4, 11, 24, 49]], 5))
     assert np.all(np.isfinite(gpu)) and np.all(np.diff(gpu[:20]) < 0) and np.all(np.diff(gpu) < 5e-4)      # binary16 groups stall before they are switched
     print("epochs 1..6: gpu - cpu", np.round(gpu[:6] - cpu[:6], 5))
-    for e, bound in enumerate((0.03, 0.012, 0.006)):
+    for e, bound in enumerate((0.03, 0.012)):
         assert abs(gpu[e] - cpu[e]) < bound, (e + 1, gpu[e], cpu[e])
-    assert np.all(np.abs(gpu[3:] - cpu[3:]) < 0.005)
+    assert np.all(np.abs(gpu[2:] - cpu[2:]) < 0.005)
     assert abs(gpu[49] - cpu[49]) < 0.002
 
 
