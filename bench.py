@@ -207,7 +207,7 @@ def main():
     ap.add_argument("--replicate", type=float, default=-1.0, help="mf_params.replicate_inflight (default: derived from learning rate and mean rating)")
     ap.add_argument("--merges", type=int, default=0, help="mf_params.replica_merges (default: the library's)")
     ap.add_argument("--step-epochs", type=int, default=-1, help="mf_params.replica_step_epochs (default: the library's 1; 0 = every epoch)")
-    ap.add_argument("--replicate-late", type=float, default=-1.0, help="mf_params.replicate_inflight_late (default: a third of --replicate's value; 0 = the same bar throughout)")
+    ap.add_argument("--replicate-late", type=float, default=-1.0, help="mf_params.replicate_inflight_late (default: a quarter of --replicate's value; 0 = the same bar throughout)")
     ap.add_argument("--late-from", type=int, default=-1, help="mf_params.replicate_late_from (default: the library's 1, the second epoch)")
     ap.add_argument("--early", type=float, default=-1.0, help="mf_params.early_inflight: fraction of the updates in flight during the first epoch (default: the library's 0.5; 1 = off)")
     ap.add_argument("--step-scale", type=float, default=-1.0, help="mf_params.replica_step_scale (default: the library's; 0 = unscaled steps on replicated rows)")
@@ -299,7 +299,7 @@ def main():
                    "row_updates_carried_out": 1.0 if a.thin == 0 else None,
                    "updates_in_flight": inflight, "replicated_rows": {"user": rep_u, "item": rep_v},
                    "replicate_above_in_flight": {"epochs_before": prm.replicate_late_from, "bar": replicate_bar,
-                                                 "later_bar": (replicate_bar / 3.0 if prm.replicate_inflight_late < 0 else (prm.replicate_inflight_late or replicate_bar))},
+                                                 "later_bar": (replicate_bar / 4.0 if prm.replicate_inflight_late < 0 else (prm.replicate_inflight_late or replicate_bar))},
                    "first_epochs": {"epochs": prm.early_inflight_epochs, "updates_in_flight_fraction": prm.early_inflight, "replica_step_scale": "library default" if a.step_scale < 0 else a.step_scale},
                    "setup_s": round(setup_s, 1)},
         "roofline": {"bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS,

@@ -121,7 +121,7 @@ int main(int argc, const char* argv[])
         if (prm.replicate_inflight < 0) std::cout << "; rows above 0.3 / (learning rate x mean rating) in flight are replicated per XCD";
         else if (prm.replicate_inflight > 0) std::cout << "; rows above " << prm.replicate_inflight << " in flight are replicated per XCD";
         if (prm.replicate_inflight != 0 && prm.replica_merges) std::cout << ", merged " << prm.replica_merges << " times per epoch";
-        if (prm.replicate_inflight != 0 && prm.replicate_inflight_late < 0) std::cout << " (above a third of that from epoch " << prm.replicate_late_from + 1 << " on)";
+        if (prm.replicate_inflight != 0 && prm.replicate_inflight_late < 0) std::cout << " (above a quarter of that from epoch " << prm.replicate_late_from + 1 << " on)";
         else if (prm.replicate_inflight != 0 && prm.replicate_inflight_late > 0) std::cout << " (above " << prm.replicate_inflight_late << " from epoch " << prm.replicate_late_from + 1 << " on)";
         if (prm.hot_row_inflight > 0) std::cout << "; rows above " << prm.hot_row_inflight << " in flight are thinned";
     }

@@ -267,7 +267,7 @@ struct HotRows {
                 MF_TRY(side[s]->low.upload_from(keep_table(cnt[s], rows[s], n, low_inflight, replicate_above, thin, prm.replica_add_inflight), rows[s]));
         }
         // Later epochs with a lower bar for replication (more rows kept as copies in the L2s, fewer added to at the memory side)
-        replicate_above_late = prm.replicate_inflight_late > 0 ? prm.replicate_inflight_late : (prm.replicate_inflight_late < 0 ? replicate_above / 3.0 : 0.0);
+        replicate_above_late = prm.replicate_inflight_late > 0 ? prm.replicate_inflight_late : (prm.replicate_inflight_late < 0 ? replicate_above / 4.0 : 0.0);
         const bool late = replicate_above > 0 && replicate_above_late > 0 && replicate_above_late < replicate_above && prm.replicate_late_from < prm.epoch;
         if (late) {
             for (int s = 0; s < 2; ++s)

@@ -441,12 +441,13 @@ typedef struct {
     float replicate_inflight_late; /* from epoch replicate_late_from on (counted from 0; default 1: the second epoch) rows above
                                  this many updates in flight get copies: a lower bar than replicate_inflight keeps more
                                  rows in the L2s and adds to fewer at the memory side.  Past the first epoch the mean of
-                                 the copies loses nothing measurable (100M ratings: bars 8.68 / 6 / 4 / 3 / 2.5 from the
-                                 fifth epoch on give 13.5 / 13.0 / 12.2 / 11.7 / 11.5 ms per epoch and the same test RMSE up
-                                 to epoch 50 within 0.0005; from the second or third epoch on, epochs 3 and 4 end 0.001
-                                 closer to the sequential run), while in the first epoch every averaged row shows (bars
+                                 the copies loses nothing measurable (100M ratings: bars 8.68 / 6 / 4 / 3 / 2 from the
+                                 second epoch on give 13.5 / 13.0 / 12.2 / 11.7 / 11.3 ms per epoch and the same test RMSE up
+                                 to epoch 50 within 0.0005, epochs 3 and 4 ending 0.001 closer to the sequential run with
+                                 the lower bars; only with every row above one update in flight replicated do epochs 2
+                                 to 8 fall behind, by 0.001), while in the first epoch every averaged row shows (bars
                                  8.68 / 6 / 4 / 3 throughout: 0.023 / 0.027 / 0.030 / 0.032 above the sequential run after
-                                 epoch 1).  < 0 (default): a third of replicate_inflight's value; 0 = the same bar
+                                 epoch 1).  < 0 (default): a quarter of replicate_inflight's value; 0 = the same bar
                                  throughout */
     uint32_t replicate_late_from;
 } mf_params;
