@@ -26,16 +26,17 @@ namespace mf {
 template <int K, bool COH, bool SAMPLED, bool MIXED = true> struct MascotRuleT {
     static constexpr int E = K / 64;                        // elements per lane
     static constexpr int kAhead = 3, kRing = 8;
-    // chunks of mixed precisions look two ratings ahead: their rows take three registers per side while in flight, and
-    // every rating compares with one older row less (measured: 3 % per mixed epoch over three ratings, 4 % over one)
+    // chunks of mixed precisions look two ratings ahead (measured at 100M and 250M ratings: three ratings make the states
+    // with some groups promoted 1-20 % slower and only the all-promoted state 3 % faster)
     static constexpr int kAheadClass2 = 2;
     // chunk classes: 1 = every rating of the chunk touches two binary16 rows (the state every group starts in): loads
     // and arithmetic without any branching; 2 = any mix of precisions, every rating inside the group tables: every
-    // path through a rating issues the same number of memory instructions; 0 = anything, including ratings that are
-    // skipped (an index outside the tables)
+    // rating loads its rows with the same instructions and branches four ways, on the precisions of its two rows, into
+    // arithmetic and stores written for that case, each way issuing one store per side; 0 = anything, including ratings
+    // that are skipped (an index outside the tables)
     static constexpr int kClasses = MIXED ? 3 : 2;
-    // the build for all-binary16 runs asks for six wavefronts per SIMD (80 registers): its hot loop needs fewer, the
-    // general path for mixed chunks, which it should never take, is what would exceed them
+    // no register limit is asked for: the build for all-binary16 runs fits six wavefronts per SIMD by itself (80), the
+    // build with the mixed path takes 83 (five), and held to 80 it spills and gains nothing (measured)
     static constexpr int kMinWavesPerSimd = 1;
     using HV = typename std::conditional<E == 2, half2_t, half_t>::type;
 
@@ -59,8 +60,8 @@ template <int K, bool COH, bool SAMPLED, bool MIXED = true> struct MascotRuleT {
         v.group_ptr = a.q; v.group_end = a.item_end; v.group_prec = a.item_prec; v.groups = a.item_groups;
     }
     static constexpr bool kSplittable = true;
-    // raw row registers: binary16 rows use r[0] only.  ph, qh: chunks of mixed precisions load a binary16 row into these
-    // and a binary32 row into p, q (load_mixed); whichever the row is not comes back as zero
+    // raw row registers: binary16 rows use r[0] only.  ph, qh (k = 64 only): chunks of mixed precisions load a binary16 row
+    // into these and a binary32 row into p, q (load_mixed); whichever the row is not comes back as zero
     struct Row { uint32_t p[E], q[E], ph, qh; };
     struct Prep { uint64_t pptr, qptr; uint32_t flags; };
     struct Info { float r; uint64_t pptr, qptr; uint32_t flags, thin; };
@@ -186,56 +187,27 @@ template <int K, bool COH, bool SAMPLED, bool MIXED = true> struct MascotRuleT {
             else r[0] = row_load((reinterpret_cast<const uint16_t*>(ptr) + lane));
         }
     }
-    // Chunks of mixed precisions (class 2): the same instructions for a row of either precision, so that a rating takes
-    // no branch on its way to the rows and the compiler can count the loads in flight.  Every access goes through a
-    // window over the row (a buffer resource of the row's size) twice, once with the instruction for each precision;
-    // the one that does not apply aims past the window and is dropped by the hardware (a dropped load returns zero).
-    // A binary32 row is moved with 8-byte accesses (k = 128; 4-byte at k = 64), a binary16 row with 4-byte ones (2-byte).
+    // Chunks of mixed precisions (class 2): the same load instruction for a row of either precision, so that a rating
+    // takes no branch on its way to the rows and the compiler can count the loads in flight (a branch between two load
+    // instructions was measured: the counted waits become waits for everything, 42 instead of 29 ms per epoch on 250M
+    // ratings).  The load goes through a window over the row (a buffer resource of the row's size): accesses past its
+    // end are dropped by the hardware, dword by dword, and come back zero.
+    // k = 128: one 8-byte load serves both precisions.  A binary32 row is read at 8 bytes per lane; a binary16 row at 4
+    // bytes per lane, where the load's first dword is the lane's pair of elements and its second the next lane's, which
+    // nothing uses (the last lane's second dword lies past the window).
+    // k = 64: a 4-byte load for a binary32 row and a 2-byte load for a binary16 row, the one that does not apply aimed past
+    // the window; `h` receives the binary16 row and arrive() merges the two registers.
     static constexpr uint32_t kPast = 0x7ffff000u;       // a byte offset past every window
-    struct Access { row_window_t row; uint32_t wide, narrow; };      // this lane's byte offset for each precision's instruction
-    static __device__ __forceinline__ Access access(uint64_t ptr, bool fp32, int lane)
-    {
-        return Access{row_window(ptr, fp32 ? K * 4u : K * 2u), fp32 ? (uint32_t)lane * (E * 4u) : kPast, fp32 ? kPast : (uint32_t)lane * (E * 2u)};
-    }
     static __device__ __forceinline__ void load_mixed(uint32_t* r, uint32_t& h, uint64_t ptr, bool fp32, int lane)
     {
-        const Access a = access(ptr, fp32, lane);
+        const row_window_t w = row_window(ptr, fp32 ? K * 4u : K * 2u);
         if constexpr (E == 2) {
-            const auto v = __builtin_amdgcn_raw_buffer_load_b64(a.row, (int)a.wide, 0, 0);
+            const auto v = __builtin_amdgcn_raw_buffer_load_b64(w, (int)((uint32_t)lane << (fp32 ? 3u : 2u)), 0, 0);
             r[0] = v[0]; r[1] = v[1];
-            h = __builtin_amdgcn_raw_buffer_load_b32(a.row, (int)a.narrow, 0, 0);
+            h = 0u;
         } else {
-            r[0] = __builtin_amdgcn_raw_buffer_load_b32(a.row, (int)a.wide, 0, 0);
-            h = __builtin_amdgcn_raw_buffer_load_b16(a.row, (int)a.narrow, 0, 0);
-        }
-    }
-    template <bool C> static __device__ __forceinline__ void store_mixed(const uint32_t* r, uint64_t ptr, bool fp32, int lane)
-    {
-        const Access a = access(ptr, fp32, lane);
-        if constexpr (E == 2) {
-            window_store<C>(a.row, a.wide, (uint64_t)r[0] | ((uint64_t)r[1] << 32));
-            window_store<C>(a.row, a.narrow, r[0]);
-        } else {
-            window_store<C>(a.row, a.wide, r[0]);
-            window_store<C>(a.row, a.narrow, (uint16_t)r[0]);
-        }
-    }
-    // d: the change of this lane's elements in binary32; a binary16 row receives it rounded
-    static __device__ __forceinline__ void add_mixed(uint64_t ptr, const float* d, bool fp32, int lane)
-    {
-        const Access a = access(ptr, fp32, lane);
-        if constexpr (E == 2) {
-            float lower, upper;
-            const uint32_t at = fp32 ? halves_of_row(d, lower, upper, lane) : (halves_of_row(d, lower, upper, lane), kPast);
-            window_add(a.row, at, lower);
-            window_add(a.row, at + K * 2u, upper);
-            window_add(a.row, a.narrow, narrow(d));
-        } else {
-            window_add(a.row, a.wide, d[0]);
-            // one element per lane: even lanes add the pair (own, right neighbour), odd lanes aim past the window
-            const uint32_t mine = (uint32_t)bits(narrow(d));
-            const uint32_t other = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)mine, 0xB1 /* quad_perm 1,0,3,2 */, 0xf, 0xf, false);
-            window_add(a.row, (lane & 1) ? kPast : a.narrow, from_bits<half2_t>(mine | (other << 16)));
+            r[0] = __builtin_amdgcn_raw_buffer_load_b32(w, (int)(fp32 ? (uint32_t)lane * 4u : kPast), 0, 0);
+            h = __builtin_amdgcn_raw_buffer_load_b16(w, (int)(fp32 ? kPast : (uint32_t)lane * 2u), 0, 0);
         }
     }
     // hot row (Schedule::keep_u): add the change of this lane's elements to the row in memory
@@ -295,7 +267,7 @@ template <int K, bool COH, bool SAMPLED, bool MIXED = true> struct MascotRuleT {
             load_side(row.q, i.qptr, i.flags & 2u, lane);
         }
     }
-    // load_mixed: the row came through one of two windows, the other gave zero
+    // load_mixed at k = 64: the row came through one of two loads, the other gave zero
     template <int CLS> __device__ __forceinline__ void arrive(Row& row) const
     {
         if constexpr (CLS == 2) { row.p[0] |= row.ph; row.q[0] |= row.qh; }
@@ -424,33 +396,52 @@ template <int K, bool COH, bool SAMPLED, bool MIXED = true> struct MascotRuleT {
     // the same for a binary16 row whose change was computed in binary16 (mascot_sgd_kernel.h:188-278)
     template <int CLS, bool HOT> __device__ __forceinline__ void write_side_half(const uint32_t* r, HV d, uint64_t ptr, uint32_t bits_) const
     {
-        if constexpr (CLS == 2) {
-            float df[E];
-#pragma unroll
-            for (int e = 0; e < E; ++e) df[e] = widen(d, e);      // exact, and narrowed again exactly by add_mixed
-            write_side<CLS, HOT>(r, df, ptr, false, bits_);
-        } else {
-            if (HOT && (bits_ & 20u) == 16u) store_side<false>(r, ptr, false, lane);
-            else if (HOT && (bits_ & 4u)) add_side_half(ptr, d, lane);
-            else store_side(r, ptr, false, lane);
-        }
+        if (HOT && (bits_ & 20u) == 16u) store_side<false>(r, ptr, false, lane);
+        else if (HOT && (bits_ & 4u)) add_side_half(ptr, d, lane);
+        else store_side(r, ptr, false, lane);
     }
     template <int CLS, bool HOT> __device__ __forceinline__ void write_side(const uint32_t* r, const float* d, uint64_t ptr, bool fp32, uint32_t bits_) const
     {
-        if constexpr (CLS == 2) {
-            if (HOT && (bits_ & 20u) == 16u) store_mixed<false>(r, ptr, fp32, lane);
-            else if (HOT && (bits_ & 4u)) add_mixed(ptr, d, fp32, lane);
-            else store_mixed<COH>(r, ptr, fp32, lane);
-        } else {
-            if (HOT && (bits_ & 20u) == 16u) store_side<false>(r, ptr, fp32, lane);
-            else if (HOT && (bits_ & 4u)) { if (fp32) add_side_float(ptr, d, lane); else add_side_half(ptr, narrow(d), lane); }
-            else store_side(r, ptr, fp32, lane);
+        static_assert(CLS != 2, "chunks of mixed precisions write through write_side_known");
+        if (HOT && (bits_ & 20u) == 16u) store_side<false>(r, ptr, fp32, lane);
+        else if (HOT && (bits_ & 4u)) { if (fp32) add_side_float(ptr, d, lane); else add_side_half(ptr, narrow(d), lane); }
+        else store_side(r, ptr, fp32, lane);
+    }
+    // The same for a side whose precision is a compile-time constant: one store, or the adds of that precision, through
+    // plain global accesses.  Chunks of mixed precisions write this way: their update branches four ways on the precisions
+    // of the rating's two rows (wave-uniform), and every way issues one store per side, so the counted waits for the row
+    // loads that are in flight hold on all of them.
+    template <bool HOT, bool FP32> __device__ __forceinline__ void write_side_known(const uint32_t* r, const float* d, uint64_t ptr, uint32_t bits_) const
+    {
+        if (HOT && (bits_ & 20u) == 16u) store_side<false>(r, ptr, FP32, lane);
+        else if (HOT && (bits_ & 4u)) {
+            if constexpr (FP32 && E == 2) {
+                float lower, upper;
+                const uint32_t at = halves_of_row(d, lower, upper, lane);
+                row_add(reinterpret_cast<float*>(ptr + at), lower);
+                row_add(reinterpret_cast<float*>(ptr + at + K * 2u), upper);
+            } else if constexpr (FP32) add_side_float(ptr, d, lane);
+            else add_side_half(ptr, narrow(d), lane);
         }
+        else store_side(r, ptr, FP32, lane);
     }
     template <int CLS, bool HOT, bool SCALED> __device__ __forceinline__ void update(Row& row, const Info& i, uint32_t processed) const
     {
+        if constexpr (CLS == 2) {
+            switch (i.flags & 3u) {
+            case 0u: update_case<CLS, HOT, SCALED, 0>(row, i, processed); break;
+            case 1u: update_case<CLS, HOT, SCALED, 1>(row, i, processed); break;
+            case 2u: update_case<CLS, HOT, SCALED, 2>(row, i, processed); break;
+            default: update_case<CLS, HOT, SCALED, 3>(row, i, processed); break;
+            }
+        } else update_case<CLS, HOT, SCALED, -1>(row, i, processed);
+    }
+    // CASE: the precisions of the two rows when they are known at compile time (bit 0 the user row is binary32, bit 1 the
+    // item row), or -1: read from the rating's flags
+    template <int CLS, bool HOT, bool SCALED, int CASE> __device__ __forceinline__ void update_case(Row& row, const Info& i, uint32_t processed) const
+    {
         if (CLS == 0 && (i.flags & kSkip)) return;
-        const bool up = CLS != 1 && (i.flags & 1u), ip = CLS != 1 && (i.flags & 2u);
+        const bool up = CASE >= 0 ? (CASE & 1) != 0 : (CLS != 1 && (i.flags & 1u)), ip = CASE >= 0 ? (CASE & 2) != 0 : (CLS != 1 && (i.flags & 2u));
         // thinned updates (only read the row) occur in chunks of class 0 only: classify() sends their chunks there
         const bool skip_p = CLS == 0 && HOT && (i.thin & 1u), skip_q = CLS == 0 && HOT && (i.thin & 2u);
         const bool sampled = SAMPLED && processed >= first_sample;
@@ -468,11 +459,11 @@ template <int K, bool COH, bool SAMPLED, bool MIXED = true> struct MascotRuleT {
             const HV gq = ruv * P - lam_h * Q;
             if (!skip_p) {
                 row.p[0] = bits(HV(__builtin_elementwise_fma(lr_p, gp, P)));
-                write_side_half<CLS, HOT>(row.p, lr_p * gp, i.pptr, i.thin);
+                write_side_half<(CLS == 2 ? 1 : CLS), HOT>(row.p, lr_p * gp, i.pptr, i.thin);
             }
             if (!skip_q) {
                 row.q[0] = bits(HV(__builtin_elementwise_fma(lr_q, gq, Q)));
-                write_side_half<CLS, HOT>(row.q, lr_q * gq, i.qptr, i.thin >> 1);
+                write_side_half<(CLS == 2 ? 1 : CLS), HOT>(row.q, lr_q * gq, i.qptr, i.thin >> 1);
             }
             if (sampled) {
                 float g[E];
@@ -511,14 +502,16 @@ template <int K, bool COH, bool SAMPLED, bool MIXED = true> struct MascotRuleT {
 #pragma unroll
                 for (int e = 0; e < E; ++e) row.p[e] = up ? bits(np_[e]) : (e == 0 ? rounded : row.p[e]);
                 if (HOT && (i.thin & 4u)) { for (int e = 0; e < E; ++e) d[e] = lr_p * gp[e]; }
-                write_side<CLS, HOT>(row.p, d, i.pptr, up, i.thin);
+                if constexpr (CASE >= 0) { if constexpr ((CASE & 1) != 0) write_side_known<HOT, true>(row.p, d, i.pptr, i.thin); else write_side_known<HOT, false>(row.p, d, i.pptr, i.thin); }
+                else write_side<CLS, HOT>(row.p, d, i.pptr, up, i.thin);
             }
             if (!skip_q) {
                 const uint32_t rounded = bits(narrow(nq_));
 #pragma unroll
                 for (int e = 0; e < E; ++e) row.q[e] = ip ? bits(nq_[e]) : (e == 0 ? rounded : row.q[e]);
                 if (HOT && (i.thin & 8u)) { for (int e = 0; e < E; ++e) d[e] = lr_q * gq[e]; }
-                write_side<CLS, HOT>(row.q, d, i.qptr, ip, i.thin >> 1);
+                if constexpr (CASE >= 0) { if constexpr ((CASE & 2) != 0) write_side_known<HOT, true>(row.q, d, i.qptr, i.thin >> 1); else write_side_known<HOT, false>(row.q, d, i.qptr, i.thin >> 1); }
+                else write_side<CLS, HOT>(row.q, d, i.qptr, ip, i.thin >> 1);
             }
             if (sampled) {
                 if (!up) sample(gp, ug, true);

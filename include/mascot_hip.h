@@ -447,8 +447,10 @@ typedef struct {
                                  the lower bars; only with every row above one update in flight replicated do epochs 2
                                  to 8 fall behind, by 0.001), while in the first epoch every averaged row shows (bars
                                  8.68 / 6 / 4 / 3 throughout: 0.023 / 0.027 / 0.030 / 0.032 above the sequential run after
-                                 epoch 1).  < 0 (default): a quarter of replicate_inflight's value; 0 = the same bar
-                                 throughout */
+                                 epoch 1).  < 0 (default): a quarter of replicate_inflight's value in runs that keep at
+                                 least 4096 updates in flight (1024 workers), the same bar throughout in smaller ones,
+                                 whose epochs are bound by the latency of a worker's chain and gain little from more
+                                 copies; 0 = the same bar throughout */
     uint32_t replicate_late_from;
 } mf_params;
 
