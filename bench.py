@@ -322,7 +322,8 @@ def main():
         "test_rmse_per_epoch": [round(float(x), 5) for x in main_run["rmse"]],
     }
     traffic = profiled_traffic(a.config, n_train, k, a.seed, W)
-    if traffic is not None and a.replicate < 0 and a.thin == 0 and a.step_scale < 0 and a.step_epochs < 0 and not a.merges:
+    if traffic is not None and a.replicate < 0 and a.thin == 0 and a.step_scale < 0 and a.step_epochs < 0 and not a.merges \
+            and a.replicate_late < 0 and a.late_from < 0 and a.early < 0:
         out["roofline"]["traffic"] = traffic["bytes_per_epoch"]
         out["roofline"]["traffic_source"] = traffic["source"]
         out["roofline"]["hbm_side"] = {"frac": traffic["bytes_per_epoch"] / (float(np.mean(plain)) / 1e3) / 1e9 / PEAK_HBM_GBS,
