@@ -334,6 +334,45 @@ def test_mascot_half_config2_with_chosen_workers(orc):
     assert abs(out["rmse"][-1] - ref[-1]) < 0.005
 
 
+def test_first_epoch_and_later_epochs_get_their_own_row_treatment():
+    """mf_train's schedule of the row treatment (mf_params.early_inflight, replicate_inflight_late): the launches of the
+    first epoch are held to half the resident workers and use tables built for that many updates in flight, with the bar
+    for per-XCD copies from mf_replicate_threshold; from the second epoch on the launches are not held and the bar is a
+    quarter of it, so more rows have copies.  A run with fewer than 1024 workers is left alone: one table set, no cap."""
+    import importlib
+    capi = importlib.import_module("icdm-2021_mascot_amd.capi")
+    h = mfutil.hip()
+    n_users, n_items = 30000, 4000
+    R = mfutil.make_ratings(123, n_users, n_items, 3_000_000, rank=8, alpha=1.05)
+    train, test = _split(R, 2_900_000)
+
+    def tables(workers, **kw):
+        prm = h.default_params(k=128, num_workers=workers, epoch=4, learning_rate=0.01, lam=0.015, decay=0.1, version=1, seed=3,
+                               user_group_num=20, item_group_num=20, sample_ratio=0.05, interval=2, error_threshold=20.0, **kw)
+        p, q = h.init_model(n_users, n_items, 128, 3)
+        s = capi.Session(h, prm, train, n_users, n_items, test, p, q)
+        out = []
+        for epoch in (0, 1, 2):
+            o = capi.HogwildOptions.from_address(s.device_state(epoch)[1])
+            out.append((o.resident_workers, o.user_slots + o.item_slots, o.replica_step_scale))
+        rmse = [s.epoch()[0] for _ in range(3)]
+        s.close()
+        assert np.all(np.isfinite(rmse)) and rmse[2] < rmse[0]
+        return out
+
+    first, second, third = tables(8192)
+    resident = int(h.lib.mf_hogwild_inflight(1, 128, 8192, 20, 20)) // 4
+    assert first[0] == resident // 2 and second[0] == 0 and third == second          # the cap: first epoch only
+    assert 0 < first[1] < second[1]                                                     # fewer rows have copies in the first epoch
+    assert first[2] > 1.0 and second[2] == 0.0                                          # scaled steps: first epoch only
+    one_bar = tables(8192, replicate_inflight_late=0.0)
+    assert first[1] == one_bar[0][1] and first[1] < one_bar[1][1] < second[1]           # F back to full: more rows above the same bar
+    off = tables(8192, early_inflight=1.0, replicate_inflight_late=0.0)
+    assert off[0][0] == 0 and off[0][1] == off[1][1] == one_bar[1][1]
+    small = tables(512)
+    assert small[0][0] == 0 and small[0][1] == small[1][1] == small[2][1]
+
+
 def _write_tsv(path, R, offset=0):
     with open(path, "w") as f:
         for r, u, i in zip(R["r"].tolist(), R["u"].tolist(), R["i"].tolist()):
