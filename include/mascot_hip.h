@@ -499,7 +499,9 @@ int mf_session_epoch(mf_session* session, double* test_rmse, float* sgd_ms);
 int mf_session_finish(mf_session* session, float* p, float* q);
 void mf_session_destroy(mf_session* session);
 /* The worker count the session runs (mf_params.num_workers, or mf_auto_workers), and its hot rows: rows replicated per
- * side and the updates in flight the tables were built for (0 when the run has no tables). */
+ * side in the tables most of the run uses (those of the later epochs when the bar for copies is lowered after the first
+ * ones, mf_params.replicate_inflight_late) and the updates in flight those tables were built for (0 when the run has no
+ * tables). */
 uint32_t mf_session_workers(const mf_session* session);
 int mf_session_hot_rows(const mf_session* session, uint32_t* user_replicated, uint32_t* item_replicated, float* inflight);
 /* The session's training ratings on the device (shuffled; for MASCOT re-indexed to sorted rows) and the launch options
