@@ -73,8 +73,8 @@ __device__ __forceinline__ void process_chunk(Rule& rule, const Rating& my, cons
 template <class Rule, int CLS, class = void> struct ahead_of { static constexpr int value = Rule::kAhead; };
 template <class Rule> struct ahead_of<Rule, 2, std::void_t<decltype(Rule::kAheadClass2)>> { static constexpr int value = Rule::kAheadClass2; };
 // A rule may prepare a row whose loads have arrived before it is compared with older rows (arrive<CLS>).
-template <int CLS, class Rule, class Row> __device__ __forceinline__ auto row_arrived(const Rule& rule, Row& row, int) -> decltype(rule.template arrive<CLS>(row), void()) { rule.template arrive<CLS>(row); }
-template <int CLS, class Rule, class Row> __device__ __forceinline__ void row_arrived(const Rule&, Row&, long) {}
+template <int CLS, class Rule, class Row, class Info> __device__ __forceinline__ auto row_arrived(const Rule& rule, Row& row, const Info& i, int) -> decltype(rule.template arrive<CLS>(row, i), void()) { rule.template arrive<CLS>(row, i); }
+template <int CLS, class Rule, class Row, class Info> __device__ __forceinline__ void row_arrived(const Rule&, Row&, const Info&, long) {}
 
 template <class Rule, int CLS, bool HOT, bool SCALED>
 __device__ __forceinline__ void process_full_chunk(Rule& rule, const Rating& my, const typename Rule::Prep& prep, uint32_t processed)
@@ -93,7 +93,7 @@ __device__ __forceinline__ void process_full_chunk(Rule& rule, const Rating& my,
     };
     auto step = [&](auto D, int j) {
         constexpr int d = decltype(D)::value;
-        row_arrived<CLS>(rule, ring[d], 0);
+        row_arrived<CLS>(rule, ring[d], inf[d], 0);
         static_for<0, A>([&](auto H) {
             constexpr int h = A - decltype(H)::value;          // A, A-1, ..., 1: newest wins
             constexpr int sh = (d - h + 2 * S) % S;

@@ -60,9 +60,8 @@ template <int K, bool COH, bool SAMPLED, bool MIXED = true> struct MascotRuleT {
         v.group_ptr = a.q; v.group_end = a.item_end; v.group_prec = a.item_prec; v.groups = a.item_groups;
     }
     static constexpr bool kSplittable = true;
-    // raw row registers: binary16 rows use r[0] only.  ph, qh (k = 64 only): chunks of mixed precisions load a binary16 row
-    // into these and a binary32 row into p, q (load_mixed); whichever the row is not comes back as zero
-    struct Row { uint32_t p[E], q[E], ph, qh; };
+    // raw row registers: binary16 rows use r[0] only
+    struct Row { uint32_t p[E], q[E]; };
     struct Prep { uint64_t pptr, qptr; uint32_t flags; };
     struct Info { float r; uint64_t pptr, qptr; uint32_t flags, thin; };
     // flags: bit0 user row is fp32, bit1 item row is fp32, bit2 rating is skipped (index outside the
@@ -195,19 +194,16 @@ template <int K, bool COH, bool SAMPLED, bool MIXED = true> struct MascotRuleT {
     // k = 128: one 8-byte load serves both precisions.  A binary32 row is read at 8 bytes per lane; a binary16 row at 4
     // bytes per lane, where the load's first dword is the lane's pair of elements and its second the next lane's, which
     // nothing uses (the last lane's second dword lies past the window).
-    // k = 64: a 4-byte load for a binary32 row and a 2-byte load for a binary16 row, the one that does not apply aimed past
-    // the window; `h` receives the binary16 row and arrive() merges the two registers.
-    static constexpr uint32_t kPast = 0x7ffff000u;       // a byte offset past every window
-    static __device__ __forceinline__ void load_mixed(uint32_t* r, uint32_t& h, uint64_t ptr, bool fp32, int lane)
+    // k = 64: one 4-byte load.  A binary32 row is read at 4 bytes per lane; of a binary16 row every lane reads the dword
+    // that holds its element and its neighbour's, and arrive() keeps the lane's half.
+    static __device__ __forceinline__ void load_mixed(uint32_t* r, uint64_t ptr, bool fp32, int lane)
     {
         const row_window_t w = row_window(ptr, fp32 ? K * 4u : K * 2u);
         if constexpr (E == 2) {
             const auto v = __builtin_amdgcn_raw_buffer_load_b64(w, (int)((uint32_t)lane << (fp32 ? 3u : 2u)), 0, 0);
             r[0] = v[0]; r[1] = v[1];
-            h = 0u;
         } else {
-            r[0] = __builtin_amdgcn_raw_buffer_load_b32(w, (int)(fp32 ? (uint32_t)lane * 4u : kPast), 0, 0);
-            h = __builtin_amdgcn_raw_buffer_load_b16(w, (int)(fp32 ? kPast : (uint32_t)lane * 2u), 0, 0);
+            r[0] = __builtin_amdgcn_raw_buffer_load_b32(w, (int)(((uint32_t)lane >> (fp32 ? 0u : 1u)) << 2), 0, 0);
         }
     }
     // hot row (Schedule::keep_u): add the change of this lane's elements to the row in memory
@@ -257,8 +253,8 @@ template <int K, bool COH, bool SAMPLED, bool MIXED = true> struct MascotRuleT {
             load_side(row.p, i.pptr, false, lane);
             load_side(row.q, i.qptr, false, lane);
         } else if constexpr (CLS == 2) {
-            load_mixed(row.p, row.ph, i.pptr, i.flags & 1u, lane);
-            load_mixed(row.q, row.qh, i.qptr, i.flags & 2u, lane);
+            load_mixed(row.p, i.pptr, i.flags & 1u, lane);
+            load_mixed(row.q, i.qptr, i.flags & 2u, lane);
         } else {
 #pragma unroll
             for (int e = 0; e < E; ++e) { row.p[e] = 0; row.q[e] = 0; }
@@ -267,10 +263,15 @@ template <int K, bool COH, bool SAMPLED, bool MIXED = true> struct MascotRuleT {
             load_side(row.q, i.qptr, i.flags & 2u, lane);
         }
     }
-    // load_mixed at k = 64: the row came through one of two loads, the other gave zero
-    template <int CLS> __device__ __forceinline__ void arrive(Row& row) const
+    // load_mixed at k = 64: a binary16 row arrives as the dword that holds the lane's element and its neighbour's; keep
+    // the lane's half in the low bits, the form every other path leaves a binary16 element in (wave-uniform selects)
+    template <int CLS> __device__ __forceinline__ void arrive(Row& row, const Info& i) const
     {
-        if constexpr (CLS == 2) { row.p[0] |= row.ph; row.q[0] |= row.qh; }
+        if constexpr (CLS == 2 && E == 1) {
+            const uint32_t shift = ((uint32_t)lane & 1u) * 16u;
+            row.p[0] = (i.flags & 1u) ? row.p[0] : ((row.p[0] >> shift) & 0xffffu);
+            row.q[0] = (i.flags & 2u) ? row.q[0] : ((row.q[0] >> shift) & 0xffffu);
+        }
     }
     // selects, no branches: a branch here would sit between the row loads and their first use
     __device__ __forceinline__ void forward(Row& nxt, const Info& in, const Row& cur, const Info& ic) const

@@ -175,7 +175,8 @@ int mf_generate_ratings_host(const mf_synth_config* cfg, uint64_t seed, uint64_t
  * arithmetic.  Worker w (one wavefront) walks ratings [w*ceil(n/W), (w+1)*ceil(n/W)); per rating it reads row u of p
  * and row i of q (row_bytes = 128, 256 or 512 bytes each: k = 64 binary16, k = 128 binary16 / k = 64 binary32,
  * k = 128 binary32) and writes both back unchanged, with the store policy, hot-row tables and replicated rows of
- * `options` (NULL = defaults; `launches` is ignored, replica slots are taken as row_bytes wide): a thinned update
+ * `options` (NULL = defaults; `launches` is ignored, replica slots are taken as row_bytes wide, so the options' replica
+ * arrays must hold MF_XCDS * slots * row_bytes bytes: with the options of an update call at rank k, row_bytes <= 4 k): a thinned update
  * only reads its row, an added update is a store here, a replicated row is read and written in this XCD's copy.
  * p and q keep their contents (writes of other code that race with the probe may be lost).  The time of this launch is
  * what the memory system sustains for the sequence of addresses and the write policy of an epoch; bench.py reports the
