@@ -419,7 +419,8 @@ typedef struct {
                                  added to the XCD's copy (MF_KEEP_REPLICATED_ADDED) instead of stored.  Default 0: at
                                  100M ratings the extra atomic adds cost 9 ms per epoch and gain 0.0007 test RMSE */
     float replica_step_scale; /* mf_hogwild_options::replica_step_scale.  < 0 (default): mf_replica_step_scale(learning_rate,
-                                 mean rating); 0 = off (unscaled steps, mean of the changed copies) */
+                                 mean rating), for MuPPET (version 3) 0: its 8-bit passes diverge, at random, at factors
+                                 the other rules run at.  0 = off (unscaled steps, mean of the changed copies) */
     uint32_t wg_counts_updates; /* 0 (default): num_workers is the number of workers (wavefronts), each of which keeps four
                                  ratings in flight (two for MuPPET and AFP), so -wg W puts 4 W updates in flight where the
                                  reference's -wg W puts W.  1: num_workers is the reference's figure, the updates in
