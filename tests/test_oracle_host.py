@@ -26,7 +26,7 @@ def test_auto_workers(lib):
         assert lib.mf_auto_workers(n) % 4 == 0
 
 
-def test_update_count_is_smallest_cover_and_matches_survey_table(orc, lib):
+def test_update_count_is_smallest_cover_and_matches_hand_computed_table(orc, lib):
     # configs of the benchmark definition with the default 2048 workers: 2, 31, 77, 382, 954 windows
     for n, want in ((400_000, 2), (8_000_000, 31), (20_000_000, 77), (100_000_000, 382), (250_000_000, 954)):
         assert orc.lib.orc_update_count(n, 2048, 128) == want == lib.mf_update_count(n, 2048, 128)
