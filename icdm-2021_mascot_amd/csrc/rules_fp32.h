@@ -17,12 +17,22 @@ template <int K> struct DenseRow {
 };
 struct DenseInfo { float r; uint32_t u, v, thin; };
 struct NoPrep {};
+// What the dense fp32 rules broadcast per rating: the two rows as addresses (the matrix row, or this XCD's copy of a
+// replicated row) and Rating::thin with four more bits, one per store window of the hot-row code (DenseBase::store).
+// Addresses and window bits are computed once per chunk across the 64 lanes (DenseBase::prepare); per rating that costs
+// two more v_readlane where the scalar unit would otherwise rebuild both addresses from the row ids for the loads and
+// again for the stores and derive the four window sizes from thin (about forty scalar instructions per rating).
+// Measured at 100M ratings: 7 to 11 % per epoch at k = 64, where these rules are bound by instruction issue, nothing at
+// k = 128, where they are bound by the memory side; at 8M and 20M ratings, where a worker's chain of ratings is bound by
+// latency, 5 and 13 % at k = 128 and 20 % at k = 64.
+struct DenseAddrInfo { float r; uint32_t thin; uint64_t u, v; };
+struct DenseAddrPrep { uint64_t pu, pv; uint32_t thin; };
 
 template <int K, bool COH> struct DenseBase {
     static constexpr int E = K / 64;
     using Row = DenseRow<K>;
-    using Info = DenseInfo;
-    using Prep = NoPrep;
+    using Info = DenseAddrInfo;      // u, v: the addresses of the two rows
+    using Prep = DenseAddrPrep;
     static constexpr int kClasses = 1;
     static constexpr int kK = K;
     template <class Params> static void row_storage(const Params& a, RowStorage& u, RowStorage& v) { u.dense = a.p; v.dense = a.q; }
@@ -38,28 +48,46 @@ template <int K, bool COH> struct DenseBase {
     __device__ __forceinline__ float step_of(float lrate, uint32_t thin, uint32_t bit) const { return (thin & bit) ? lrate_rep : lrate; }
     __device__ __forceinline__ float scale_of(uint32_t thin, uint32_t bit) const { return (thin & bit) ? rep_scale : 1.0f; }
 
-    __device__ __forceinline__ Prep prepare(const Rating&, bool) const { return Prep(); }
-    __device__ __forceinline__ int classify(const Rating&, const Prep&, bool) const { return 0; }
-    static __device__ __forceinline__ Info no_row() { return Info{0.f, 0xffffffffu, 0xffffffffu, 0u}; }   // matches no rating
-    // u, v: the rows to address (Rating::ru, rv); equal values are the same row, which is all forward() needs
-    __device__ __forceinline__ Info info(const Rating& my, const Prep&, int j) const
-    {
-        Info i;
-        i.r = bcast(my.r, j);
-        i.u = bcast(my.ru, j);
-        i.v = bcast(my.rv, j);
-        i.thin = bcast(my.thin, j);
-        return i;
-    }
-    // first element of a row of the matrix or, for a replicated row, of this XCD's copy (wave-uniform: scalar selects)
+    // Bits of Info::thin above Rating::thin's six: the size of a row in bytes, a single bit, shifted left by 0..3 says
+    // that the user / item row's window for device-coherent stores and the user / item row's window for cached stores
+    // (the copy of a replicated row) is open, so that a window's size is one shift and one mask.
+    static constexpr uint32_t kRowBytes = K * 4u;
+    static_assert((kRowBytes & (kRowBytes - 1u)) == 0u && kRowBytes > 63u, "the window bits lie above Rating::thin's");
+    // first element of a row of the matrix or, for a replicated row, of this XCD's copy
     template <class T> static __device__ __forceinline__ T* row_of(T* matrix, T* replicas, uint32_t row)
     {
         return ((row & kReplicaRow) ? replicas : matrix) + (size_t)(row & ~kReplicaRow) * K;
     }
+    // side 0: the user row, 1: the item row.  A row's new value is stored unless the update is thinned or added
+    // instead; a replicated row's copy is stored with an ordinary cached store (it stays in this XCD's L2) through a
+    // second window with that cache policy.
+    static __device__ __forceinline__ bool stores_row(uint32_t thin, int side) { return !((thin & (5u << side)) || (COH && (thin & (16u << side)))); }
+    static __device__ __forceinline__ bool stores_copy(uint32_t thin, int side) { return COH && (thin & (20u << side)) == (16u << side); }
+    __device__ __forceinline__ Prep prepare(const Rating& my, bool) const
+    {
+        Prep pr;
+        pr.pu = reinterpret_cast<uint64_t>(row_of(P, RP, my.ru));
+        pr.pv = reinterpret_cast<uint64_t>(row_of(Q, RQ, my.rv));
+        pr.thin = my.thin | (stores_row(my.thin, 0) ? kRowBytes : 0u) | (stores_row(my.thin, 1) ? kRowBytes << 1 : 0u)
+                  | (stores_copy(my.thin, 0) ? kRowBytes << 2 : 0u) | (stores_copy(my.thin, 1) ? kRowBytes << 3 : 0u);
+        return pr;
+    }
+    __device__ __forceinline__ int classify(const Rating&, const Prep&, bool) const { return 0; }
+    static __device__ __forceinline__ Info no_row() { return Info{0.f, 0u, 1ull, 1ull}; }   // matches no rating: no row lies at an odd address
+    // equal addresses are the same row, which is all forward() needs
+    __device__ __forceinline__ Info info(const Rating& my, const Prep& pr, int j) const
+    {
+        Info i;
+        i.r = bcast(my.r, j);
+        i.thin = bcast(pr.thin, j);
+        i.u = bcast(pr.pu, j);
+        i.v = bcast(pr.pv, j);
+        return i;
+    }
     template <int CLS> __device__ __forceinline__ void load(Row& row, const Info& i) const
     {
-        const float* pp = row_of(P, RP, i.u) + lane;
-        const float* qq = row_of(Q, RQ, i.v) + lane;
+        const float* pp = reinterpret_cast<const float*>(i.u) + lane;
+        const float* qq = reinterpret_cast<const float*>(i.v) + lane;
 #pragma unroll
         for (int e = 0; e < E; ++e) { row.p[e] = row_load(pp + 64 * e); row.q[e] = row_load(qq + 64 * e); }
     }
@@ -70,27 +98,23 @@ template <int K, bool COH> struct DenseBase {
     // lose more to the dropped stores than the longer look-ahead gives them, and keep their branches.)
     template <bool HOT> __device__ __forceinline__ void store(const Row& row, const Info& i, const float* dp, const float* dq) const
     {
-        float* prow = row_of(P, RP, i.u);
-        float* qrow = row_of(Q, RQ, i.v);
-        float* pp = prow + lane;
-        float* qq = qrow + lane;
+        float* pp = reinterpret_cast<float*>(i.u) + lane;
+        float* qq = reinterpret_cast<float*>(i.v) + lane;
         if constexpr (!HOT) {
 #pragma unroll
             for (int e = 0; e < E; ++e) { row_store<COH>(pp + 64 * e, row.p[e]); row_store<COH>(qq + 64 * e, row.q[e]); }
         } else {
             const bool add_p = (i.thin & 5u) == 4u, add_q = (i.thin & 10u) == 8u;
-            // a replicated row is stored with an ordinary cached store (it stays in this XCD's L2): a second window per
-            // side with that cache policy, open for replicated rows only
-            const row_window_t wp = row_window(reinterpret_cast<uint64_t>(prow), ((i.thin & 5u) || (COH && (i.thin & 16u))) ? 0u : K * 4u);
-            const row_window_t wq = row_window(reinterpret_cast<uint64_t>(qrow), ((i.thin & 10u) || (COH && (i.thin & 32u))) ? 0u : K * 4u);
+            const row_window_t wp = row_window(i.u, i.thin & kRowBytes);
+            const row_window_t wq = row_window(i.v, (i.thin >> 1) & kRowBytes);
 #pragma unroll
             for (int e = 0; e < E; ++e) {
                 window_store<COH>(wp, (uint32_t)(lane + 64 * e) * 4u, bits(row.p[e]));
                 window_store<COH>(wq, (uint32_t)(lane + 64 * e) * 4u, bits(row.q[e]));
             }
             if constexpr (COH) {
-                const row_window_t rp = row_window(reinterpret_cast<uint64_t>(prow), (i.thin & 20u) == 16u ? K * 4u : 0u);
-                const row_window_t rq = row_window(reinterpret_cast<uint64_t>(qrow), (i.thin & 40u) == 32u ? K * 4u : 0u);
+                const row_window_t rp = row_window(i.u, (i.thin >> 2) & kRowBytes);
+                const row_window_t rq = row_window(i.v, (i.thin >> 3) & kRowBytes);
 #pragma unroll
                 for (int e = 0; e < E; ++e) {
                     window_store<false>(rp, (uint32_t)(lane + 64 * e) * 4u, bits(row.p[e]));

@@ -234,7 +234,7 @@ struct HotRows {
         if (!wanted(prm)) return 0;
         step_scale = prm.replica_step_scale < 0 ? mf_replica_step_scale(prm.learning_rate, mean_rating) : prm.replica_step_scale;
         // MuPPET takes no longer steps by default.  Measured at 100M ratings, learning rate 0.01, first epoch with half the
-        // updates in flight: the other rules run at factors 4.3 (their default) and 6 and diverge at 8; MuPPET with its
+        // updates in flight: the other rules run at factors 4.3 (their default) and 6 and diverge at 7 or 8; MuPPET with its
         // 8-bit passes left rows of the order of 1e7 in 6 of 6 runs at 4.3 and in 4 of 12 at 2, at random, and none in 16
         // unscaled runs (test RMSE after the epoch 1.091-1.101 at k = 128; scaled and with all updates in flight:
         // 1.098-1.105 in 10 of 10 runs, 10 ms sooner).
