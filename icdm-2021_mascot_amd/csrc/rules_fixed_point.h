@@ -423,8 +423,8 @@ template <int K, bool COH> struct MuppetRule : DenseBase<K, COH> {
         for (int e = 0; e < E; ++e) {
             dp[e] = ds_p * gbp[e];
             dq[e] = ds_q * gbq[e];
-            row.p[e] = (i.thin & 1u) ? row.p[e] : row.p[e] + dp[e];
-            row.q[e] = (i.thin & 2u) ? row.q[e] : row.q[e] + dq[e];
+            row.p[e] = Base::template skips<CLS>(i.thin, 1u) ? row.p[e] : row.p[e] + dp[e];
+            row.q[e] = Base::template skips<CLS>(i.thin, 2u) ? row.q[e] : row.q[e] + dq[e];
         }
         this->template store<HOT>(row, i, dp, dq);
         if (fwd != 32 && bwd != 32 && processed >= first_sample) {
@@ -649,8 +649,8 @@ template <int K, bool COH> struct AfpRule : DenseBase<K, COH> {
         for (int e = 0; e < E; ++e) {
             dp[e] = ds_p * gbp[e];
             dq[e] = ds_q * gbq[e];
-            row.p[e] = (i.thin & 1u) ? row.p[e] : row.p[e] + dp[e];
-            row.q[e] = (i.thin & 2u) ? row.q[e] : row.q[e] + dq[e];
+            row.p[e] = Base::template skips<CLS>(i.thin, 1u) ? row.p[e] : row.p[e] + dp[e];
+            row.q[e] = Base::template skips<CLS>(i.thin, 2u) ? row.q[e] : row.q[e] + dq[e];
         }
         this->template store<HOT>(row, i, dp, dq);
         cur_iter += 1;

@@ -15,8 +15,6 @@ template <int K> struct DenseRow {
     static constexpr int E = K / 64;
     float p[E], q[E];
 };
-struct DenseInfo { float r; uint32_t u, v, thin; };
-struct NoPrep {};
 // What the dense fp32 rules broadcast per rating: the two rows as addresses (the matrix row, or this XCD's copy of a
 // replicated row) and Rating::thin with four more bits, one per store window of the hot-row code (DenseBase::store).
 // Addresses and window bits are computed once per chunk across the 64 lanes (DenseBase::prepare); per rating that costs
@@ -33,7 +31,9 @@ template <int K, bool COH> struct DenseBase {
     using Row = DenseRow<K>;
     using Info = DenseAddrInfo;      // u, v: the addresses of the two rows
     using Prep = DenseAddrPrep;
-    static constexpr int kClasses = 1;
+    // Chunk classes: 1 = no rating of the chunk has an update that is skipped (thinning is opt-in, so every chunk of a
+    // default run): its loop carries no selects for it; 0 = the general loop.
+    static constexpr int kClasses = 2;
     static constexpr int kK = K;
     template <class Params> static void row_storage(const Params& a, RowStorage& u, RowStorage& v) { u.dense = a.p; v.dense = a.q; }
     float* P;
@@ -72,7 +72,12 @@ template <int K, bool COH> struct DenseBase {
                   | (stores_copy(my.thin, 0) ? kRowBytes << 2 : 0u) | (stores_copy(my.thin, 1) ? kRowBytes << 3 : 0u);
         return pr;
     }
-    __device__ __forceinline__ int classify(const Rating&, const Prep&, bool) const { return 0; }
+    __device__ __forceinline__ int classify(const Rating& my, const Prep&, bool valid) const
+    {
+        return __builtin_amdgcn_ballot_w64(valid && (my.thin & 3u)) == 0ull ? 1 : 0;
+    }
+    // bit = 1 (user row) or 2 (item row) of Info::thin: this side's update is skipped
+    template <int CLS> static __device__ __forceinline__ bool skips(uint32_t thin, uint32_t bit) { return CLS == 0 && (thin & bit); }
     static __device__ __forceinline__ Info no_row() { return Info{0.f, 0u, 1ull, 1ull}; }   // matches no rating: no row lies at an odd address
     // equal addresses are the same row, which is all forward() needs
     __device__ __forceinline__ Info info(const Rating& my, const Prep& pr, int j) const
@@ -187,8 +192,8 @@ template <int K, bool COH> struct SgdRule : DenseBase<K, COH> {
             const float pe = row.p[e], qe = row.q[e];
             dp[e] = lr_p * (ruv * qe - lambda * pe);
             dq[e] = lr_q * (ruv * pe - lambda * qe);
-            row.p[e] = (i.thin & 1u) ? pe : pe + dp[e];
-            row.q[e] = (i.thin & 2u) ? qe : qe + dq[e];
+            row.p[e] = Base::template skips<CLS>(i.thin, 1u) ? pe : pe + dp[e];
+            row.q[e] = Base::template skips<CLS>(i.thin, 2u) ? qe : qe + dq[e];
         }
         this->template store<HOT>(row, i, dp, dq);
     }
@@ -231,8 +236,8 @@ template <int K, bool COH> struct MptRule : DenseBase<K, COH> {
             const half_t gq = ruv * ph[e] - lambda_h * qh[e];
             dp[e] = lr_p * (scaling_factor_rev * (float)gp);
             dq[e] = lr_q * (scaling_factor_rev * (float)gq);
-            row.p[e] = (i.thin & 1u) ? row.p[e] : row.p[e] + dp[e];
-            row.q[e] = (i.thin & 2u) ? row.q[e] : row.q[e] + dq[e];
+            row.p[e] = Base::template skips<CLS>(i.thin, 1u) ? row.p[e] : row.p[e] + dp[e];
+            row.q[e] = Base::template skips<CLS>(i.thin, 2u) ? row.q[e] : row.q[e] + dq[e];
         }
         this->template store<HOT>(row, i, dp, dq);
     }
@@ -248,9 +253,9 @@ template <int K, bool COH> struct MptRule : DenseBase<K, COH> {
 template <int K, bool COH> struct MemQuantRule {
     static constexpr int E = K / 64;
     struct Row { uint32_t p, q; };      // the binary16 values as loaded (a pair at k = 128): half the registers of widened rows
-    using Info = DenseInfo;
-    using Prep = NoPrep;
-    static constexpr int kClasses = 1;
+    using Info = DenseAddrInfo;         // u, v: the addresses of the two rows, computed once per chunk (as for the fp32 rules)
+    struct Prep { uint64_t pu, pv; };
+    static constexpr int kClasses = 2;      // 1: no update of the chunk is skipped (as for the fp32 rules)
     static constexpr int kAhead = 3, kRing = 8;
     static constexpr bool kSplittable = true;
     struct Params { uint16_t* p; uint16_t* q; float lrate; float lambda; bool accumulate; void* rep_p; void* rep_q; float rep_scale; };
@@ -268,13 +273,19 @@ template <int K, bool COH> struct MemQuantRule {
     }
     static constexpr int kK = K;
     static void row_storage(const Params& a, RowStorage& u, RowStorage& v) { u.dense = a.p; u.elem_bytes = 2; v.dense = a.q; v.elem_bytes = 2; }
-    __device__ __forceinline__ Prep prepare(const Rating&, bool) const { return Prep(); }
-    __device__ __forceinline__ int classify(const Rating&, const Prep&, bool) const { return 0; }
-    static __device__ __forceinline__ Info no_row() { return Info{0.f, 0xffffffffu, 0xffffffffu, 0u}; }
-    __device__ __forceinline__ Info info(const Rating& my, const Prep&, int j) const
+    __device__ __forceinline__ Prep prepare(const Rating& my, bool) const
+    {
+        return Prep{reinterpret_cast<uint64_t>(row_of(P, RP, my.ru)), reinterpret_cast<uint64_t>(row_of(Q, RQ, my.rv))};
+    }
+    __device__ __forceinline__ int classify(const Rating& my, const Prep&, bool valid) const
+    {
+        return __builtin_amdgcn_ballot_w64(valid && (my.thin & 3u)) == 0ull ? 1 : 0;
+    }
+    static __device__ __forceinline__ Info no_row() { return Info{0.f, 0u, 1ull, 1ull}; }      // no row lies at an odd address
+    __device__ __forceinline__ Info info(const Rating& my, const Prep& pr, int j) const
     {
         Info i;
-        i.r = bcast(my.r, j); i.u = bcast(my.ru, j); i.v = bcast(my.rv, j); i.thin = bcast(my.thin, j);
+        i.r = bcast(my.r, j); i.thin = bcast(my.thin, j); i.u = bcast(pr.pu, j); i.v = bcast(pr.pv, j);
         return i;
     }
     __device__ __forceinline__ uint32_t load_side(const uint16_t* row) const
@@ -284,8 +295,8 @@ template <int K, bool COH> struct MemQuantRule {
     }
     template <int CLS> __device__ __forceinline__ void load(Row& row, const Info& i) const
     {
-        row.p = load_side(row_of(P, RP, i.u));
-        row.q = load_side(row_of(Q, RQ, i.v));
+        row.p = load_side(reinterpret_cast<const uint16_t*>(i.u));
+        row.q = load_side(reinterpret_cast<const uint16_t*>(i.v));
     }
     __device__ __forceinline__ void forward(Row& nxt, const Info& in, const Row& cur, const Info& ic) const
     {
@@ -362,8 +373,8 @@ template <int K, bool COH> struct MemQuantRule {
             nq[e] = qf[e] + dq[e];
         }
         // the register copy is what the row holds afterwards: the sum rounded to binary16
-        if (!(i.thin & 1u)) { row.p = narrow(np); write_side(row_of(P, RP, i.u), row.p, dp, i.thin & 4u, i.thin & 16u); }
-        if (!(i.thin & 2u)) { row.q = narrow(nq); write_side(row_of(Q, RQ, i.v), row.q, dq, i.thin & 8u, i.thin & 32u); }
+        if (!(CLS == 0 && (i.thin & 1u))) { row.p = narrow(np); write_side(reinterpret_cast<uint16_t*>(i.u), row.p, dp, i.thin & 4u, i.thin & 16u); }
+        if (!(CLS == 0 && (i.thin & 2u))) { row.q = narrow(nq); write_side(reinterpret_cast<uint16_t*>(i.v), row.q, dq, i.thin & 8u, i.thin & 32u); }
     }
     __device__ __forceinline__ void finish(const Params&, uint32_t) const {}
 };
