@@ -556,6 +556,63 @@ def test_hot_row_thinning_drops_whole_row_updates(orc, k, variant):
 
 
 @pytest.mark.parametrize("k", [64, 128])
+@pytest.mark.parametrize("variant", ["single", "mpt", "muppet", "afp", "mem_quant"])
+def test_chunks_with_skipped_updates_take_the_general_loop_to_the_same_rows(k, variant):
+    """The dense rules run a chunk of 64 ratings in which no update is skipped in a loop without the selects for skipped
+    updates, and any other chunk in the general loop.  One worker, every row touched exactly once, so no update depends
+    on another: with a quarter of the user updates carried out (keep 63) every item row and every updated user row must
+    come out as in the run without thinning (bit for bit for binary32 rows), and a skipped user row as it went in."""
+    import torch
+    h = mfutil.hip()
+    n = 4096
+    rng = np.random.default_rng(321 + k)
+    R = np.zeros(n, mfutil.NODE)
+    R["u"], R["i"], R["r"] = np.arange(n), rng.permutation(n), rng.integers(1, 6, n)
+    P0 = (rng.standard_normal((n, k)) * 0.1).astype(np.float32)
+    Q0 = (rng.standard_normal((n, k)) * 0.1).astype(np.float32)
+    dt = np.float32
+    if variant == "mem_quant":
+        P0, Q0, dt = P0.astype(np.float16), Q0.astype(np.float16), np.float16
+    starts = np.arange(0, n, 128, dtype=np.uint32).reshape(-1, 1)
+    uc = starts.shape[0]
+
+    def run(keep_u):
+        dR, dS, dP, dQ = to_dev(R), to_dev(starts), to_dev(P0), to_dev(Q0)
+        opt = mfutil.HogwildOptions(k, np.full(n, keep_u, np.uint8), np.full(n, 255, np.uint8))
+        head = (dR.data_ptr(), n, dP.data_ptr(), dQ.data_ptr(), k, 1, uc, 128)
+        tail = (5, 0, dS.data_ptr(), mfutil.stream_ptr(), opt.ptr)
+        if variant == "single":
+            h.mf_single_sgd_hogwild_opt(*head, LR, LAM, *tail)
+        elif variant == "mpt":
+            h.mf_mpt_sgd_hogwild_opt(*head, LR, 0x5240, 1000.0, *tail)          # binary16 50 = lambda x 1000
+        elif variant == "muppet":
+            sm, sn = torch.zeros(k, dtype=torch.float32, device="cuda"), torch.zeros(1, dtype=torch.float32, device="cuda")
+            h.mf_muppet_sgd_hogwild_opt(*head, LR, LAM, uc * 128, sm.data_ptr(), sn.data_ptr(), 8, 8, *tail)
+        elif variant == "afp":
+            h.mf_afp_sgd_hogwild_opt(*head, LR, LAM, 1, *tail)
+        else:
+            h.mf_mem_quant_sgd_hogwild_opt(*head, LR, LAM, *tail)
+        torch.cuda.synchronize()
+        return from_dev(dP, dt, P0.shape), from_dev(dQ, dt, Q0.shape)
+
+    P1, Q1 = run(255)
+    assert np.all(np.any(P1 != P0, axis=1)) and np.all(np.any(Q1 != Q0, axis=1))
+    P2, Q2 = run(63)
+    assert np.array_equal(Q2.view(np.uint8), Q1.view(np.uint8))
+    changed = np.any(P2 != P0, axis=1)
+    assert 0.20 < changed.mean() < 0.30
+    if variant == "mem_quant":
+        # an update of a thinned row that is carried out is added to the row in memory, rounded to binary16 first, where
+        # the run without thinning stores the rounded sum: within one binary16 ulp of the larger of change and result
+        got, want, old = P2[changed].astype(np.float64), P1[changed].astype(np.float64), P0[changed].astype(np.float64)
+        scale = np.maximum(np.abs(want), np.abs(want - old)).astype(np.float16)
+        assert np.all(np.abs(got - want) <= np.spacing(scale).astype(np.float64))
+    else:
+        assert np.array_equal(P2[changed].view(np.uint8), P1[changed].view(np.uint8))      # binary32: old + change is the stored value
+    assert np.array_equal(P2[~changed].view(np.uint8), P0[~changed].view(np.uint8))
+
+
+@pytest.mark.parametrize("k", [64, 128])
 @pytest.mark.parametrize("variant", ["single", "mpt", "mascot", "muppet", "afp"])
 def test_hot_row_updates_add_up(orc, k, variant):
     """k wavefronts in k/4 workgroups update one hot item row at the same time.  User u's row is 0.5 * e_u, the item
